@@ -1,0 +1,60 @@
+"""Builds libapt_hip.so (the C-ABI HIP library) for gfx950 with hipcc.
+
+The library has no dependency on torch or Python: it is plain HIP.  hipcc
+cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is
+installed.  The result is written next to this file and loaded by capi.py.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libapt_hip.so")
+SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Wall", "-Wno-unused-function",
+    # packed-FP32 code generation is kept off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _obj(src):
+    return os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
+
+
+def build(force=True, verbose=False):
+    """Compile every source and link libapt_hip.so.  Returns its path."""
+    procs = []
+    headers = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "apt_amd.h")]
+    newest_hdr = max(os.path.getmtime(h) for h in headers)
+    objs = []
+    for s in SOURCES:
+        src = os.path.join(CSRC, s)
+        obj = _obj(s)
+        objs.append(obj)
+        stale = (force or not os.path.exists(obj)
+                 or os.path.getmtime(obj) < max(os.path.getmtime(src), newest_hdr))
+        if stale:
+            cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+            if verbose:
+                print(" ".join(cmd), file=sys.stderr)
+            procs.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    for s, p in procs:
+        out, _ = p.communicate()
+        text = out.decode(errors="replace")
+        # hipcc's host pass does not know the packed-fp32 feature name; harmless
+        text = "\n".join(l for l in text.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {s}:\n{text}")
+        if verbose and text.strip():
+            print(text, file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--incremental" not in sys.argv, verbose=True))

@@ -1,0 +1,309 @@
+"""ctypes binding of libapt_hip.so (declared in include/apt_amd.h).
+
+This is the only place Python touches the C ABI.  Arguments are torch tensors
+used purely as device buffers: the functions pass data pointers, sizes and the
+current HIP stream.  There is no CPU fallback: if the library is missing or a
+tensor is not on the GPU the call raises.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libapt_hip.so")
+
+_lib = None
+
+
+class AptError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+class CGraph(C.Structure):
+    _fields_ = [("indptr", C.c_void_p), ("indices", C.c_void_p),
+                ("row_begin", C.c_int64), ("num_rows", C.c_int64),
+                ("cached_indptr", C.c_void_p), ("cached_indices", C.c_void_p),
+                ("num_cached_rows", C.c_int64), ("adj_pos_map", C.c_void_p),
+                ("num_total_nodes", C.c_int64)]
+
+
+class CFeatStore(C.Structure):
+    _fields_ = [("local_table", C.c_void_p), ("num_local_rows", C.c_int64),
+                ("local_dim", C.c_int64), ("cache_table", C.c_void_p),
+                ("num_cache_rows", C.c_int64), ("pos_map", C.c_void_p),
+                ("num_total_nodes", C.c_int64), ("col_offset", C.c_int64),
+                ("out_dim", C.c_int64), ("elem_size", C.c_int)]
+
+
+# every symbol include/apt_amd.h declares: name -> (restype, argtypes)
+_P, _I64, _I, _U64, _SZ = C.c_void_p, C.c_int64, C.c_int, C.c_uint64, C.c_size_t
+SYMBOLS = {
+    "apt_last_error": (C.c_char_p, []),
+    "apt_abi_version": (_I, []),
+    "apt_set_tuning": (_I, [C.c_char_p, _I]),
+    "apt_sample_neighbors": (_I, [C.POINTER(CGraph), _P, _I64, _P, _I, _I, _U64, _I, _P, _P, _P, _P]),
+    "apt_relabel_workspace_bytes": (_SZ, [_I64]),
+    "apt_relabel": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_gather_rows": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P]),
+    "apt_permute_rows": (_I, [_P, _I64, _P, _I64, _I64, _I, _P, _P]),
+    "apt_scatter_rows": (_I, [_P, _P, _I64, _I64, _I, _P, _I64, _P]),
+    "apt_bucket_workspace_bytes": (_SZ, [_I64, _I]),
+    "apt_cluster_permute": (_I, [_P, _I64, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_cluster_reqs": (_I, [_P, _I64, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+}
+
+
+def lib():
+    """Load libapt_hip.so (built by apt_amd/build.py).  Raises if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m apt_amd.build` "
+                "(hipcc, gfx950).  There is no CPU fallback.")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise AptError(f"[{status}] {lib().apt_last_error().decode()}")
+
+
+def set_tuning(key, value):
+    check(lib().apt_set_tuning(key.encode(), int(value)))
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev_i64(t, name):
+    if t is None:
+        return None
+    if not (t.is_cuda and t.dtype == torch.int64 and t.is_contiguous()):
+        raise TypeError(f"{name} must be a contiguous int64 tensor on the GPU "
+                        f"(got {t.dtype}, {t.device}, contiguous={t.is_contiguous()})")
+    return t
+
+
+class Graph:
+    """Device-resident CSR graph in the layout of apt_graph."""
+
+    def __init__(self, indptr, indices, row_begin=0, cached_indptr=None, cached_indices=None,
+                 adj_pos_map=None, num_total_nodes=None):
+        self.indptr = _dev_i64(indptr, "indptr")
+        self.indices = _dev_i64(indices, "indices")
+        self.cached_indptr = _dev_i64(cached_indptr, "cached_indptr")
+        self.cached_indices = _dev_i64(cached_indices, "cached_indices")
+        self.adj_pos_map = _dev_i64(adj_pos_map, "adj_pos_map")
+        self.row_begin = int(row_begin)
+        self.num_rows = indptr.numel() - 1
+        self.num_cached_rows = 0 if cached_indptr is None else cached_indptr.numel() - 1
+        if num_total_nodes is None:
+            num_total_nodes = (adj_pos_map.numel() if adj_pos_map is not None
+                               else self.row_begin + self.num_rows)
+        self.num_total_nodes = int(num_total_nodes)
+        self.c = CGraph(_ptr(self.indptr), _ptr(self.indices), self.row_begin, self.num_rows,
+                        _ptr(self.cached_indptr), _ptr(self.cached_indices),
+                        self.num_cached_rows, _ptr(self.adj_pos_map), self.num_total_nodes)
+
+    @property
+    def device(self):
+        return self.indptr.device
+
+
+class FeatStore:
+    """Device-resident feature tables in the layout of apt_feat_store."""
+
+    def __init__(self, local_table, cache_table=None, pos_map=None, col_offset=0, out_dim=None,
+                 num_total_nodes=None):
+        if not (local_table.is_cuda and local_table.is_contiguous() and local_table.dim() == 2):
+            raise TypeError("local_table must be a contiguous 2-D tensor on the GPU")
+        if local_table.element_size() not in (2, 4):
+            raise TypeError(f"unsupported feature dtype {local_table.dtype}")
+        if cache_table is not None and cache_table.numel() == 0:
+            cache_table = None
+        if cache_table is not None:
+            if not (cache_table.is_cuda and cache_table.is_contiguous()
+                    and cache_table.dtype == local_table.dtype and cache_table.dim() == 2):
+                raise TypeError("cache_table must be a contiguous 2-D GPU tensor of the local dtype")
+            if pos_map is None:
+                raise ValueError("a cache table needs a position map")
+        self.local_table = local_table
+        self.cache_table = cache_table
+        self.pos_map = _dev_i64(pos_map, "pos_map")
+        self.col_offset = int(col_offset)
+        self.local_dim = local_table.shape[1]
+        if out_dim is None:
+            out_dim = cache_table.shape[1] if cache_table is not None else self.local_dim - self.col_offset
+        self.out_dim = int(out_dim)
+        if cache_table is not None and cache_table.shape[1] != self.out_dim:
+            raise ValueError("cache_table width must equal out_dim")
+        if num_total_nodes is None:
+            num_total_nodes = pos_map.numel() if pos_map is not None else local_table.shape[0]
+        self.num_total_nodes = int(num_total_nodes)
+        self.dtype = local_table.dtype
+        self.c = CFeatStore(_ptr(local_table), local_table.shape[0], self.local_dim,
+                            _ptr(cache_table), 0 if cache_table is None else cache_table.shape[0],
+                            _ptr(self.pos_map), self.num_total_nodes, self.col_offset,
+                            self.out_dim, local_table.element_size())
+
+    @property
+    def device(self):
+        return self.local_table.device
+
+
+def sample_neighbors(graph, frontier, fanout, replace, rng_seed, hop, num_frontier_dev=None,
+                     out_neighbors=None, out_counts=None, out_total=None, want_counts=True):
+    """-> (neighbors int64[n*fanout] padded with -1, counts int64[n] or None)."""
+    frontier = _dev_i64(frontier, "frontier")
+    n = frontier.numel()
+    if fanout <= 0:
+        raise AptError(f"fanout {fanout} must be > 0")
+    if out_neighbors is None:
+        out_neighbors = torch.empty(n * fanout, dtype=torch.int64, device=frontier.device)
+    if out_counts is None and want_counts:
+        out_counts = torch.empty(n, dtype=torch.int64, device=frontier.device)
+    check(lib().apt_sample_neighbors(C.byref(graph.c), _ptr(frontier), n, _ptr(num_frontier_dev),
+                                     int(fanout), int(bool(replace)),
+                                     int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(hop),
+                                     _ptr(out_neighbors), _ptr(out_counts), _ptr(out_total),
+                                     _stream()))
+    return out_neighbors, out_counts
+
+
+def relabel_workspace_bytes(num_items):
+    return int(lib().apt_relabel_workspace_bytes(int(num_items)))
+
+
+def relabel(seeds, neighbors, num_seeds_dev=None, neighbor_stride=0, unique=None, relabeled=None,
+            num_unique_dev=None, workspace=None, sync=True):
+    """-> (unique, relabeled, num_unique).  With sync=True `unique` is narrowed
+    to the count and num_unique is an int; otherwise both buffers keep their
+    capacity and num_unique is the device int64[1] tensor."""
+    seeds = _dev_i64(seeds, "seeds")
+    neighbors = _dev_i64(neighbors, "neighbors")
+    dev = seeds.device
+    ns, nn = seeds.numel(), neighbors.numel()
+    if unique is None:
+        unique = torch.empty(ns + nn, dtype=torch.int64, device=dev)
+    if relabeled is None:
+        relabeled = torch.empty(nn, dtype=torch.int64, device=dev)
+    if num_unique_dev is None:
+        num_unique_dev = torch.empty(1, dtype=torch.int64, device=dev)
+    need = relabel_workspace_bytes(ns + nn)
+    if need == 0:
+        raise AptError(f"relabel: {ns + nn} items exceed the supported maximum")
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    host = C.c_int64(-1)
+    check(lib().apt_relabel(_ptr(seeds), ns, _ptr(num_seeds_dev), _ptr(neighbors), nn,
+                            int(neighbor_stride), _ptr(unique), _ptr(relabeled),
+                            _ptr(num_unique_dev), C.cast(C.pointer(host), C.c_void_p) if sync else None,
+                            _ptr(workspace), workspace.numel(), _stream()))
+    if sync:
+        return unique[:host.value], relabeled, int(host.value)
+    return unique, relabeled, num_unique_dev
+
+
+def gather_rows(store, index, num_index_dev=None, out=None, miss_count=None):
+    """out[r, :] = feature row of node index[r] -> out [n, out_dim]."""
+    index = _dev_i64(index, "index")
+    n = index.numel()
+    if out is None:
+        out = torch.empty((n, store.out_dim), dtype=store.dtype, device=index.device)
+    check(lib().apt_gather_rows(C.byref(store.c), _ptr(index), n, _ptr(num_index_dev), _ptr(out),
+                                _ptr(miss_count), _stream()))
+    return out
+
+
+def _rows2d(t, name):
+    if not (t.is_cuda and t.is_contiguous() and t.dim() == 2 and t.element_size() in (2, 4)):
+        raise TypeError(f"{name} must be a contiguous 2-D GPU tensor with 2- or 4-byte elements")
+    return t
+
+
+def permute_rows(table, perm, out=None):
+    """out[i, :] = table[perm[i], :]"""
+    table = _rows2d(table, "table")
+    perm = _dev_i64(perm, "perm")
+    n = perm.numel()
+    if out is None:
+        out = torch.empty((n, table.shape[1]), dtype=table.dtype, device=table.device)
+    check(lib().apt_permute_rows(_ptr(table), table.shape[0], _ptr(perm), n, table.shape[1],
+                                 table.element_size(), _ptr(out), _stream()))
+    return out
+
+
+def scatter_rows(table, perm, num_out_rows=None, out=None):
+    """out[perm[i], :] = table[i, :]; rows nobody names are zero."""
+    table = _rows2d(table, "table")
+    perm = _dev_i64(perm, "perm")
+    n = perm.numel()
+    if n != table.shape[0]:
+        raise AptError(f"scatter_rows: {table.shape[0]} rows but {n} destinations")
+    if num_out_rows is None:
+        num_out_rows = n
+    if out is None:
+        out = torch.zeros((num_out_rows, table.shape[1]), dtype=table.dtype, device=table.device)
+    check(lib().apt_scatter_rows(_ptr(table), _ptr(perm), n, table.shape[1], table.element_size(),
+                                 _ptr(out), int(num_out_rows), _stream()))
+    return out
+
+
+def cluster_permute(ids, min_vids, num_buckets, id_offset=0, rank=0, node_beg=0, node_end=None):
+    """-> (bucket_size, bucket_offset, sorted_ids, permutation), all on the GPU."""
+    ids = _dev_i64(ids, "ids")
+    min_vids = _dev_i64(min_vids, "min_vids")
+    if min_vids.numel() < num_buckets + 1:
+        raise AptError(f"min_vids has {min_vids.numel()} entries, {num_buckets + 1} needed")
+    if node_end is None:
+        node_end = num_buckets
+    dev, n = ids.device, ids.numel()
+    bs = torch.empty(num_buckets, dtype=torch.int64, device=dev)
+    bo = torch.empty(num_buckets, dtype=torch.int64, device=dev)
+    so = torch.empty(n, dtype=torch.int64, device=dev)
+    pm = torch.empty(n, dtype=torch.int64, device=dev)
+    need = int(lib().apt_bucket_workspace_bytes(n, int(num_buckets)))
+    if need == 0:
+        raise AptError(f"cluster_permute: unsupported size (n={n}, buckets={num_buckets})")
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    check(lib().apt_cluster_permute(_ptr(ids), n, _ptr(min_vids), int(num_buckets), int(id_offset),
+                                    int(rank), int(node_beg), int(node_end), _ptr(bs), _ptr(bo),
+                                    _ptr(so), _ptr(pm), _ptr(ws), ws.numel(), _stream()))
+    return bs, bo, so, pm
+
+
+def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num_remote_workers):
+    """-> (bucket_size, bucket_offset, sorted_ids, permutation), all on the GPU."""
+    ids = _dev_i64(ids, "ids")
+    feat_pos_map = _dev_i64(feat_pos_map, "feat_pos_map")
+    remote_worker_map = _dev_i64(remote_worker_map, "remote_worker_map")
+    min_vids = _dev_i64(min_vids, "min_vids")
+    if min_vids.numel() < world_size + 1 or remote_worker_map.numel() < world_size:
+        raise AptError("cluster_reqs: min_vids / remote_worker_map shorter than world_size")
+    dev, n = ids.device, ids.numel()
+    bs = torch.empty(num_remote_workers, dtype=torch.int64, device=dev)
+    bo = torch.empty(num_remote_workers, dtype=torch.int64, device=dev)
+    so = torch.empty(n, dtype=torch.int64, device=dev)
+    pm = torch.empty(n, dtype=torch.int64, device=dev)
+    need = int(lib().apt_bucket_workspace_bytes(n, int(num_remote_workers)))
+    if need == 0:
+        raise AptError(f"cluster_reqs: unsupported size (n={n}, buckets={num_remote_workers})")
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    check(lib().apt_cluster_reqs(_ptr(ids), n, _ptr(feat_pos_map), feat_pos_map.numel(),
+                                 _ptr(remote_worker_map), _ptr(min_vids), int(world_size),
+                                 int(num_remote_workers), _ptr(bs), _ptr(bo), _ptr(so), _ptr(pm),
+                                 _ptr(ws), ws.numel(), _stream()))
+    return bs, bo, so, pm

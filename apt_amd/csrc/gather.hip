@@ -1,0 +1,265 @@
+// Indexed row gather from HBM-resident feature tables, and the row
+// permute / scatter that FeatShuffle does on the GPU.
+//
+// Replaces _CSRRowWiseLoadSubtensorAlignedAllKernel / IndexSelectAll
+// (reference src/cuda/npc_kernel.cu:187-246) and the index_select /
+// index_select_backward halves of FeatShuffle (src/feat_shuffle.cc:14-16,27).
+// The reference moves one 4-byte element per thread and reads
+// feat_pos_map[index[row]] twice per thread; here a lane group owns a row,
+// reads the id and the position once, and moves the row as 16-byte vectors
+// (8/4/2-byte vectors when the row geometry is not 16-byte aligned), with
+// several rows per group in flight.  Pure copy: results are bit-exact.
+#include "common.hpp"
+
+namespace apt {
+
+constexpr int kGatherBlock = 256;
+
+struct GatherParams {
+  const char* local_table;
+  int64_t num_local_rows;
+  int64_t local_row_bytes;   // local_dim * elem_size
+  int64_t col_offset_bytes;
+  const char* cache_table;
+  int64_t num_cache_rows;
+  const int64_t* pos_map;
+  int64_t num_total_nodes;
+  int64_t out_row_bytes;
+  const int64_t* index;
+  int64_t n;
+  const int64_t* n_dev;
+  char* out;
+  int64_t* miss_count;
+  int scatter;               // 1: out[index[r]] = in[r] (pack); rows come from local_table
+  int64_t num_out_rows;      // scatter only
+};
+
+template <int V> struct VecT;
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <> struct VecT<16> { using type = u32x4_t; };
+template <> struct VecT<8> { using type = u32x2_t; };
+template <> struct VecT<4> { using type = uint32_t; };
+template <> struct VecT<2> { using type = uint16_t; };
+
+// Source address of the row for node v, or nullptr when it is not present
+// (reference :196-205 for the two-table addressing).
+__device__ __forceinline__ const char* source_row(const GatherParams& p, int64_t v) {
+  if (v < 0) return nullptr;
+  if (p.pos_map != nullptr) {
+    if (v >= p.num_total_nodes) return nullptr;
+    const int64_t pos = p.pos_map[v];
+    if (pos < -1) {
+      const int64_t row = -pos - 2;
+      if (row >= p.num_local_rows) return nullptr;
+      return p.local_table + row * p.local_row_bytes + p.col_offset_bytes;
+    }
+    if (pos < 0 || pos >= p.num_cache_rows) return nullptr;
+    return p.cache_table + pos * p.out_row_bytes;
+  }
+  if (v >= p.num_local_rows) return nullptr;
+  return p.local_table + v * p.local_row_bytes + p.col_offset_bytes;
+}
+
+// LPR lanes per row, R rows per group per step, V bytes per lane access.
+template <int V, int LPR, int R>
+__global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
+  using Vec = typename VecT<V>::type;
+  constexpr int kGroups = kGatherBlock / LPR;
+  const int64_t n = actual_count(p.n, p.n_dev);
+  const int grp = threadIdx.x / LPR;
+  const int l = threadIdx.x % LPR;
+  const int64_t vec_per_row = p.out_row_bytes / V;
+  const int64_t rows_per_block = static_cast<int64_t>(kGroups) * R;
+  int64_t misses = 0;
+  for (int64_t base = static_cast<int64_t>(blockIdx.x) * rows_per_block; base < n;
+       base += static_cast<int64_t>(gridDim.x) * rows_per_block) {
+    const char* src[R];
+    char* dst[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+      const int64_t r = base + static_cast<int64_t>(k) * kGroups + grp;
+      src[k] = nullptr;
+      dst[k] = nullptr;
+      if (r < n) {
+        const int64_t v = p.index[r];
+        if (p.scatter) {
+          // pack: row r of the input goes to row index[r] of the output
+          if (v >= 0 && v < p.num_out_rows) {
+            src[k] = p.local_table + r * p.out_row_bytes;
+            dst[k] = p.out + v * p.out_row_bytes;
+          }
+        } else {
+          src[k] = source_row(p, v);
+          dst[k] = p.out + r * p.out_row_bytes;
+          if (src[k] == nullptr && l == 0) ++misses;
+        }
+      }
+    }
+    for (int64_t c = l; c < vec_per_row; c += LPR) {
+      Vec val[R];
+#pragma unroll
+      for (int k = 0; k < R; ++k) {
+        val[k] = Vec{};
+        if (src[k] != nullptr)
+          val[k] = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(src[k]) + c);
+      }
+#pragma unroll
+      for (int k = 0; k < R; ++k) {
+        if (dst[k] != nullptr)
+          __builtin_nontemporal_store(val[k], reinterpret_cast<Vec*>(dst[k]) + c);
+      }
+    }
+  }
+  if (p.miss_count != nullptr && misses != 0)
+    atomicAdd(reinterpret_cast<unsigned long long*>(p.miss_count),
+              static_cast<unsigned long long>(misses));
+}
+
+int tuning_gather_rows();  // 0 = default
+
+template <int V, int LPR>
+static int launch_gather_r(const GatherParams& p, hipStream_t st) {
+  int R = tuning_gather_rows();
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = 4;
+  const int groups = kGatherBlock / LPR;
+  int64_t blocks = ceil_div(p.n, static_cast<int64_t>(groups) * R);
+  if (blocks > (1 << 20)) blocks = 1 << 20;
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kGatherBlock);
+  switch (R) {
+    case 1: hipLaunchKernelGGL((gather_kernel<V, LPR, 1>), grid, block, 0, st, p); break;
+    case 2: hipLaunchKernelGGL((gather_kernel<V, LPR, 2>), grid, block, 0, st, p); break;
+    case 8: hipLaunchKernelGGL((gather_kernel<V, LPR, 8>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((gather_kernel<V, LPR, 4>), grid, block, 0, st, p); break;
+  }
+  APT_LAUNCH_CHECK("gather_kernel");
+  return APT_OK;
+}
+
+template <int V>
+static int launch_gather_v(const GatherParams& p, hipStream_t st) {
+  const int64_t vec_per_row = p.out_row_bytes / V;
+  if (vec_per_row <= 8) return launch_gather_r<V, 8>(p, st);
+  if (vec_per_row <= 16) return launch_gather_r<V, 16>(p, st);
+  if (vec_per_row <= 32) return launch_gather_r<V, 32>(p, st);
+  return launch_gather_r<V, 64>(p, st);
+}
+
+// Widest vector that every row start and the row length are multiples of.
+static int vector_bytes(const GatherParams& p, int elem_size) {
+  uintptr_t bits = reinterpret_cast<uintptr_t>(p.local_table) |
+                   reinterpret_cast<uintptr_t>(p.out) |
+                   static_cast<uintptr_t>(p.local_row_bytes) |
+                   static_cast<uintptr_t>(p.col_offset_bytes) |
+                   static_cast<uintptr_t>(p.out_row_bytes);
+  if (p.cache_table != nullptr) bits |= reinterpret_cast<uintptr_t>(p.cache_table);
+  for (int v = 16; v > elem_size; v >>= 1)
+    if ((bits & (v - 1)) == 0) return v;
+  return elem_size;
+}
+
+static int launch_gather(const GatherParams& p, int elem_size, hipStream_t st) {
+  switch (vector_bytes(p, elem_size)) {
+    case 16: return launch_gather_v<16>(p, st);
+    case 8: return launch_gather_v<8>(p, st);
+    case 4: return launch_gather_v<4>(p, st);
+    default: return launch_gather_v<2>(p, st);
+  }
+}
+
+}  // namespace apt
+
+extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
+                               int64_t num_index, const int64_t* num_index_dev, void* out,
+                               int64_t* miss_count, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(store != nullptr, APT_EINVAL, "apt_gather_rows: store is NULL");
+  APT_REQUIRE(num_index >= 0, APT_EINVAL, "apt_gather_rows: num_index %lld < 0",
+              (long long)num_index);
+  APT_REQUIRE(store->elem_size == 2 || store->elem_size == 4, APT_EINVAL,
+              "apt_gather_rows: elem_size %d (2 or 4 supported)", store->elem_size);
+  APT_REQUIRE(store->out_dim > 0 && store->local_dim >= 0 && store->col_offset >= 0, APT_EINVAL,
+              "apt_gather_rows: bad dims (local_dim %lld, col_offset %lld, out_dim %lld)",
+              (long long)store->local_dim, (long long)store->col_offset,
+              (long long)store->out_dim);
+  APT_REQUIRE(store->num_local_rows == 0 ||
+                  (store->local_table != nullptr &&
+                   store->col_offset + store->out_dim <= store->local_dim),
+              APT_EINVAL,
+              "apt_gather_rows: column window [%lld, %lld) outside local_dim %lld",
+              (long long)store->col_offset, (long long)(store->col_offset + store->out_dim),
+              (long long)store->local_dim);
+  APT_REQUIRE(store->num_cache_rows == 0 ||
+                  (store->cache_table != nullptr && store->pos_map != nullptr),
+              APT_EINVAL, "apt_gather_rows: cache rows need cache_table and pos_map");
+  APT_REQUIRE(store->num_local_rows >= 0 && store->num_cache_rows >= 0, APT_EINVAL,
+              "apt_gather_rows: negative row count");
+  if (num_index == 0) return APT_OK;
+  APT_REQUIRE(index != nullptr && out != nullptr, APT_EINVAL,
+              "apt_gather_rows: index/out is NULL");
+  GatherParams p;
+  p.local_table = static_cast<const char*>(store->local_table);
+  p.num_local_rows = store->num_local_rows;
+  p.local_row_bytes = store->local_dim * store->elem_size;
+  p.col_offset_bytes = store->col_offset * store->elem_size;
+  p.cache_table = store->num_cache_rows > 0 ? static_cast<const char*>(store->cache_table) : nullptr;
+  p.num_cache_rows = store->num_cache_rows;
+  p.pos_map = store->pos_map;
+  p.num_total_nodes = store->num_total_nodes;
+  p.out_row_bytes = store->out_dim * store->elem_size;
+  p.index = index;
+  p.n = num_index;
+  p.n_dev = num_index_dev;
+  p.out = static_cast<char*>(out);
+  p.miss_count = miss_count;
+  p.scatter = 0;
+  p.num_out_rows = 0;
+  return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
+}
+
+static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_t dim,
+                          int elem_size, void* out, int scatter, int64_t num_rows_other,
+                          void* stream, const char* who) {
+  using namespace apt;
+  APT_REQUIRE(n >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (n %lld, dim %lld)", who,
+              (long long)n, (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "%s: elem_size %d (2 or 4 supported)",
+              who, elem_size);
+  if (n == 0) return APT_OK;
+  APT_REQUIRE(in != nullptr && perm != nullptr && out != nullptr, APT_EINVAL,
+              "%s: in/perm/out is NULL", who);
+  GatherParams p;
+  p.local_table = static_cast<const char*>(in);
+  p.num_local_rows = scatter ? n : num_rows_other;
+  p.local_row_bytes = dim * elem_size;
+  p.col_offset_bytes = 0;
+  p.cache_table = nullptr;
+  p.num_cache_rows = 0;
+  p.pos_map = nullptr;
+  p.num_total_nodes = 0;
+  p.out_row_bytes = dim * elem_size;
+  p.index = perm;
+  p.n = n;
+  p.n_dev = nullptr;
+  p.out = static_cast<char*>(out);
+  p.miss_count = nullptr;
+  p.scatter = scatter;
+  p.num_out_rows = scatter ? num_rows_other : 0;
+  return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int apt_permute_rows(const void* in, int64_t num_in_rows, const int64_t* perm,
+                                int64_t n, int64_t dim, int elem_size, void* out, void* stream) {
+  APT_REQUIRE(num_in_rows >= 0, APT_EINVAL, "apt_permute_rows: num_in_rows %lld < 0",
+              (long long)num_in_rows);
+  return permute_common(in, perm, n, dim, elem_size, out, 0, num_in_rows, stream,
+                        "apt_permute_rows");
+}
+
+extern "C" int apt_scatter_rows(const void* in, const int64_t* perm, int64_t n, int64_t dim,
+                                int elem_size, void* out, int64_t num_out_rows, void* stream) {
+  APT_REQUIRE(num_out_rows >= 0, APT_EINVAL, "apt_scatter_rows: num_out_rows %lld < 0",
+              (long long)num_out_rows);
+  return permute_common(in, perm, n, dim, elem_size, out, 1, num_out_rows, stream,
+                        "apt_scatter_rows");
+}

@@ -1,0 +1,41 @@
+// Library-wide state of libapt_hip.so: per-thread error text, ABI version and
+// the tuning knobs the benchmark uses to compare kernel variants.
+#include "common.hpp"
+
+#include <cstring>
+
+namespace apt {
+
+char* last_error_buf() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+static int g_sample_lanes = 0;
+static int g_gather_rows = 0;
+
+int tuning_sample_lanes() { return g_sample_lanes; }
+int tuning_gather_rows() { return g_gather_rows; }
+
+}  // namespace apt
+
+extern "C" const char* apt_last_error(void) { return apt::last_error_buf(); }
+
+extern "C" int apt_abi_version(void) { return 1; }
+
+extern "C" int apt_set_tuning(const char* key, int value) {
+  if (key == nullptr) return apt::fail(APT_EINVAL, "apt_set_tuning: key is NULL");
+  if (std::strcmp(key, "sample_lanes_per_row") == 0) {
+    if (value != 0 && value != 8 && value != 16 && value != 32 && value != 64)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: sample_lanes_per_row must be 0, 8, 16, 32 or 64");
+    apt::g_sample_lanes = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "gather_rows_in_flight") == 0) {
+    if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: gather_rows_in_flight must be 0, 1, 2, 4 or 8");
+    apt::g_gather_rows = value;
+    return APT_OK;
+  }
+  return apt::fail(APT_EINVAL, "apt_set_tuning: unknown key '%s'", key);
+}

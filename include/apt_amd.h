@@ -1,0 +1,225 @@
+/*
+ * apt_amd.h — C ABI of the MI355X (gfx950) mini-batch construction library.
+ *
+ * One shared library (libapt_hip.so) implements these entry points with
+ * hand-written HIP kernels.  Every pointer named "device" is device memory of
+ * the GPU that is current when the call is made; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  Nothing here allocates or
+ * frees device memory: outputs and scratch come from the caller.  Calls are
+ * asynchronous unless the comment says otherwise.
+ *
+ * Return value: 0 on success, a negative APT_E* code on failure; the message
+ * for the calling thread's last failure is apt_last_error().  A failing call
+ * launches nothing.
+ *
+ * Conventions shared with the reference (src/utils.h:14-21):
+ *   ids and offsets are int64; ENCODE_ID(i) = -(i)-2 marks "row i of the
+ *   second table" in a position map; -1 in a feature position map means
+ *   "not present".  In id arrays a negative id is padding: it has no
+ *   neighbours, is not relabelled and stays negative in outputs.
+ *
+ * Each entry point cites the reference interface it replaces.
+ */
+#ifndef APT_AMD_H_
+#define APT_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APT_OK 0
+#define APT_EINVAL (-1)  /* bad argument (null pointer, negative size, ...) */
+#define APT_ELIMIT (-2)  /* size beyond what the entry point supports */
+#define APT_EWORKSPACE (-3) /* workspace too small */
+#define APT_EHIP (-4)    /* a HIP runtime call failed */
+
+#define APT_MAX_BUCKETS 64 /* reference: MAX_NUM_DEVICES 33 (src/cuda/npc_kernel.h:13) */
+
+const char* apt_last_error(void);
+int apt_abi_version(void);
+
+/* Kernel-variant knobs for measurement (process-wide, not thread-safe, no
+ * counterpart in the reference whose launch shapes are compile-time constants,
+ * src/cuda/npc_kernel.h:10-14).  value 0 restores the default.
+ *   "sample_lanes_per_row"   8|16|32|64 lanes of a wavefront per frontier row
+ *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing */
+int apt_set_tuning(const char* key, int value);
+
+/* A CSR (CSC in the reference's naming: row v lists the in-neighbours of v)
+ * graph as the reference registers it with mix_cache_graphs
+ * (src/cache_graphs.cc:12-49, src/state.h:18-23).
+ *   indptr/indices        the "global" table (uva_* in the reference): row r
+ *                         describes node row_begin + r, r in [0, num_rows).
+ *   cached_indptr/indices optional second table (dev_* in the reference).
+ *   adj_pos_map           optional int64[num_total_nodes]: >= 0 -> row of the
+ *                         cached table, < -1 -> row -(p)-2 of the global
+ *                         table.  NULL = identity (node v is global row
+ *                         v - row_begin; nodes outside the range have no row
+ *                         and degree 0).
+ * All pointers are device memory. */
+typedef struct apt_graph {
+  const int64_t* indptr;
+  const int64_t* indices;
+  int64_t row_begin;
+  int64_t num_rows;
+  const int64_t* cached_indptr;
+  const int64_t* cached_indices;
+  int64_t num_cached_rows;
+  const int64_t* adj_pos_map;
+  int64_t num_total_nodes;
+} apt_graph;
+
+/* One hop of uniform neighbour sampling.
+ * Replaces LocalSampleNeighbors / _CSRRowWiseSampleReplaceKernel
+ * (src/cuda/npc_kernel.cu:248-316), op local_sample_one_layer
+ * (src/sampling.cc:13-17).
+ *
+ *   frontier          device int64[num_frontier]
+ *   num_frontier_dev  optional device int64[1]; when not NULL the kernel
+ *                     processes min(*num_frontier_dev, num_frontier) rows and
+ *                     the host value only sizes the launch
+ *   replace != 0      the reference's semantics: every row with degree > 0
+ *                     gets exactly `fanout` draws with replacement
+ *   replace == 0      without replacement: min(fanout, degree) neighbours;
+ *                     a row with degree <= fanout is copied whole, in CSR order
+ *   rng_seed, hop     Philox4x32-10 key (rng_seed) and counter word; the draw
+ *                     for output slot s of node v uses counter (v, hop, s), so
+ *                     results do not depend on launch geometry
+ *   out_neighbors     device int64[num_frontier * fanout], row-major, unused
+ *                     slots hold -1 (the reference leaves them uninitialised)
+ *   out_counts        optional device int64[num_frontier]
+ *   out_total         optional device int64[1], incremented by the number of
+ *                     sampled edges (caller clears it)
+ */
+int apt_sample_neighbors(const apt_graph* graph, const int64_t* frontier,
+                         int64_t num_frontier, const int64_t* num_frontier_dev,
+                         int fanout, int replace, uint64_t rng_seed, int hop,
+                         int64_t* out_neighbors, int64_t* out_counts,
+                         int64_t* out_total, void* stream);
+
+/* Relabel to compact ids in first-occurrence order.
+ * Replaces TensorRelabelCSC (src/cuda/relabel.cu:175-185), op relabel_csc
+ * (src/relabel.cc:9-15).
+ *
+ *   unique   = distinct non-negative values of cat(seeds, neighbors) in order
+ *              of first occurrence; device int64[num_seeds + num_neighbors]
+ *              capacity, the first *num_unique entries are written
+ *   relabeled[j] = position of neighbors[j] in unique (or neighbors[j] itself
+ *              if negative); device int64[num_neighbors]
+ *   num_seeds_dev      optional device int64[1] overriding num_seeds (<= it)
+ *   neighbor_stride    when num_seeds_dev is given the neighbours considered
+ *                      are the first *num_seeds_dev * neighbor_stride entries;
+ *                      otherwise ignored
+ *   num_unique_dev     device int64[1], receives the count
+ *   num_unique_host    optional host int64*; when not NULL the call
+ *                      synchronises the stream and stores the count there
+ *   workspace          device scratch of at least
+ *                      apt_relabel_workspace_bytes(num_seeds + num_neighbors)
+ */
+size_t apt_relabel_workspace_bytes(int64_t num_items);
+int apt_relabel(const int64_t* seeds, int64_t num_seeds,
+                const int64_t* num_seeds_dev, const int64_t* neighbors,
+                int64_t num_neighbors, int64_t neighbor_stride,
+                int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev,
+                int64_t* num_unique_host, void* workspace,
+                size_t workspace_bytes, void* stream);
+
+/* Feature tables as the reference registers them with cache_feats_shared
+ * (src/cache_feats.cc:14-61, src/state.h:10-16).
+ *   local_table  [num_local_rows, local_dim] elements ("uva_feats")
+ *   cache_table  [num_cache_rows, out_dim] elements ("dev_feats"), optional
+ *   pos_map      optional int64[num_total_nodes]: >= 0 cache row, < -1 local
+ *                row -(p)-2, -1 not present.  NULL = identity into
+ *                local_table.
+ *   col_offset   first column of local_table rows that is copied
+ *                ("feat_dim_offset"); out_dim columns are copied
+ *   elem_size    bytes per element: 4 (fp32, the reference) or 2 (bf16/fp16)
+ */
+typedef struct apt_feat_store {
+  const void* local_table;
+  int64_t num_local_rows;
+  int64_t local_dim;
+  const void* cache_table;
+  int64_t num_cache_rows;
+  const int64_t* pos_map;
+  int64_t num_total_nodes;
+  int64_t col_offset;
+  int64_t out_dim;
+  int elem_size;
+} apt_feat_store;
+
+/* Indexed feature gather: out[r, :] = row of node index[r].
+ * Replaces IndexSelectAll / _CSRRowWiseLoadSubtensorAlignedAllKernel
+ * (src/cuda/npc_kernel.cu:187-246), op load_subtensor
+ * (src/load_subtensor.cc:19-40).
+ *   index          device int64[num_index]
+ *   num_index_dev  optional device int64[1] (as in apt_sample_neighbors)
+ *   out            device [num_index, out_dim] elements
+ *   miss_count     optional device int64[1], incremented once per requested
+ *                  node that is not present (position -1, a negative id, or
+ *                  an id/position out of range); such rows are zero-filled
+ *                  (the reference reads out of bounds there)
+ */
+int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
+                    int64_t num_index, const int64_t* num_index_dev, void* out,
+                    int64_t* miss_count, void* stream);
+
+/* Row permutation of a dense [rows, dim] table, the on-GPU halves of
+ * FeatShuffle (src/feat_shuffle.cc:9-30) and the row gather by inverse_idx in
+ * front of it (python/npc/model/sage_model.py:67):
+ *   unpack (fwd):  out[i, :] = in[perm[i], :], i < n   (index_select, :27);
+ *                  a perm[i] outside [0, num_in_rows) yields a zero row
+ *   pack   (bwd):  out[perm[i], :] = in[i, :], i < n   (index_select_backward
+ *                  of a bijection, :14-16); rows of out that no perm[i] names
+ *                  are left untouched, so the caller zero-fills out first when
+ *                  perm is not onto; a perm[i] outside [0, num_out_rows) is
+ *                  skipped. */
+int apt_permute_rows(const void* in, int64_t num_in_rows, const int64_t* perm,
+                     int64_t n, int64_t dim, int elem_size, void* out,
+                     void* stream);
+int apt_scatter_rows(const void* in, const int64_t* perm, int64_t n,
+                     int64_t dim, int elem_size, void* out, int64_t num_out_rows,
+                     void* stream);
+
+/* Stable bucketing of ids by owner.
+ * Replaces ClusterAndPermute (src/cuda/npc_kernel.cu:318-382,434-470), the
+ * local half of ShuffleSeeds (src/sampling.cc:159-175).
+ *   owner(v): d = id_offset; while (d+1 < num_buckets && min_vids[d+1] <= v) ++d;
+ *             if (d < node_beg || d >= node_end) d = rank;
+ *   bucket_size[num_buckets], bucket_offset[num_buckets] (inclusive cumsum),
+ *   sorted_ids[n] (ids grouped by bucket, input order kept inside a bucket —
+ *   the reference's order inside a bucket is whatever its atomics produce),
+ *   permutation[n] (slot of ids[i] in sorted_ids).
+ *   min_vids     device int64[num_buckets + 1]
+ *   workspace    device scratch, apt_bucket_workspace_bytes(n, num_buckets)
+ */
+size_t apt_bucket_workspace_bytes(int64_t n, int num_buckets);
+int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* min_vids,
+                        int num_buckets, int64_t id_offset, int rank,
+                        int node_beg, int node_end, int64_t* bucket_size,
+                        int64_t* bucket_offset, int64_t* sorted_ids,
+                        int64_t* permutation, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* Bucketing of feature requests into "present here" (bucket 0) and per remote
+ * worker buckets.  Replaces MultiMachinesClusterAndPermute
+ * (src/cuda/npc_kernel.cu:384-432,472-508), op cluster_reqs
+ * (src/load_subtensor.cc:83-86).
+ *   bucket(v) = feat_pos_map[v] != -1 ? 0 : remote_worker_map[owner(v)]
+ *   with owner(v) the min_vids scan above started at 0 and no rank override.
+ *   bucket_offset is optional (NULL to skip). */
+int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* feat_pos_map,
+                     int64_t num_total_nodes, const int64_t* remote_worker_map,
+                     const int64_t* min_vids, int world_size,
+                     int num_remote_workers, int64_t* bucket_size,
+                     int64_t* bucket_offset, int64_t* sorted_ids,
+                     int64_t* permutation, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APT_AMD_H_ */

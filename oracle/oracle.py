@@ -1,0 +1,259 @@
+"""ctypes front end of oracle/liborc.so (built from oracle/oracle.c).
+
+TEST INFRASTRUCTURE ONLY: the checker for the HIP library and the CPU baseline
+that bench.py reports.  All arrays are numpy, C-contiguous; ids are int64.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liborc.so")
+
+__all__ = [
+    "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
+    "sample_neighbors", "sample_positions", "relabel", "gather_rows",
+    "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
+    "set_threads", "max_threads", "sample_blocks",
+]
+
+
+def build(force=False):
+    """Compile oracle.c with gcc (a few seconds)."""
+    src = os.path.join(_HERE, "oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liborc.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+_lib = None
+
+
+class _CGraph(C.Structure):
+    _fields_ = [("indptr", C.c_void_p), ("indices", C.c_void_p),
+                ("row_begin", C.c_int64), ("num_rows", C.c_int64),
+                ("cached_indptr", C.c_void_p), ("cached_indices", C.c_void_p),
+                ("num_cached_rows", C.c_int64), ("adj_pos_map", C.c_void_p),
+                ("num_total_nodes", C.c_int64)]
+
+
+class _CFeat(C.Structure):
+    _fields_ = [("local_table", C.c_void_p), ("num_local_rows", C.c_int64),
+                ("local_dim", C.c_int64), ("cache_table", C.c_void_p),
+                ("num_cache_rows", C.c_int64), ("pos_map", C.c_void_p),
+                ("num_total_nodes", C.c_int64), ("col_offset", C.c_int64),
+                ("out_dim", C.c_int64), ("elem_size", C.c_int)]
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        L.orc_draw64.restype = C.c_uint64
+        L.orc_draw64.argtypes = [C.c_uint64, C.c_int64, C.c_int, C.c_uint32]
+        L.orc_bounded.restype = C.c_uint64
+        L.orc_bounded.argtypes = [C.c_uint64, C.c_uint64]
+        L.orc_sample_neighbors.restype = C.c_int64
+        L.orc_sample_positions.restype = C.c_int64
+        L.orc_sample_positions.argtypes = [C.c_int64, C.c_int, C.c_int, C.c_uint64,
+                                           C.c_int64, C.c_int, C.c_void_p]
+        L.orc_relabel.restype = C.c_int64
+        L.orc_gather_rows.restype = C.c_int64
+        L.orc_set_threads.argtypes = [C.c_int]
+        _lib = L
+    return _lib
+
+
+def set_threads(t):
+    lib().orc_set_threads(int(t))
+
+
+def max_threads():
+    return int(lib().orc_max_threads())
+
+
+def _i64(a):
+    a = np.ascontiguousarray(a, dtype=np.int64)
+    return a
+
+
+def _p(a):
+    return None if a is None else C.c_void_p(a.ctypes.data)
+
+
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, dtype=np.uint32).copy()
+    k = np.asarray(key, dtype=np.uint32).copy()
+    o = np.zeros(4, dtype=np.uint32)
+    lib().orc_philox4x32_10(_p(c), _p(k), _p(o))
+    return o
+
+
+def draw64(rng_seed, node, hop, slot):
+    return int(lib().orc_draw64(rng_seed, node, hop, slot))
+
+
+def bounded(r, n):
+    return int(lib().orc_bounded(r, n))
+
+
+class Graph:
+    """Host copy of a graph in the layout of apt_graph (include/apt_amd.h)."""
+
+    def __init__(self, indptr, indices, row_begin=0, cached_indptr=None,
+                 cached_indices=None, adj_pos_map=None, num_total_nodes=None):
+        self.indptr = _i64(indptr)
+        self.indices = _i64(indices)
+        self.row_begin = int(row_begin)
+        self.num_rows = len(self.indptr) - 1
+        self.cached_indptr = None if cached_indptr is None else _i64(cached_indptr)
+        self.cached_indices = None if cached_indices is None else _i64(cached_indices)
+        self.num_cached_rows = 0 if cached_indptr is None else len(self.cached_indptr) - 1
+        self.adj_pos_map = None if adj_pos_map is None else _i64(adj_pos_map)
+        if num_total_nodes is None:
+            num_total_nodes = (len(self.adj_pos_map) if adj_pos_map is not None
+                               else self.row_begin + self.num_rows)
+        self.num_total_nodes = int(num_total_nodes)
+
+    def c(self):
+        return _CGraph(_p(self.indptr), _p(self.indices), self.row_begin, self.num_rows,
+                       _p(self.cached_indptr), _p(self.cached_indices),
+                       self.num_cached_rows, _p(self.adj_pos_map), self.num_total_nodes)
+
+
+class FeatStore:
+    """Host copy of feature tables in the layout of apt_feat_store."""
+
+    def __init__(self, local_table, cache_table=None, pos_map=None, col_offset=0,
+                 out_dim=None, num_total_nodes=None):
+        self.local_table = np.ascontiguousarray(local_table)
+        self.cache_table = None if cache_table is None else np.ascontiguousarray(cache_table)
+        self.pos_map = None if pos_map is None else _i64(pos_map)
+        self.col_offset = int(col_offset)
+        self.local_dim = self.local_table.shape[1]
+        if out_dim is None:
+            out_dim = (self.cache_table.shape[1] if self.cache_table is not None
+                       and self.cache_table.shape[0] > 0 else self.local_dim - self.col_offset)
+        self.out_dim = int(out_dim)
+        self.elem_size = self.local_table.dtype.itemsize
+        if num_total_nodes is None:
+            num_total_nodes = len(self.pos_map) if self.pos_map is not None else self.local_table.shape[0]
+        self.num_total_nodes = int(num_total_nodes)
+
+    def c(self):
+        ct = self.cache_table
+        return _CFeat(_p(self.local_table), self.local_table.shape[0], self.local_dim,
+                      _p(ct), 0 if ct is None else ct.shape[0], _p(self.pos_map),
+                      self.num_total_nodes, self.col_offset, self.out_dim, self.elem_size)
+
+
+def sample_neighbors(graph, frontier, fanout, replace, rng_seed, hop):
+    """-> (neighbors int64[n*fanout] padded with -1, counts int64[n])."""
+    f = _i64(frontier)
+    out = np.empty(len(f) * fanout, dtype=np.int64)
+    cnt = np.empty(len(f), dtype=np.int64)
+    g = graph.c()
+    lib().orc_sample_neighbors(C.byref(g), _p(f), C.c_int64(len(f)), C.c_int(fanout),
+                               C.c_int(int(bool(replace))), C.c_uint64(rng_seed),
+                               C.c_int(hop), _p(out), _p(cnt))
+    return out, cnt
+
+
+def sample_positions(deg, fanout, replace, rng_seed, node, hop):
+    out = np.empty(fanout, dtype=np.int64)
+    c = lib().orc_sample_positions(deg, fanout, int(bool(replace)), rng_seed, node, hop, _p(out))
+    return out[:c]
+
+
+def relabel(seeds, neighbors):
+    """-> (unique int64[U], relabeled int64[len(neighbors)])."""
+    s = _i64(seeds)
+    nb = _i64(neighbors)
+    uniq = np.empty(len(s) + len(nb), dtype=np.int64)
+    rel = np.empty(len(nb), dtype=np.int64)
+    u = lib().orc_relabel(_p(s), C.c_int64(len(s)), _p(nb), C.c_int64(len(nb)), _p(uniq), _p(rel))
+    return uniq[:u].copy(), rel
+
+
+def gather_rows(store, index):
+    """-> (out [n, out_dim], number of requests that were not present)."""
+    idx = _i64(index)
+    out = np.empty((len(idx), store.out_dim), dtype=store.local_table.dtype)
+    st = store.c()
+    miss = lib().orc_gather_rows(C.byref(st), _p(idx), C.c_int64(len(idx)), _p(out))
+    return out, int(miss)
+
+
+def permute_rows(table, perm):
+    t = np.ascontiguousarray(table)
+    p = _i64(perm)
+    out = np.empty((len(p), t.shape[1]), dtype=t.dtype)
+    lib().orc_permute_rows(_p(t), _p(p), C.c_int64(len(p)), C.c_int64(t.shape[1]),
+                           C.c_int(t.dtype.itemsize), _p(out))
+    return out
+
+
+def scatter_rows(table, perm, num_out_rows=None):
+    t = np.ascontiguousarray(table)
+    p = _i64(perm)
+    out = np.zeros((num_out_rows or len(p), t.shape[1]), dtype=t.dtype)
+    lib().orc_scatter_rows(_p(t), _p(p), C.c_int64(len(p)), C.c_int64(t.shape[1]),
+                           C.c_int(t.dtype.itemsize), _p(out))
+    return out
+
+
+def cluster_permute(ids, min_vids, num_buckets, id_offset=0, rank=0, node_beg=0, node_end=None):
+    """-> (bucket_size, bucket_offset, sorted_ids, permutation)."""
+    v = _i64(ids)
+    mv = _i64(min_vids)
+    if node_end is None:
+        node_end = num_buckets
+    bs = np.zeros(num_buckets, dtype=np.int64)
+    bo = np.zeros(num_buckets, dtype=np.int64)
+    so = np.empty(len(v), dtype=np.int64)
+    pm = np.empty(len(v), dtype=np.int64)
+    lib().orc_cluster_permute(_p(v), C.c_int64(len(v)), _p(mv), C.c_int(num_buckets),
+                              C.c_int64(id_offset), C.c_int(rank), C.c_int(node_beg),
+                              C.c_int(node_end), _p(bs), _p(bo), _p(so), _p(pm))
+    return bs, bo, so, pm
+
+
+def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num_remote_workers):
+    """-> (bucket_size, bucket_offset, sorted_ids, permutation)."""
+    v = _i64(ids)
+    fm = _i64(feat_pos_map)
+    rw = _i64(remote_worker_map)
+    mv = _i64(min_vids)
+    bs = np.zeros(num_remote_workers, dtype=np.int64)
+    bo = np.zeros(num_remote_workers, dtype=np.int64)
+    so = np.empty(len(v), dtype=np.int64)
+    pm = np.empty(len(v), dtype=np.int64)
+    lib().orc_cluster_reqs(_p(v), C.c_int64(len(v)), _p(fm), C.c_int64(len(fm)), _p(rw), _p(mv),
+                           C.c_int(world_size), C.c_int(num_remote_workers), _p(bs), _p(bo),
+                           _p(so), _p(pm))
+    return bs, bo, so, pm
+
+
+def sample_blocks(graph, seeds, hop_fanouts, replace, rng_seed):
+    """Multi-hop driver restating python/npc/sampler.py:187-203,358-364 (DP
+    branch): hop h samples the current frontier with hop_fanouts[h] (the
+    caller has already reversed the reference's k-hop..1-hop list), relabels,
+    and the unique ids become the next frontier.
+
+    -> (input_nodes, blocks) with blocks outermost-first; each block is a dict
+    with seeds, neighbors (padded), counts, unique, relabeled (padded).
+    """
+    frontier = _i64(seeds)
+    blocks = []
+    for h, f in enumerate(hop_fanouts):
+        nbr, cnt = sample_neighbors(graph, frontier, f, replace, rng_seed, h)
+        uniq, rel = relabel(frontier, nbr)
+        blocks.insert(0, dict(seeds=frontier, neighbors=nbr, counts=cnt, unique=uniq,
+                              relabeled=rel, fanout=f))
+        frontier = uniq
+    return frontier, blocks
