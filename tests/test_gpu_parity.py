@@ -1,0 +1,279 @@
+"""HIP library vs CPU oracle through the C ABI, bit-exact (needs an MI355X)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import small_graph, special_graph
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def _graphs(orc, capi, indptr, indices, **kw):
+    og = orc.Graph(indptr, indices, **kw)
+    dkw = {k: (dev(v) if isinstance(v, np.ndarray) else v) for k, v in kw.items()}
+    return og, capi.Graph(dev(indptr), dev(indices), **dkw)
+
+
+# ------------------------------------------------------------------ sampling
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("fanout", [1, 5, 10, 15, 16, 17, 64, 65, 130])
+def test_sampling_special_rows(orc, capi, replace, fanout):
+    indptr, indices, degs = special_graph()
+    og, dg = _graphs(orc, capi, indptr, indices)
+    frontier = np.concatenate([np.arange(len(degs)), [-1, len(indptr) + 3, 5, 6, 6]])
+    want_n, want_c = orc.sample_neighbors(og, frontier, fanout, replace, 42, 3)
+    total = torch.zeros(1, dtype=torch.int64, device=DEV)
+    got_n, got_c = capi.sample_neighbors(dg, dev(frontier), fanout, replace, 42, 3, out_total=total)
+    assert np.array_equal(host(got_c), want_c)
+    assert np.array_equal(host(got_n), want_n)
+    assert int(total.item()) == int(want_c.sum())
+
+
+@pytest.mark.parametrize("lanes", [0, 8, 16, 32, 64])
+@pytest.mark.parametrize("replace", [False, True])
+def test_sampling_random_graph_all_lane_groups(orc, capi, lanes, replace):
+    indptr, indices = small_graph(20000, 16, seed=11)
+    og, dg = _graphs(orc, capi, indptr, indices)
+    rng = np.random.default_rng(lanes)
+    frontier = rng.integers(0, 20000, size=70001)               # ragged: not a multiple of any tile
+    capi.set_tuning("sample_lanes_per_row", lanes)
+    try:
+        for fanout, hop in [(5, 0), (10, 1), (15, 2)]:
+            want_n, want_c = orc.sample_neighbors(og, frontier, fanout, replace, 7, hop)
+            got_n, got_c = capi.sample_neighbors(dg, dev(frontier), fanout, replace, 7, hop)
+            assert np.array_equal(host(got_c), want_c)
+            assert np.array_equal(host(got_n), want_n)
+    finally:
+        capi.set_tuning("sample_lanes_per_row", 0)
+
+
+def test_sampling_position_map_and_partition(orc, capi):
+    indptr, indices = small_graph(5000, 12, seed=12)
+    n = 5000
+    cached = np.arange(0, n, 7)
+    c_indptr = np.zeros(len(cached) + 1, dtype=np.int64)
+    c_indptr[1:] = np.cumsum(indptr[cached + 1] - indptr[cached])
+    c_indices = np.concatenate([indices[indptr[v]:indptr[v + 1]] for v in cached])
+    pos = -np.arange(n, dtype=np.int64) - 2
+    pos[cached] = np.arange(len(cached))
+    og, dg = _graphs(orc, capi, indptr, indices, cached_indptr=c_indptr, cached_indices=c_indices,
+                     adj_pos_map=pos)
+    f = np.random.default_rng(0).integers(-2, n + 10, size=9000)
+    for replace in (False, True):
+        want = orc.sample_neighbors(og, f, 6, replace, 3, 0)
+        got = capi.sample_neighbors(dg, dev(f), 6, replace, 3, 0)
+        assert np.array_equal(host(got[0]), want[0]) and np.array_equal(host(got[1]), want[1])
+    og, dg = _graphs(orc, capi, indptr[1000:3001] - indptr[1000],
+                     indices[indptr[1000]:indptr[3000]], row_begin=1000)
+    want = orc.sample_neighbors(og, f, 6, False, 3, 0)
+    got = capi.sample_neighbors(dg, dev(f), 6, False, 3, 0)
+    assert np.array_equal(host(got[0]), want[0]) and np.array_equal(host(got[1]), want[1])
+
+
+def test_sampling_device_side_count_and_empty(orc, capi):
+    indptr, indices = small_graph(3000, 10, seed=13)
+    og, dg = _graphs(orc, capi, indptr, indices)
+    f = np.arange(3000)
+    cnt = torch.tensor([1234], dtype=torch.int64, device=DEV)
+    out = torch.full((3000 * 4,), -7, dtype=torch.int64, device=DEV)
+    capi.sample_neighbors(dg, dev(f), 4, False, 1, 0, num_frontier_dev=cnt, out_neighbors=out)
+    want, _ = orc.sample_neighbors(og, f[:1234], 4, False, 1, 0)
+    o = host(out)
+    assert np.array_equal(o[:1234 * 4], want) and np.all(o[1234 * 4:] == -7)
+    e = capi.sample_neighbors(dg, dev(np.array([], dtype=np.int64)), 4, False, 1, 0)
+    assert e[0].numel() == 0 and e[1].numel() == 0
+
+
+def test_sampling_bad_arguments(capi):
+    indptr, indices = small_graph(100, 4, seed=1)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    with pytest.raises(capi.AptError):
+        capi.sample_neighbors(dg, dev(np.arange(4)), 0, False, 1, 0)
+    with pytest.raises(capi.AptError):
+        capi.sample_neighbors(dg, dev(np.arange(4)), 5000, False, 1, 0)
+    with pytest.raises(TypeError):
+        capi.sample_neighbors(dg, torch.arange(4), 3, False, 1, 0)          # CPU tensor
+    with pytest.raises(TypeError):
+        capi.sample_neighbors(dg, torch.arange(4, device=DEV, dtype=torch.int32), 3, False, 1, 0)
+
+
+# ------------------------------------------------------------------ relabel
+def _relabel_case(orc, capi, seeds, nbrs):
+    want_u, want_r = orc.relabel(seeds, nbrs)
+    u, r, n = capi.relabel(dev(np.asarray(seeds, np.int64)), dev(np.asarray(nbrs, np.int64)))
+    assert n == len(want_u)
+    assert np.array_equal(host(u), want_u)
+    assert np.array_equal(host(r), want_r)
+
+
+def test_relabel_random_sizes(orc, capi):
+    rng = np.random.default_rng(0)
+    for ns, f, hi in [(1, 1, 5), (10, 3, 20), (1024, 5, 3000), (6144, 10, 100000),
+                      (67584, 15, 2_400_000), (1023, 1, 1 << 40)]:
+        seeds = rng.permutation(min(hi, 10_000_000))[:ns].astype(np.int64)
+        nbrs = rng.integers(0, hi, size=ns * f)
+        _relabel_case(orc, capi, seeds, nbrs)
+
+
+def test_relabel_specials(orc, capi):
+    rng = np.random.default_rng(1)
+    e = np.array([], dtype=np.int64)
+    _relabel_case(orc, capi, np.array([5, 9, 7]), e)
+    _relabel_case(orc, capi, e, np.array([3, 3, 1, 3]))
+    _relabel_case(orc, capi, e, e)
+    _relabel_case(orc, capi, np.array([4]), np.full(5000, 4))
+    _relabel_case(orc, capi, np.array([2, 2, 8, 2]), np.array([8, 1, 2, 1]))
+    _relabel_case(orc, capi, np.arange(512), rng.integers(0, 512, 512))
+    _relabel_case(orc, capi, np.arange(1024), rng.integers(0, 1024, 1024 * 3))
+    big = 111_059_956
+    _relabel_case(orc, capi, np.array([big - 1, 0, big - 2]), rng.integers(big - 50, big, 640))
+    _relabel_case(orc, capi, np.arange(8) * 4096, rng.integers(0, 8, 1000) * 4096)
+    _relabel_case(orc, capi, np.array([3, 1]), np.array([1, -1, 7, -1, 3]))
+    # heavy duplication (hub ids) in a large list
+    hubs = rng.integers(0, 50, size=300000)
+    tail = rng.integers(0, 5_000_000, size=300000)
+    _relabel_case(orc, capi, rng.permutation(5_000_000)[:4096], rng.permutation(np.concatenate([hubs, tail])))
+
+
+def test_relabel_device_side_count(orc, capi):
+    rng = np.random.default_rng(2)
+    cap, f, real = 5000, 5, 3210
+    seeds = rng.permutation(100000)[:cap]
+    nbrs = rng.integers(0, 100000, size=cap * f)
+    cnt = torch.tensor([real], dtype=torch.int64, device=DEV)
+    u, r, nu = capi.relabel(dev(seeds), dev(nbrs), num_seeds_dev=cnt, neighbor_stride=f, sync=False)
+    want_u, want_r = orc.relabel(seeds[:real], nbrs[:real * f])
+    n = int(nu.item())
+    assert n == len(want_u)
+    assert np.array_equal(host(u)[:n], want_u)
+    assert np.array_equal(host(r)[:real * f], want_r)
+
+
+# ------------------------------------------------------------------ gather
+def _rand_table(rng, rows, dim, dtype):
+    if dtype == torch.float32:
+        return rng.standard_normal((rows, dim)).astype(np.float32)
+    return rng.integers(0, 65535, size=(rows, dim)).astype(np.uint16)   # raw 16-bit patterns
+
+
+def _to_dev_table(a, dtype):
+    t = torch.from_numpy(a.view(np.int16) if a.dtype == np.uint16 else a).to(DEV)
+    return t.view(dtype) if a.dtype == np.uint16 else t
+
+
+@pytest.mark.parametrize("dtype,dim", [(torch.float32, 128), (torch.float32, 100), (torch.bfloat16, 128),
+                                       (torch.float32, 7), (torch.bfloat16, 5), (torch.float32, 256),
+                                       (torch.float32, 602), (torch.bfloat16, 1024), (torch.float32, 2)])
+@pytest.mark.parametrize("rows_in_flight", [0, 1, 8])
+def test_gather_identity_map(orc, capi, dtype, dim, rows_in_flight):
+    rng = np.random.default_rng(dim)
+    table = _rand_table(rng, 5000, dim, dtype)
+    idx = np.concatenate([rng.integers(0, 5000, size=20011), [-1, 5000, 4999, 0]])
+    want, wmiss = orc.gather_rows(orc.FeatStore(table), idx)
+    capi.set_tuning("gather_rows_in_flight", rows_in_flight)
+    try:
+        miss = torch.zeros(1, dtype=torch.int64, device=DEV)
+        st = capi.FeatStore(_to_dev_table(table, dtype))
+        out = capi.gather_rows(st, dev(idx), miss_count=miss)
+    finally:
+        capi.set_tuning("gather_rows_in_flight", 0)
+    got = host(out.view(torch.int16) if dtype == torch.bfloat16 else out)
+    assert np.array_equal(got.view(want.dtype), want)
+    assert int(miss.item()) == wmiss == 2
+
+
+@pytest.mark.parametrize("D,Dr,off", [(128, 128, 0), (128, 32, 64), (24, 8, 12), (25, 7, 3), (100, 50, 50)])
+def test_gather_two_tables(orc, capi, D, Dr, off):
+    rng = np.random.default_rng(D + off)
+    total, nloc, ncache = 20000, 6000, 1500
+    local = rng.standard_normal((nloc, D)).astype(np.float32)
+    cache = rng.standard_normal((ncache, Dr)).astype(np.float32)
+    local_idx = rng.permutation(total)[:nloc]
+    cached_idx = np.concatenate([local_idx[:700], np.setdiff1d(np.arange(total), local_idx)[:800]])
+    pos = np.full(total, -1, dtype=np.int64)
+    pos[local_idx] = -np.arange(nloc) - 2
+    pos[cached_idx] = np.arange(ncache)
+    idx = np.concatenate([rng.integers(0, total, 30000), [-1, total, total + 7]])
+    want, wmiss = orc.gather_rows(orc.FeatStore(local, cache, pos, col_offset=off, out_dim=Dr), idx)
+    miss = torch.zeros(1, dtype=torch.int64, device=DEV)
+    st = capi.FeatStore(dev(local), dev(cache), dev(pos), col_offset=off, out_dim=Dr)
+    out = capi.gather_rows(st, dev(idx), miss_count=miss)
+    assert np.array_equal(host(out), want)
+    assert int(miss.item()) == wmiss
+
+
+def test_gather_empty_and_device_count(orc, capi):
+    rng = np.random.default_rng(9)
+    table = rng.standard_normal((1000, 64)).astype(np.float32)
+    st = capi.FeatStore(dev(table))
+    assert capi.gather_rows(st, dev(np.array([], dtype=np.int64))).shape == (0, 64)
+    idx = rng.integers(0, 1000, 4000)
+    cnt = torch.tensor([2500], dtype=torch.int64, device=DEV)
+    out = torch.full((4000, 64), 5.0, device=DEV)
+    capi.gather_rows(st, dev(idx), num_index_dev=cnt, out=out)
+    o = host(out)
+    assert np.array_equal(o[:2500], table[idx[:2500]]) and np.all(o[2500:] == 5.0)
+
+
+def test_permute_scatter_rows(orc, capi):
+    rng = np.random.default_rng(10)
+    for dim, dtype in [(16, torch.float32), (256, torch.float32), (64, torch.bfloat16), (3, torch.float32)]:
+        x = _rand_table(rng, 4321, dim, dtype)
+        perm = rng.permutation(4321)
+        xd = _to_dev_table(x, dtype)
+        up = capi.permute_rows(xd, dev(perm))
+        pk = capi.scatter_rows(xd, dev(perm))
+        as_np = lambda t: host(t.view(torch.int16) if dtype == torch.bfloat16 else t).view(x.dtype)
+        assert np.array_equal(as_np(up), orc.permute_rows(x, perm))
+        assert np.array_equal(as_np(pk), orc.scatter_rows(x, perm))
+        assert np.array_equal(as_np(capi.permute_rows(pk, dev(perm))), x)       # round trip
+    # un-unique gather: more outputs than inputs
+    inv = rng.integers(0, 100, size=999)
+    x = rng.standard_normal((100, 32)).astype(np.float32)
+    assert np.array_equal(host(capi.permute_rows(dev(x), dev(inv))), x[inv])
+
+
+# ------------------------------------------------------------------ bucketing
+def test_cluster_permute_reference_fixture(orc, capi):
+    for W in (1, 2, 4, 8):
+        for rank in range(W):
+            min_vids = 100 * np.arange(W + 1)
+            seeds = W * np.arange(99) + rank
+            want = orc.cluster_permute(seeds, min_vids, W, 0, rank, 0, W)
+            got = capi.cluster_permute(dev(seeds), dev(min_vids), W, 0, rank, 0, W)
+            for g, w in zip(got, want):
+                assert np.array_equal(host(g), w)
+
+
+def test_cluster_permute_random(orc, capi):
+    rng = np.random.default_rng(5)
+    for W, n in [(8, 5000), (8, 1_080_000), (33, 70001), (64, 12345), (1, 1000), (8, 0)]:
+        min_vids = np.concatenate([[0], np.sort(rng.integers(1, 10**7, W - 1)), [10**7]]).astype(np.int64)
+        ids = rng.integers(0, 10**7, size=n)
+        for (off, rank, beg, end) in [(0, 0, 0, W), (0, W // 2, W // 2, W), (min(2, W - 1), 0, 0, W)]:
+            want = orc.cluster_permute(ids, min_vids, W, off, rank, beg, end)
+            got = capi.cluster_permute(dev(ids), dev(min_vids), W, off, rank, beg, end)
+            for g, w in zip(got, want):
+                assert np.array_equal(host(g), w)
+
+
+def test_cluster_reqs(orc, capi):
+    rng = np.random.default_rng(6)
+    W, R, total = 8, 4, 200000
+    min_vids = np.arange(W + 1) * (total // W)
+    fm = np.where(rng.random(total) < 0.4, -1, rng.integers(-5000, 5000, total)).astype(np.int64)
+    rwm = np.array([0, 0, 1, 1, 2, 2, 3, 3])
+    ids = rng.integers(0, total, size=300000)
+    want = orc.cluster_reqs(ids, fm, rwm, min_vids, W, R)
+    got = capi.cluster_reqs(dev(ids), dev(fm), dev(rwm), dev(min_vids), W, R)
+    for g, w in zip(got, want):
+        assert np.array_equal(host(g), w)
