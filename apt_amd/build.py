@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libapt_hip.so")
-SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip"]
+SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "synth.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -28,7 +28,8 @@ def _obj(src):
 def build(force=True, verbose=False):
     """Compile every source and link libapt_hip.so.  Returns its path."""
     procs = []
-    headers = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "apt_amd.h")]
+    headers = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "apt_amd.h"),
+               os.path.join(HERE, "..", "include", "apt_synth.h")]
     newest_hdr = max(os.path.getmtime(h) for h in headers)
     objs = []
     for s in SOURCES:

@@ -51,6 +51,8 @@ SYMBOLS = {
     "apt_bucket_workspace_bytes": (_SZ, [_I64, _I]),
     "apt_cluster_permute": (_I, [_P, _I64, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_cluster_reqs": (_I, [_P, _I64, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+    # include/apt_synth.h
+    "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
 }
 
 
@@ -307,3 +309,14 @@ def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num
                                  int(num_remote_workers), _ptr(bs), _ptr(bo), _ptr(so), _ptr(pm),
                                  _ptr(ws), ws.numel(), _stream()))
     return bs, bo, so, pm
+
+
+def synth_rmat_fill(indptr, num_nodes, num_edges, levels, seed, thr0, thr1, indices):
+    indptr = _dev_i64(indptr, "indptr")
+    indices = _dev_i64(indices, "indices")
+    if indices.numel() < num_edges or indptr.numel() != num_nodes + 1:
+        raise AptError("synth_rmat_fill: buffer sizes do not match")
+    check(lib().apt_synth_rmat_fill(_ptr(indptr), int(num_nodes), int(num_edges), int(levels),
+                                    int(seed) & 0xFFFFFFFFFFFFFFFF, int(thr0), int(thr1),
+                                    _ptr(indices), _stream()))
+    return indices

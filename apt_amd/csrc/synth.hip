@@ -1,0 +1,90 @@
+// R-MAT neighbour-list generator (benchmark / test input, not on the
+// reference's path).  See include/apt_synth.h.
+#include "common.hpp"
+#include "../../include/apt_synth.h"
+
+namespace apt {
+
+constexpr int kSynBlock = 256;
+constexpr int kSynEdgesPerBlock = 4096;
+
+// Last row r in [lo, hi] with indptr[r] <= e.
+__device__ __forceinline__ int64_t row_of_edge(const int64_t* indptr, int64_t lo, int64_t hi,
+                                               int64_t e) {
+  while (lo < hi) {
+    const int64_t mid = lo + (hi - lo + 1) / 2;
+    if (indptr[mid] <= e) lo = mid;
+    else hi = mid - 1;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(kSynBlock) void rmat_fill_kernel(
+    const int64_t* __restrict__ indptr, int64_t num_nodes, int64_t num_edges, int levels,
+    uint64_t seed, uint32_t thr0, uint32_t thr1, int64_t* __restrict__ indices) {
+  __shared__ int64_t s_lo, s_hi;
+  const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kSynEdgesPerBlock;
+  if (e0 >= num_edges) return;
+  const int64_t e1 = min(e0 + kSynEdgesPerBlock, num_edges) - 1;
+  if (threadIdx.x == 0) s_lo = row_of_edge(indptr, 0, num_nodes - 1, e0);
+  if (threadIdx.x == 1) s_hi = row_of_edge(indptr, 0, num_nodes - 1, e1);
+  __syncthreads();
+  const int64_t lo = s_lo, hi = s_hi;
+  for (int64_t e = e0 + threadIdx.x; e <= e1; e += kSynBlock) {
+    const int64_t u = row_of_edge(indptr, lo, hi, e);
+    int64_t v = 0;
+    for (uint32_t attempt = 0; attempt < 32; ++attempt) {
+      v = 0;
+      for (int l0 = 0; l0 < levels; l0 += 8) {
+        uint32_t w[4];
+        {
+          uint32_t c0 = static_cast<uint32_t>(static_cast<uint64_t>(e));
+          uint32_t c1 = static_cast<uint32_t>(static_cast<uint64_t>(e) >> 32);
+          uint32_t c2 = static_cast<uint32_t>(l0), c3 = attempt;
+          uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
+#pragma unroll
+          for (int r = 0; r < 10; ++r) {
+            const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+            const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+            const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+            c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+            k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+          }
+          w[0] = c0; w[1] = c1; w[2] = c2; w[3] = c3;
+        }
+        const int lim = min(8, levels - l0);
+        for (int k = 0; k < lim; ++k) {
+          const int bitpos = levels - 1 - (l0 + k);          // MSB first
+          const uint32_t r16 = (w[k >> 1] >> ((k & 1) * 16)) & 0xFFFFu;
+          const uint32_t thr = ((u >> bitpos) & 1) ? thr1 : thr0;
+          v = (v << 1) | (r16 < thr ? 1 : 0);
+        }
+      }
+      if (v < num_nodes) break;
+    }
+    if (v >= num_nodes) v %= num_nodes;
+    indices[e] = v;
+  }
+}
+
+}  // namespace apt
+
+extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_edges,
+                                   int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
+                                   int64_t* indices, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_nodes > 0 && num_edges >= 0, APT_EINVAL, "apt_synth_rmat_fill: bad sizes");
+  APT_REQUIRE(levels >= 1 && levels <= 40 && (num_nodes - 1) >> levels == 0, APT_EINVAL,
+              "apt_synth_rmat_fill: %d levels do not cover %lld nodes", levels, (long long)num_nodes);
+  APT_REQUIRE(thr0 <= 65536 && thr1 <= 65536, APT_EINVAL, "apt_synth_rmat_fill: bad thresholds");
+  if (num_edges == 0) return APT_OK;
+  APT_REQUIRE(indptr != nullptr && indices != nullptr, APT_EINVAL,
+              "apt_synth_rmat_fill: indptr/indices is NULL");
+  const int64_t blocks = ceil_div(num_edges, kSynEdgesPerBlock);
+  APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT, "apt_synth_rmat_fill: too many edges");
+  hipLaunchKernelGGL(rmat_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kSynBlock), 0,
+                     static_cast<hipStream_t>(stream), indptr, num_nodes, num_edges, levels, seed,
+                     thr0, thr1, indices);
+  APT_LAUNCH_CHECK("rmat_fill_kernel");
+  return APT_OK;
+}

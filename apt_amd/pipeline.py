@@ -1,0 +1,85 @@
+"""Whole mini-batch on the GPU without host round trips.
+
+The reference's driver (python/npc/sampler.py:187-203,358-364 then
+python/npc/ops.py:598-600) synchronises the stream after every kernel and reads
+the unique count back on every hop.  Here every buffer is allocated once at its
+upper bound (hop h holds at most B * prod(1 + f_i) frontier rows), the counts
+stay in device memory and are read by the next kernel, and the host waits once
+per batch, when it wants the sizes.
+"""
+import torch
+
+from . import capi
+
+
+class MiniBatchPipeline:
+    def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True):
+        """hop_fanouts: fanout per hop starting from the seeds (the reference's
+        --fan_out list reversed)."""
+        self.graph, self.feat = graph, feat
+        self.fanouts = [int(f) for f in hop_fanouts]
+        self.replace = bool(replace)
+        dev = graph.device
+        self.device = dev
+        self.caps = [int(batch_size)]
+        for f in self.fanouts:
+            self.caps.append(self.caps[-1] * (1 + f))
+        i64 = dict(dtype=torch.int64, device=dev)
+        self.neighbors = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
+        self.relabeled = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
+        self.counts = [torch.empty(self.caps[h], **i64) for h in range(len(self.fanouts))]
+        self.frontier = [None] + [torch.empty(self.caps[h + 1], **i64) for h in range(len(self.fanouts))]
+        # sizes[h] = rows of the frontier entering hop h; sizes[-1] = input nodes; then edge total
+        self.sizes = torch.zeros(len(self.fanouts) + 2, **i64)
+        self.workspace = torch.empty(capi.relabel_workspace_bytes(self.caps[-1]), dtype=torch.uint8,
+                                     device=dev)
+        self.features = None
+        if gather and feat is not None:
+            self.features = torch.empty((self.caps[-1], feat.out_dim), dtype=feat.dtype, device=dev)
+        self.misses = torch.zeros(1, **i64)
+
+    def _size(self, h):
+        return self.sizes[h:h + 1]
+
+    def sample(self, seeds, rng_seed):
+        """Sampling + relabel for every hop, asynchronous."""
+        if seeds.numel() != self.caps[0]:
+            raise ValueError(f"expected {self.caps[0]} seeds, got {seeds.numel()}")
+        self.frontier[0] = seeds
+        self.sizes.zero_()
+        self.sizes[0:1].fill_(seeds.numel())
+        total = self.sizes[-1:]
+        for h, f in enumerate(self.fanouts):
+            n_dev = None if h == 0 else self._size(h)
+            capi.sample_neighbors(self.graph, self.frontier[h], f, self.replace, rng_seed, h,
+                                  num_frontier_dev=n_dev, out_neighbors=self.neighbors[h],
+                                  out_counts=self.counts[h], out_total=total)
+            capi.relabel(self.frontier[h], self.neighbors[h], num_seeds_dev=n_dev, neighbor_stride=f,
+                         unique=self.frontier[h + 1], relabeled=self.relabeled[h],
+                         num_unique_dev=self._size(h + 1), workspace=self.workspace, sync=False)
+
+    def gather(self):
+        """Features of the input nodes (the last hop's unique ids), asynchronous."""
+        H = len(self.fanouts)
+        capi.gather_rows(self.feat, self.frontier[H], num_index_dev=self._size(H), out=self.features,
+                         miss_count=self.misses)
+
+    def run(self, seeds, rng_seed):
+        self.sample(seeds, rng_seed)
+        if self.features is not None:
+            self.gather()
+
+    def result(self):
+        """Waits for the batch and narrows the buffers to their real sizes ->
+        dict(input_nodes, blocks (outermost first), features, num_edges)."""
+        sizes = self.sizes.cpu().tolist()
+        H = len(self.fanouts)
+        blocks = []
+        for h, f in enumerate(self.fanouts):
+            n = sizes[h]
+            blocks.insert(0, dict(seeds=self.frontier[h][:n], neighbors=self.neighbors[h][:n * f],
+                                  relabeled=self.relabeled[h][:n * f], counts=self.counts[h][:n],
+                                  unique=self.frontier[h + 1][:sizes[h + 1]], fanout=f))
+        feats = None if self.features is None else self.features[:sizes[H]]
+        return dict(input_nodes=self.frontier[H][:sizes[H]], blocks=blocks, features=feats,
+                    num_edges=sizes[-1], sizes=sizes[:-1])

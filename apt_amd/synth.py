@@ -59,3 +59,71 @@ def csr_from_edges(num_nodes, row, col):
 def rmat_csr_numpy(num_nodes, num_edges, seed):
     row, col = rmat_edges_numpy(num_nodes, num_edges, seed)
     return csr_from_edges(num_nodes, row, col)
+
+
+def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B, c=RMAT_C):
+    """Large R-MAT graph built directly in CSR on the GPU, without a sort.
+
+    R-MAT's recursive quadrant choice factorises over bits: row id u has
+    probability prod_l (a+b if bit_l(u)==0 else c+d), and given the row the
+    neighbour's bits are independent.  So row degrees are drawn as
+    Poisson(E * p_u / Z) (ids >= num_nodes excluded, i.e. rejected) and every
+    neighbour slot is then filled independently by apt_synth_rmat_fill.
+    Neighbour lists are unsorted and may repeat an id (multigraph), which the
+    samplers treat as distinct positions.
+
+    -> (indptr int64[num_nodes+1], indices int64[E'], E' ~ num_edges)
+    """
+    import math
+
+    import torch
+
+    from . import capi
+
+    d = 1.0 - a - b - c
+    levels = max(1, int(math.ceil(math.log2(max(num_nodes, 2)))))
+    gen = torch.Generator(device=device)
+    gen.manual_seed(int(seed))
+    l0, l1 = math.log(a + b), math.log(c + d)
+    indptr = torch.zeros(num_nodes + 1, dtype=torch.int64, device=device)
+    chunk = 1 << 24
+    # normaliser over ids < num_nodes, in float64
+    z = 0.0
+    logp_chunks = []
+    for s in range(0, num_nodes, chunk):
+        u = torch.arange(s, min(s + chunk, num_nodes), dtype=torch.int64, device=device)
+        pc = torch.zeros_like(u)
+        for bit in range(levels):
+            pc += (u >> bit) & 1
+        logp = (levels - pc).to(torch.float64) * l0 + pc.to(torch.float64) * l1
+        z += float(torch.exp(logp).sum().item())
+        logp_chunks.append((s, logp.to(torch.float32)))
+        del u, pc, logp
+    scale = math.log(num_edges) - math.log(z)
+    for s, logp in logp_chunks:
+        rate = torch.exp(logp.to(torch.float64) + scale).to(torch.float32)
+        deg = torch.poisson(rate, generator=gen).to(torch.int64)
+        indptr[s + 1:s + 1 + deg.numel()] = deg
+        del rate, deg
+    del logp_chunks
+    torch.cumsum(indptr, 0, out=indptr)
+    total = int(indptr[-1].item())
+    indices = torch.empty(total, dtype=torch.int64, device=device)
+    thr0 = int(round(65536 * b / (a + b)))
+    thr1 = int(round(65536 * d / (c + d)))
+    capi.synth_rmat_fill(indptr, num_nodes, total, levels, seed, thr0, thr1, indices)
+    return indptr, indices
+
+
+def random_features(num_rows, dim, dtype, seed, device="cuda:0"):
+    """~N(0,1) feature table generated on the GPU in chunks."""
+    import torch
+
+    gen = torch.Generator(device=device)
+    gen.manual_seed(int(seed))
+    out = torch.empty((num_rows, dim), dtype=dtype, device=device)
+    step = max(1, (1 << 28) // max(dim, 1))
+    for s in range(0, num_rows, step):
+        e = min(s + step, num_rows)
+        out[s:e] = torch.randn((e - s, dim), generator=gen, device=device, dtype=torch.float32).to(dtype)
+    return out

@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Mini-batch construction benchmark on one MI355X.
+
+A step is one mini-batch: multi-hop uniform neighbour sampling without
+replacement + relabel on every hop + feature gather of the input nodes, with
+the graph, the feature table and the seeds resident in HBM.  Prints ONE JSON
+line: sampled edges/s for the whole step, the gather kernel's achieved HBM
+bandwidth against the 8 TB/s peak (roofline), and the CPU oracle timed on this
+machine's host cores on a bounded sample of the same workload (cpu_baseline).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload full|medium|small]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # BASELINE.json configs[3]: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
+    "full": dict(nodes=111_059_956, edges=3_200_000_000, dim=128, dtype="bf16", batch=4096,
+                 fan_out=[15, 10, 5]),
+    # configs[1]: products-sized, 62M edges, 100 x fp32, batch 1024
+    "medium": dict(nodes=2_449_029, edges=62_000_000, dim=100, dtype="fp32", batch=1024,
+                   fan_out=[15, 10, 5]),
+    # configs[0]: CPU-runnable plumbing case
+    "small": dict(nodes=100_000, edges=1_500_000, dim=128, dtype="fp32", batch=1024, fan_out=[10, 5]),
+}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="full", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch_size", type=int, default=None)
+    ap.add_argument("--fan_out", type=str, default=None,
+                    help="comma list, k-hop..1-hop as in the reference (the seeds use the last entry)")
+    ap.add_argument("--replace", action="store_true", help="sample with replacement (reference semantics)")
+    ap.add_argument("--cpu_batches", type=int, default=None, help="batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu_threads", type=int, default=None)
+    ap.add_argument("--seed", type=int, default=1)
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives); use --gpus 1")
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: launched with WORLD_SIZE > 1; this build runs on one GPU only")
+
+    import torch
+
+    from apt_amd import capi, synth
+    from apt_amd.pipeline import MiniBatchPipeline
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    capi.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = dict(WORKLOADS[args.workload])
+    if args.batch_size:
+        w["batch"] = args.batch_size
+    if args.fan_out:
+        w["fan_out"] = [int(x) for x in args.fan_out.split(",")]
+    hops = list(reversed(w["fan_out"]))            # reference python/npc/sampler.py:191
+    dtype = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    esize = 2 if w["dtype"] == "bf16" else 4
+    B, K, W = w["batch"], args.steps, args.warmup
+
+    t0 = time.time()
+    indptr, indices = synth.rmat_csr_gpu(w["nodes"], w["edges"], args.seed, dev)
+    feats = synth.random_features(w["nodes"], w["dim"], dtype, args.seed + 1, dev)
+    torch.cuda.synchronize()
+    t_setup = time.time() - t0
+    num_edges_graph = int(indices.numel())
+    max_deg = int((indptr[1:] - indptr[:-1]).max().item())
+
+    graph = capi.Graph(indptr, indices)
+    store = capi.FeatStore(feats)
+    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace)
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed + 2)
+    need = (K + W) * B
+    if need <= w["nodes"]:
+        pool = torch.randperm(w["nodes"], generator=gen, device=dev)[:need]
+        seed_sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(K + W)]
+    else:   # more seeds than nodes: each batch still without repetition
+        seed_sets = [torch.randperm(w["nodes"], generator=gen, device=dev)[:B].contiguous()
+                     for _ in range(K + W)]
+
+    # ---- warm-up
+    for i in range(W):
+        pipe.run(seed_sets[i], args.seed + 100 + i)
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly K steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        pipe.run(seed_sets[W + i], args.seed + 100 + W + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    # ---- per-stage pass over the same K batches (HIP events on the launch stream)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    t_sample = t_gather = 0.0
+    edges = rows = 0
+    hop_sizes = []
+    for i in range(K):
+        e0, e1, e2 = ev(), ev(), ev()
+        e0.record()
+        pipe.sample(seed_sets[W + i], args.seed + 100 + W + i)
+        e1.record()
+        pipe.gather()
+        e2.record()
+        torch.cuda.synchronize()
+        t_sample += e0.elapsed_time(e1)
+        t_gather += e1.elapsed_time(e2)
+        sizes = pipe.sizes.cpu().tolist()
+        edges += sizes[-1]
+        rows += sizes[len(hops)]
+        hop_sizes.append(sizes[:-1])
+    assert int(pipe.misses.item()) == 0
+    bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
+    gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
+    edges_per_s = edges / elapsed
+
+    # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
+    cpu = None
+    n_cpu = args.cpu_batches
+    if n_cpu is None:
+        n_cpu = {"full": 6, "medium": 20, "small": 40}[args.workload]
+    n_cpu = min(n_cpu, K)
+    if n_cpu > 0:
+        import numpy as np
+
+        import oracle as orc
+        threads = args.cpu_threads or min(16, orc.max_threads())
+        orc.set_threads(threads)
+        h_indptr = indptr.cpu().numpy()
+        h_indices = indices.cpu().numpy()
+        if dtype == torch.bfloat16:
+            h_feats = feats.view(torch.int16).cpu().numpy().view(np.uint16)
+        else:
+            h_feats = feats.cpu().numpy()
+        og = orc.Graph(h_indptr, h_indices)
+        ofs = orc.FeatStore(h_feats)
+        cpu_edges = 0
+        tc = 0.0
+        for i in range(n_cpu):
+            s = seed_sets[W + i].cpu().numpy()
+            t1 = time.perf_counter()
+            inp, blocks = orc.sample_blocks(og, s, hops, args.replace, args.seed + 100 + W + i)
+            orc.gather_rows(ofs, inp)
+            tc += time.perf_counter() - t1
+            cpu_edges += sum(int(b["counts"].sum()) for b in blocks)
+        cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
+                   sample=f"{n_cpu} of the {K} timed batches (same seeds and rng keys): sampling and "
+                          f"gather on {threads} OpenMP threads, relabel on 1; {tc:.1f} s of CPU work")
+        del h_indices, h_feats
+
+    out = {
+        "metric": "sampled edges/s (3-hop 15,10,5) + feature-gather GB/s as % of HBM peak",
+        "value": edges_per_s,
+        "unit": "edges/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": elapsed / K * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int64",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: R-MAT {w['nodes']} nodes / {num_edges_graph} directed edges "
+                        f"(max degree {max_deg}), features {w['dim']} x {w['dtype']}, batch {B}, "
+                        f"fan_out {w['fan_out']} (hops from the seeds: {hops}), "
+                        f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
+                        f"gather of all input nodes",
+            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"],
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": "gather_kernel",
+            "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gather_gbps / HBM_PEAK_GBPS, "traffic": None,
+            "bytes_per_row": bytes_per_row, "rows_per_launch": rows / K,
+            "avg_launch_us": t_gather / K * 1e3,
+        },
+        "cpu_baseline": cpu,
+        "stages": {
+            "edges_per_step": edges / K,
+            "input_nodes_per_step": rows / K,
+            "sample_relabel_ms": t_sample / K,
+            "gather_ms": t_gather / K,
+            "sample_relabel_edges_per_s": edges / (t_sample * 1e-3),
+            "frontier_sizes_last_step": hop_sizes[-1],
+            "setup_s": t_setup,
+        },
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,31 @@
+/*
+ * apt_synth.h — synthetic-input helpers of libapt_hip.so (benchmark and test
+ * support; no counterpart in the reference, which loads OGB datasets through
+ * DGL, scripts/preprocess_dataset.py).
+ */
+#ifndef APT_SYNTH_H_
+#define APT_SYNTH_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Fill the neighbour lists of an R-MAT graph whose row degrees are already
+ * fixed by indptr (device int64[num_nodes + 1]).  R-MAT factorises: given the
+ * bits of the row id u, each bit of a neighbour is an independent Bernoulli
+ * draw with P(1 | row bit 0) = b/(a+b) and P(1 | row bit 1) = d/(c+d), so the
+ * neighbour of edge slot e is drawn from Philox keyed by (seed, e) with no
+ * sort or transpose.  Candidates >= num_nodes are redrawn.
+ *   thr0, thr1   the two probabilities scaled to [0, 65536]
+ *   indices      device int64[indptr[num_nodes]] (output)
+ */
+int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_edges,
+                        int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
+                        int64_t* indices, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,148 @@
+"""The fused multi-hop pipeline and the operator layer vs the oracle's driver."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import small_graph
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _setup(orc, capi, n=30000, deg=14, dim=100, seed=21):
+    indptr, indices = small_graph(n, deg, seed=seed)
+    feats = np.random.default_rng(seed).standard_normal((n, dim)).astype(np.float32)
+    return indptr, indices, feats
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_pipeline_matches_oracle_driver(orc, capi, replace):
+    from apt_amd.pipeline import MiniBatchPipeline
+    indptr, indices, feats = _setup(orc, capi)
+    og = orc.Graph(indptr, indices)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    fs = capi.FeatStore(dev(feats))
+    hops = [5, 10, 15]
+    pipe = MiniBatchPipeline(dg, fs, 512, hops, replace=replace)
+    rng = np.random.default_rng(0)
+    for batch in range(3):                                   # buffers are reused across batches
+        seeds = rng.permutation(len(indptr) - 1)[:512]
+        pipe.run(dev(seeds), 1000 + batch)
+        res = pipe.result()
+        want_in, want_blocks = orc.sample_blocks(og, seeds, hops, replace, 1000 + batch)
+        assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+        for got, want in zip(res["blocks"], want_blocks):
+            for k in ("seeds", "neighbors", "relabeled", "counts", "unique"):
+                assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+        assert res["num_edges"] == sum(int(b["counts"].sum()) for b in want_blocks)
+        want_f, miss = orc.gather_rows(orc.FeatStore(feats), want_in)
+        assert miss == 0 and int(pipe.misses.item()) == 0
+        assert np.array_equal(res["features"].cpu().numpy(), want_f)
+        # structure (reference sampler.py:358-364): dst nodes are a prefix of src nodes
+        assert np.array_equal(want_in[:512], seeds)
+
+
+def test_operator_layer_dp_sampler(orc, capi):
+    import apt_amd as npc
+    from apt_amd.state import STATE
+    indptr, indices, feats = _setup(orc, capi, n=8000, dim=32, seed=5)
+    n = len(indptr) - 1
+    STATE.reset()
+    e = torch.empty(0, dtype=torch.int64)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
+    npc.cache_feats_shared(n, torch.from_numpy(feats), torch.empty(0, 32), e, torch.arange(n), 0)
+    og = orc.Graph(indptr, indices)
+    seeds = np.random.default_rng(1).permutation(n)[:256]
+    # reference-style: fanouts listed k-hop..1-hop, with replacement
+    npc.set_rng_seed(99)
+    sampler = npc.MixedPSNeighborSampler(0, 1, [15, 10, 5], "DP")
+    input_nodes, output_nodes, blocks = sampler.sample(None, dev(seeds))
+    frontier = seeds
+    for hop, (fanout, blk) in enumerate(zip([5, 10, 15], reversed(blocks))):
+        nbr, cnt = orc.sample_neighbors(og, frontier, fanout, True, 99, hop)
+        uniq, rel = orc.relabel(frontier, nbr)
+        keep = rel >= 0
+        assert np.array_equal(blk.row.cpu().numpy(), rel[keep])
+        assert np.array_equal(blk.col.cpu().numpy(), np.repeat(np.arange(len(frontier)), fanout)[keep])
+        assert blk.num_dst == len(frontier) and blk.num_src == len(uniq)
+        assert np.array_equal(blk.src_ids.cpu().numpy(), uniq)
+        frontier = uniq
+    assert np.array_equal(input_nodes.cpu().numpy(), frontier)
+    assert np.array_equal(output_nodes.cpu().numpy(), seeds)
+    _, x = npc.load_batch(type("A", (), {"system": "DP"})(), (input_nodes, output_nodes, blocks))
+    assert np.array_equal(x.cpu().numpy(), feats[frontier])
+    assert np.array_equal(npc.cpu_load_subtensor(input_nodes.cpu()).cpu().numpy(), feats[frontier])
+    with pytest.raises(IndexError):
+        npc.load_subtensor(torch.tensor([0, n + 5]))
+    with pytest.raises(NotImplementedError):
+        npc.np_sample_and_shuffle(dev(seeds), 5)
+    STATE.reset()
+
+
+def test_operator_layer_caches_and_buckets(orc, capi):
+    import apt_amd as npc
+    from apt_amd.state import STATE
+    indptr, indices, feats = _setup(orc, capi, n=6000, dim=24, seed=6)
+    n = len(indptr) - 1
+    rng = np.random.default_rng(2)
+    STATE.reset()
+    # graph cache: rows of the 500 highest-degree nodes in a second table
+    deg = np.diff(indptr)
+    hot = np.argsort(-deg, kind="stable")[:500]
+    c_indptr = np.zeros(501, dtype=np.int64)
+    c_indptr[1:] = np.cumsum(deg[hot])
+    c_indices = np.concatenate([indices[indptr[v]:indptr[v + 1]] for v in hot])
+    npc.mix_cache_graphs(500, torch.from_numpy(hot), torch.from_numpy(c_indptr), torch.from_numpy(c_indices),
+                         torch.from_numpy(indptr), torch.from_numpy(indices))
+    npc.set_rng_seed(5)
+    s, nb = npc.local_sample_one_layer(dev(np.arange(n)), 4)
+    want, _ = orc.sample_neighbors(orc.Graph(indptr, indices), np.arange(n), 4, True, 5, 0)
+    assert np.array_equal(nb.cpu().numpy(), want)
+    # feature cache with a column window (the reference's "model parallel" slice)
+    local_idx = rng.permutation(n)[:4000]
+    cached_idx = np.concatenate([local_idx[:300], np.setdiff1d(np.arange(n), local_idx)[:200]])
+    off, Dr = 8, 8
+    cache = rng.standard_normal((500, Dr)).astype(np.float32)
+    npc.cache_feats_shared(n, torch.from_numpy(feats[:4000]), torch.from_numpy(cache), torch.from_numpy(cached_idx),
+                           torch.from_numpy(local_idx), off)
+    pos = np.full(n, -1, dtype=np.int64)
+    pos[local_idx] = -np.arange(4000) - 2
+    pos[cached_idx] = np.arange(500)
+    present = np.flatnonzero(pos != -1)
+    idx = rng.choice(present, 3000)
+    want, miss = orc.gather_rows(orc.FeatStore(feats[:4000], cache, pos, col_offset=off, out_dim=Dr), idx)
+    assert miss == 0
+    assert np.array_equal(npc.load_subtensor(dev(idx)).cpu().numpy(), want)
+    # bucketing: 8 owners on one GPU
+    npc.set_topology(rank=2, world_size=8, node_size=8)
+    min_vids = np.arange(9) * (n // 8)
+    min_vids[-1] = n
+    npc.register_min_vids(torch.from_numpy(min_vids), 0)
+    ids = rng.integers(0, n, 5000)
+    got = npc.cluster_and_permute(dev(ids))
+    want = orc.cluster_permute(ids, min_vids, 8, 0, 2, 0, 8)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+    rwm = np.array([0, 1, 1, 2, 2, 3, 3, 3])
+    npc.register_multi_machines_scheme(torch.from_numpy(rwm), torch.arange(4))
+    got = npc.cluster_reqs(dev(ids))
+    want = orc.cluster_reqs(ids, pos, rwm, min_vids, 8, 4)
+    assert np.array_equal(got[0].cpu().numpy(), want[0])
+    assert np.array_equal(got[1].cpu().numpy(), want[2])
+    assert np.array_equal(got[2].cpu().numpy(), want[3])
+    # one GPU: shuffle_seeds / feat_shuffle degenerate to local permutes
+    npc.set_topology(rank=0, world_size=1)
+    npc.register_min_vids(torch.tensor([0, n]), 0)
+    recv, perm, recv_off, dev_off = npc.shuffle_seeds(dev(ids))
+    assert np.array_equal(recv.cpu().numpy()[perm.cpu().numpy()], ids)
+    assert recv_off.tolist() == [5000] and dev_off.tolist() == [5000]
+    h = torch.randn(5000, 16, device=DEV)
+    fwd = npc.feat_shuffle(h, dev_off, recv_off, perm, 16, 1)
+    assert torch.equal(fwd, h[perm])
+    bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm, 16, 0)
+    assert torch.equal(bwd, h)                                  # pack undoes unpack
+    STATE.reset()
