@@ -43,6 +43,7 @@ def parse_args():
     ap.add_argument("--cpu_batches", type=int, default=None, help="batches timed on the CPU oracle (0 = skip)")
     ap.add_argument("--cpu_threads", type=int, default=None)
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
 
@@ -61,6 +62,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     capi.lib()
+    for kv in filter(None, args.tune.split(",")):
+        key, val = kv.split("=")
+        capi.set_tuning(key, int(val))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
