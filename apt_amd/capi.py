@@ -51,6 +51,13 @@ SYMBOLS = {
     "apt_bucket_workspace_bytes": (_SZ, [_I64, _I]),
     "apt_cluster_permute": (_I, [_P, _I64, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_cluster_reqs": (_I, [_P, _I64, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_rank_table_bytes": (_SZ, [_I64]),
+    "apt_rank_table_init": (_I, [_P, _SZ, _P]),
+    "apt_minibatch_workspace_bytes": (_SZ, [_I64, C.POINTER(C.c_int), _I]),
+    "apt_minibatch_capacity": (_I64, [_I64, C.POINTER(C.c_int), _I, _I]),
+    "apt_minibatch_sample": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
+                                  _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
+                                  _SZ, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
 }
@@ -320,3 +327,57 @@ def synth_rmat_fill(indptr, num_nodes, num_edges, levels, seed, thr0, thr1, indi
                                     int(seed) & 0xFFFFFFFFFFFFFFFF, int(thr0), int(thr1),
                                     _ptr(indices), _stream()))
     return indices
+
+
+def rank_table(num_total_nodes, device):
+    """Allocates and initialises the node-indexed rank table of the fused
+    mini-batch driver (uint32 per node, all 0xFFFFFFFF)."""
+    nbytes = int(lib().apt_rank_table_bytes(int(num_total_nodes)))
+    if nbytes == 0 and num_total_nodes != 0:
+        raise AptError(f"rank table: {num_total_nodes} nodes not supported")
+    t = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+    check(lib().apt_rank_table_init(_ptr(t), t.numel(), _stream()))
+    return t
+
+
+class MinibatchPlan:
+    """Argument block of apt_minibatch_sample for fixed (batch, hop_fanouts):
+    capacities, buffers and the host-side pointer arrays."""
+
+    def __init__(self, graph, batch, hop_fanouts, replace=False, want_counts=True, table=None):
+        self.graph = graph
+        self.batch = int(batch)
+        self.fanouts = [int(f) for f in hop_fanouts]
+        self.replace = bool(replace)
+        H = len(self.fanouts)
+        self._cf = (C.c_int * H)(*self.fanouts)
+        dev = graph.device
+        self.caps = [int(lib().apt_minibatch_capacity(self.batch, self._cf, H, h)) for h in range(H + 1)]
+        if min(self.caps) < 0:
+            raise AptError("minibatch plan: unsupported batch / fanouts")
+        i64 = dict(dtype=torch.int64, device=dev)
+        self.nodes = torch.empty(max(self.caps[H], 1), **i64)
+        self.neighbors = [torch.empty(max(self.caps[h] * f, 1), **i64) for h, f in enumerate(self.fanouts)]
+        self.relabeled = [torch.empty(max(self.caps[h] * f, 1), **i64) for h, f in enumerate(self.fanouts)]
+        self.counts = [torch.empty(max(self.caps[h], 1), **i64) for h in range(H)] if want_counts else None
+        self.sizes = torch.zeros(H + 2, **i64)
+        self.rng_seed_dev = torch.zeros(1, **i64)
+        self.table = table if table is not None else rank_table(graph.num_total_nodes, dev)
+        self.table_len = graph.num_total_nodes
+        need = int(lib().apt_minibatch_workspace_bytes(self.batch, self._cf, H))
+        self.workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        self._nb = (C.c_void_p * H)(*[t.data_ptr() for t in self.neighbors])
+        self._rl = (C.c_void_p * H)(*[t.data_ptr() for t in self.relabeled])
+        self._ct = (C.c_void_p * H)(*[t.data_ptr() for t in self.counts]) if want_counts else None
+
+    def launch(self, seeds, rng_seed=None):
+        """Asynchronous.  rng_seed=None reads the seed from self.rng_seed_dev."""
+        seeds = _dev_i64(seeds, "seeds")
+        if seeds.numel() != self.batch:
+            raise AptError(f"expected {self.batch} seeds, got {seeds.numel()}")
+        check(lib().apt_minibatch_sample(
+            C.byref(self.graph.c), _ptr(seeds), self.batch, self._cf, len(self.fanouts),
+            int(self.replace), 0 if rng_seed is None else int(rng_seed) & 0xFFFFFFFFFFFFFFFF,
+            _ptr(self.rng_seed_dev) if rng_seed is None else None, _ptr(self.table), self.table_len,
+            _ptr(self.nodes), self._nb, self._rl, self._ct, _ptr(self.sizes), _ptr(self.workspace),
+            self.workspace.numel(), _stream()))

@@ -1,0 +1,423 @@
+// Fused multi-hop mini-batch construction: sample -> relabel for every hop in
+// one call, without host round trips.
+//
+// Counterpart of the DP branch of MixedPSNeighborSampler.sample (reference
+// python/npc/sampler.py:187-203,358-364), which per hop calls
+// local_sample_one_layer, relabel_csc (torch::cat + 3 hash passes + cub scan,
+// src/cuda/relabel.cu:78-185) and reads the unique count back to the host.
+//
+// Relabel here uses a node-indexed rank table instead of a hash table: one
+// uint32 per node of the graph, resident in HBM for the life of the process
+// (444 MB for 111M nodes; a few per mille of 288 GB).  table[v] is 0xFFFFFFFF
+// when v is not in the batch, otherwise the compact id of v.  Because the
+// unique list of hop h is the unique list of hop h-1 followed by the new nodes
+// in first-occurrence order (the order the reference's AtomicMin-on-index
+// produces), the list only ever grows and ids never change:
+//   * the frontier of hop h is nodes[0 : n_h], already marked with its ids;
+//   * a sampled neighbour that is already in the batch is relabelled by one
+//     load, with no atomic at all (hubs are almost always already there);
+//   * the others race with atomicMin on (n_h + slot index); the smallest index
+//     owns the node, owners are ranked with ballots + a two-level prefix, get
+//     id n_h + rank and are appended to the list.
+// Random atomics are the scarcest resource on this GPU (~20 G/s against
+// ~45 G/s random loads), which is why the table is indexed directly (no CAS
+// to claim a slot, no probing) and why nodes already present never touch one.
+// The table is restored to all-0xFFFFFFFF before the call returns control of
+// the stream, by walking the final node list.
+#include "common.hpp"
+
+namespace apt {
+
+int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
+                  const int64_t* num_frontier_dev, int fanout, int replace, uint64_t rng_seed,
+                  const uint64_t* rng_seed_dev, int hop, int64_t* out_neighbors, int64_t* out_counts,
+                  int64_t* out_total, hipStream_t st, const char* who);
+
+constexpr int kMbBlock = 256;
+constexpr int kMbIters = 4;
+constexpr int kMbTile = kMbBlock * kMbIters;     // items per workgroup in count / place
+constexpr int kMbWaves = kMbBlock / kWave;
+constexpr uint32_t kEmpty = 0xFFFFFFFFu;
+constexpr int64_t kPending = -2;                  // relabeled[] slot still to be looked up
+constexpr int kMaxHops = APT_MAX_HOPS;
+
+struct HopParams {
+  const int64_t* seeds;      // first hop: the caller's seeds; later hops: unused
+  int64_t ns_cap;            // frontier rows, host-side upper bound
+  const int64_t* ns_dev;     // actual frontier rows (NULL on the first hop)
+  int64_t fanout;
+  const int64_t* neighbors;  // [ns_cap * fanout], -1 padded
+  int64_t* relabeled;        // [ns_cap * fanout]
+  uint32_t* table;
+  int64_t table_len;
+  int64_t* nodes;            // growing unique list
+  int64_t* n_next;           // receives the size of the list after this hop
+  uint64_t* flags;           // owner bit per item, one word per wavefront-load
+  uint32_t* tile_cnt;
+};
+
+struct HopSizes {
+  int64_t ns, nn;
+};
+
+__device__ __forceinline__ HopSizes hop_sizes(const HopParams& p) {
+  HopSizes s;
+  s.ns = actual_count(p.ns_cap, p.ns_dev);
+  s.nn = s.ns * p.fanout;
+  return s;
+}
+
+__device__ __forceinline__ bool in_table(const HopParams& p, int64_t v) {
+  return v >= 0 && v < p.table_len;
+}
+
+// First hop only: seeds may repeat, so they race like everything else; the
+// smallest seed index owns the node.  Also clears the per-batch counters.
+__global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, int64_t* sizes,
+                                                                 int num_sizes) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x;
+  if (i < num_sizes) sizes[i] = i == 0 ? p.ns_cap : 0;
+  if (i < p.ns_cap) {
+    const int64_t v = p.seeds[i];
+    if (in_table(p, v)) atomicMin(&p.table[v], static_cast<uint32_t>(i));
+  }
+}
+
+// Every sampled slot: already in the batch -> relabelled now; otherwise bid
+// for ownership with (ns + slot index).  FIRST: the table holds seed indices,
+// not ids, so nothing can be finalised yet.
+template <bool FIRST>
+__global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p) {
+  const HopSizes s = hop_sizes(p);
+  for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < s.nn;
+       j += static_cast<int64_t>(gridDim.x) * kMbBlock) {
+    const int64_t v = p.neighbors[j];
+    int64_t out = kPending;
+    if (!in_table(p, v)) {
+      out = v < 0 ? v : -1;  // padding, or an id the table cannot hold: no edge
+    } else {
+      const uint32_t bid = static_cast<uint32_t>(s.ns + j);
+      // Values only decrease, so a stale read can only cause a redundant atomic.
+      const uint32_t cur = p.table[v];
+      if (!FIRST && cur < static_cast<uint32_t>(s.ns)) out = cur;
+      else if (cur > bid) atomicMin(&p.table[v], bid);
+    }
+    p.relabeled[j] = out;
+  }
+}
+
+// Item i of a hop: FIRST -> seeds followed by neighbours (index = bid);
+// later hops -> neighbours only (bid = ns + index).
+template <bool FIRST>
+__device__ __forceinline__ bool mb_is_owner(const HopParams& p, const HopSizes& s, int64_t i,
+                                            int64_t items) {
+  if (i >= items) return false;
+  int64_t v;
+  uint32_t bid;
+  if (FIRST) {
+    v = i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns];
+    bid = static_cast<uint32_t>(i);
+    if (!in_table(p, v)) return false;
+  } else {
+    if (p.relabeled[i] != kPending) return false;  // padding or already in the batch
+    v = p.neighbors[i];
+    bid = static_cast<uint32_t>(s.ns + i);
+  }
+  return p.table[v] == bid;
+}
+
+template <bool FIRST>
+__global__ __launch_bounds__(kMbBlock) void mb_count_kernel(HopParams p) {
+  const HopSizes s = hop_sizes(p);
+  const int64_t items = FIRST ? s.ns + s.nn : s.nn;
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kMbTile;
+  if (base >= items) return;
+  __shared__ uint32_t s_wave[kMbWaves];
+  const int wave = threadIdx.x / kWave;
+  uint32_t c = 0;
+#pragma unroll
+  for (int it = 0; it < kMbIters; ++it) {
+    const uint64_t m = ballot(mb_is_owner<FIRST>(p, s, base + it * kMbBlock + threadIdx.x, items));
+    if (lane_id() == 0) p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + wave] = m;
+    c += __popcll(m);
+  }
+  if (lane_id() == 0) s_wave[wave] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t t = 0;
+    for (int w = 0; w < kMbWaves; ++w) t += s_wave[w];
+    p.tile_cnt[blockIdx.x] = t;
+  }
+}
+
+// Owners get id base + (number of owners before them), are appended to the
+// node list and written into the table.
+template <bool FIRST>
+__global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
+  const HopSizes s = hop_sizes(p);
+  const int64_t items = FIRST ? s.ns + s.nn : s.nn;
+  const int64_t first_id = FIRST ? 0 : s.ns;
+  if (items == 0) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) *p.n_next = first_id;
+    return;
+  }
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kMbTile;
+  if (base >= items) return;
+  const int64_t tiles = (items + kMbTile - 1) / kMbTile;
+  __shared__ int64_t s_red[kMbWaves];
+  const int wave = threadIdx.x / kWave;
+  const int lane = lane_id();
+  int64_t part = 0;
+  for (int64_t b = threadIdx.x; b < blockIdx.x; b += kMbBlock) part += p.tile_cnt[b];
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_down(part, off, kWave);
+  if (lane == 0) s_red[wave] = part;
+  uint64_t mask[kMbIters][kMbWaves];
+#pragma unroll
+  for (int it = 0; it < kMbIters; ++it)
+#pragma unroll
+    for (int w = 0; w < kMbWaves; ++w)
+      mask[it][w] = p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + w];
+  __syncthreads();
+  int64_t running = first_id;
+  for (int w = 0; w < kMbWaves; ++w) running += s_red[w];
+#pragma unroll
+  for (int it = 0; it < kMbIters; ++it) {
+    int64_t before = running;
+#pragma unroll
+    for (int w = 0; w < kMbWaves; ++w) {
+      const int c = __popcll(mask[it][w]);
+      if (w < wave) before += c;
+      running += c;
+    }
+    uint64_t mine = 0;
+#pragma unroll
+    for (int w = 0; w < kMbWaves; ++w)
+      if (w == wave) mine = mask[it][w];
+    if ((mine >> lane) & 1) {
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      const int64_t id = before + rank_below(mine);
+      int64_t v;
+      if (FIRST) {
+        v = i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns];
+        if (i >= s.ns) p.relabeled[i - s.ns] = id;
+      } else {
+        v = p.neighbors[i];
+        p.relabeled[i] = id;
+      }
+      p.nodes[id] = v;
+      p.table[v] = static_cast<uint32_t>(id);
+    }
+  }
+  if (blockIdx.x == tiles - 1 && threadIdx.x == 0) *p.n_next = running;
+}
+
+struct LookupParams {
+  int num_hops;
+  int64_t block_begin[kMaxHops + 1];  // workgroup ranges per hop
+  const int64_t* neighbors[kMaxHops];
+  int64_t* relabeled[kMaxHops];
+  const int64_t* ns_dev[kMaxHops];
+  int64_t ns_cap[kMaxHops];
+  int64_t fanout[kMaxHops];
+  const uint32_t* table;
+};
+
+// Slots that lost the ownership race read the winner's id (all hops at once).
+__global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
+  int h = 0;
+  while (h + 1 < p.num_hops && static_cast<int64_t>(blockIdx.x) >= p.block_begin[h + 1]) ++h;
+  const int64_t nn = actual_count(p.ns_cap[h], p.ns_dev[h]) * p.fanout[h];
+  const int64_t blocks = p.block_begin[h + 1] - p.block_begin[h];
+  for (int64_t j = (static_cast<int64_t>(blockIdx.x) - p.block_begin[h]) * kMbBlock + threadIdx.x;
+       j < nn; j += blocks * kMbBlock) {
+    if (p.relabeled[h][j] == kPending) p.relabeled[h][j] = p.table[p.neighbors[h][j]];
+  }
+}
+
+// table[v] := empty for every node of the batch.
+__global__ __launch_bounds__(kMbBlock) void mb_reset_kernel(uint32_t* table, const int64_t* nodes,
+                                                            const int64_t* n_dev, int64_t n_cap) {
+  const int64_t n = actual_count(n_cap, n_dev);
+  for (int64_t r = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; r < n;
+       r += static_cast<int64_t>(gridDim.x) * kMbBlock)
+    table[nodes[r]] = kEmpty;
+}
+
+__global__ __launch_bounds__(kMbBlock) void mb_fill_table_kernel(uint4* table, int64_t vecs) {
+  const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
+       i += static_cast<int64_t>(gridDim.x) * kMbBlock)
+    table[i] = ones;
+}
+
+static size_t mb_align(size_t x) { return (x + 255) / 256 * 256; }
+
+struct MbLayout {
+  size_t flags_off, tile_off, total;
+  int64_t caps[kMaxHops + 1];
+  int64_t max_items;
+};
+
+static bool mb_layout(int64_t batch, const int* fanouts, int num_hops, MbLayout& L) {
+  L.caps[0] = batch;
+  L.max_items = 1;
+  for (int h = 0; h < num_hops; ++h) {
+    if (fanouts[h] <= 0) return false;
+    const int64_t f = fanouts[h];
+    if (L.caps[h] > (int64_t{1} << 31) / (1 + f)) return false;  // ids and bids are 32-bit
+    L.caps[h + 1] = L.caps[h] * (1 + f);
+    const int64_t items = h == 0 ? L.caps[h] * (1 + f) : L.caps[h] * f;
+    if (items > L.max_items) L.max_items = items;
+  }
+  const int64_t tiles = ceil_div(L.max_items, kMbTile);
+  size_t off = 0;
+  L.flags_off = off; off = mb_align(off + sizeof(uint64_t) * tiles * kMbIters * kMbWaves);
+  L.tile_off = off;  off = mb_align(off + sizeof(uint32_t) * tiles);
+  L.total = off;
+  return true;
+}
+
+}  // namespace apt
+
+extern "C" size_t apt_rank_table_bytes(int64_t num_total_nodes) {
+  if (num_total_nodes < 0 || num_total_nodes >= (int64_t{1} << 32) - 1) return 0;
+  return (static_cast<size_t>(num_total_nodes) * sizeof(uint32_t) + 255) / 256 * 256;
+}
+
+extern "C" int apt_rank_table_init(void* table, size_t table_bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(table != nullptr && table_bytes % 16 == 0 &&
+                  (reinterpret_cast<uintptr_t>(table) & 15) == 0,
+              APT_EINVAL, "apt_rank_table_init: table must be 16-byte aligned and sized");
+  if (table_bytes == 0) return APT_OK;
+  const int64_t vecs = static_cast<int64_t>(table_bytes / 16);
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(vecs, kMbBlock), 16384));
+  hipLaunchKernelGGL(mb_fill_table_kernel, dim3(blocks), dim3(kMbBlock), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint4*>(table), vecs);
+  APT_LAUNCH_CHECK("mb_fill_table_kernel");
+  return APT_OK;
+}
+
+extern "C" size_t apt_minibatch_workspace_bytes(int64_t batch, const int* hop_fanouts, int num_hops) {
+  apt::MbLayout L;
+  if (batch < 0 || hop_fanouts == nullptr || num_hops < 1 || num_hops > apt::kMaxHops) return 0;
+  if (!apt::mb_layout(batch, hop_fanouts, num_hops, L)) return 0;
+  return L.total;
+}
+
+extern "C" int64_t apt_minibatch_capacity(int64_t batch, const int* hop_fanouts, int num_hops, int hop) {
+  apt::MbLayout L;
+  if (batch < 0 || hop_fanouts == nullptr || num_hops < 1 || num_hops > apt::kMaxHops) return -1;
+  if (hop < 0 || hop > num_hops || !apt::mb_layout(batch, hop_fanouts, num_hops, L)) return -1;
+  return L.caps[hop];
+}
+
+extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                                    const int* hop_fanouts, int num_hops, int replace,
+                                    uint64_t rng_seed, const uint64_t* rng_seed_dev,
+                                    void* rank_table, int64_t rank_table_len, int64_t* nodes,
+                                    int64_t* const* neighbors, int64_t* const* relabeled,
+                                    int64_t* const* counts, int64_t* sizes, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(graph != nullptr, APT_EINVAL, "apt_minibatch_sample: graph is NULL");
+  APT_REQUIRE(batch >= 0, APT_EINVAL, "apt_minibatch_sample: batch %lld < 0", (long long)batch);
+  APT_REQUIRE(hop_fanouts != nullptr && num_hops >= 1 && num_hops <= kMaxHops, APT_ELIMIT,
+              "apt_minibatch_sample: num_hops %d outside [1, %d]", num_hops, kMaxHops);
+  MbLayout L;
+  APT_REQUIRE(mb_layout(batch, hop_fanouts, num_hops, L), APT_ELIMIT,
+              "apt_minibatch_sample: fanouts must be > 0 and batch * prod(1 + fanout) < 2^31");
+  APT_REQUIRE(rank_table != nullptr && rank_table_len > 0 && rank_table_len < (int64_t{1} << 32) - 1,
+              APT_EINVAL, "apt_minibatch_sample: rank table missing or too long");
+  APT_REQUIRE(sizes != nullptr && neighbors != nullptr && relabeled != nullptr, APT_EINVAL,
+              "apt_minibatch_sample: sizes/neighbors/relabeled is NULL");
+  APT_REQUIRE(batch == 0 || (seeds != nullptr && nodes != nullptr), APT_EINVAL,
+              "apt_minibatch_sample: seeds/nodes is NULL");
+  APT_REQUIRE(workspace != nullptr && workspace_bytes >= L.total, APT_EWORKSPACE,
+              "apt_minibatch_sample: workspace of %zu bytes, %zu needed", workspace_bytes, L.total);
+  for (int h = 0; h < num_hops; ++h)
+    APT_REQUIRE(batch == 0 || (neighbors[h] != nullptr && relabeled[h] != nullptr), APT_EINVAL,
+                "apt_minibatch_sample: neighbors[%d]/relabeled[%d] is NULL", h, h);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char* ws = static_cast<char*>(workspace);
+  int64_t* total = sizes + num_hops + 1;
+
+  HopParams hp{};
+  hp.table = static_cast<uint32_t*>(rank_table);
+  hp.table_len = rank_table_len;
+  hp.nodes = nodes;
+  hp.flags = reinterpret_cast<uint64_t*>(ws + L.flags_off);
+  hp.tile_cnt = reinterpret_cast<uint32_t*>(ws + L.tile_off);
+  hp.seeds = seeds;
+  hp.ns_cap = batch;
+  hp.ns_dev = nullptr;
+
+  // sizes[0] = batch, the rest 0; first-hop seeds bid for their nodes.
+  {
+    const int64_t work = std::max<int64_t>(batch, num_hops + 2);
+    hipLaunchKernelGGL(mb_mark_seeds_kernel, dim3(static_cast<unsigned>(ceil_div(work, kMbBlock))),
+                       dim3(kMbBlock), 0, st, hp, sizes, num_hops + 2);
+    APT_LAUNCH_CHECK("mb_mark_seeds_kernel");
+  }
+  if (batch == 0) return APT_OK;
+
+  auto grid_for = [](int64_t n, int64_t per_block, int64_t cap) {
+    return dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, per_block), cap))));
+  };
+  for (int h = 0; h < num_hops; ++h) {
+    const int64_t ns_cap = L.caps[h];
+    const int64_t f = hop_fanouts[h];
+    const int64_t nn_cap = ns_cap * f;
+    const int64_t* frontier = h == 0 ? seeds : nodes;
+    const int64_t* ns_dev = h == 0 ? nullptr : sizes + h;
+    int rc = sample_launch(graph, frontier, ns_cap, ns_dev, static_cast<int>(f), replace, rng_seed,
+                           rng_seed_dev, h, neighbors[h], counts != nullptr ? counts[h] : nullptr,
+                           total, st, "apt_minibatch_sample");
+    if (rc != APT_OK) return rc;
+    hp.ns_cap = ns_cap;
+    hp.ns_dev = ns_dev;
+    hp.fanout = f;
+    hp.neighbors = neighbors[h];
+    hp.relabeled = relabeled[h];
+    hp.n_next = sizes + h + 1;
+    const int64_t items_cap = h == 0 ? ns_cap + nn_cap : nn_cap;
+    const dim3 tiles = grid_for(items_cap, kMbTile, int64_t{1} << 30);
+    const dim3 flat = grid_for(nn_cap, kMbBlock, 1 << 16);
+    if (h == 0) {
+      hipLaunchKernelGGL(mb_mark_neighbors_kernel<true>, flat, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      hipLaunchKernelGGL(mb_count_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_count_kernel");
+      hipLaunchKernelGGL(mb_place_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_place_kernel");
+    } else {
+      hipLaunchKernelGGL(mb_mark_neighbors_kernel<false>, flat, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      hipLaunchKernelGGL(mb_count_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_count_kernel");
+      hipLaunchKernelGGL(mb_place_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_place_kernel");
+    }
+  }
+  LookupParams lp{};
+  lp.num_hops = num_hops;
+  lp.table = static_cast<const uint32_t*>(rank_table);
+  int64_t nblocks = 0;
+  for (int h = 0; h < num_hops; ++h) {
+    lp.block_begin[h] = nblocks;
+    lp.neighbors[h] = neighbors[h];
+    lp.relabeled[h] = relabeled[h];
+    lp.ns_dev[h] = h == 0 ? nullptr : sizes + h;
+    lp.ns_cap[h] = L.caps[h];
+    lp.fanout[h] = hop_fanouts[h];
+    nblocks += std::max<int64_t>(1, std::min<int64_t>(ceil_div(L.caps[h] * hop_fanouts[h], kMbBlock), 1 << 15));
+  }
+  lp.block_begin[num_hops] = nblocks;
+  hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kMbBlock), 0, st, lp);
+  APT_LAUNCH_CHECK("mb_lookup_kernel");
+  hipLaunchKernelGGL(mb_reset_kernel, grid_for(L.caps[num_hops], kMbBlock, 1 << 15), dim3(kMbBlock), 0,
+                     st, static_cast<uint32_t*>(rank_table), nodes, sizes + num_hops, L.caps[num_hops]);
+  APT_LAUNCH_CHECK("mb_reset_kernel");
+  return APT_OK;
+}

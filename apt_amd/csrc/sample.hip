@@ -25,6 +25,7 @@ struct SampleParams {
   const int64_t* n_dev;
   int fanout;
   uint64_t seed;
+  const uint64_t* seed_dev;  // overrides seed when not NULL
   int hop;
   int64_t* out;
   int64_t* counts;
@@ -68,7 +69,36 @@ __device__ __forceinline__ void resolve_row(const apt_graph& g, int64_t v,
   nbrs = indices + s;
 }
 
+// Position inside its row that lane `l` of a group reads for output slot `l`
+// (fanout <= LPS), or -1 for an unused slot.  Every lane of the wave runs the
+// same instruction stream: rows whose degree fits in the fanout feed the
+// identity permutation through the Floyd resolution loop, which then never
+// finds a collision.
 template <int LPS, bool REPLACE>
+__device__ __forceinline__ int64_t slot_position(int l, int fanout, int64_t deg, int64_t node,
+                                                 uint64_t seed, int hop) {
+  const uint64_t r = draw64(seed, node, hop, static_cast<uint32_t>(l));
+  if (REPLACE) {
+    // reference :277-283: fanout independent draws when the row is not empty
+    return (l < fanout && deg > 0) ? static_cast<int64_t>(bounded(r, static_cast<uint64_t>(deg))) : -1;
+  }
+  // Floyd: slot i draws t in [0, j], j = deg - fanout + i, and takes t unless
+  // an earlier slot already holds t, then it takes j.
+  const bool big = deg > fanout;
+  const int64_t j = big ? deg - fanout + l : l;
+  int64_t tpos = -1 - l;  // lanes past the fanout never match a position
+  if (l < fanout) tpos = big ? static_cast<int64_t>(bounded(r, static_cast<uint64_t>(j + 1))) : l;
+  bool coll = false;
+  for (int q = 0; q + 1 < fanout; ++q) {
+    const int64_t pq = __shfl(coll ? j : tpos, q, LPS);
+    if (l > q && tpos == pq) coll = true;
+  }
+  const int64_t pick = coll ? j : tpos;
+  const int64_t cnt = big ? fanout : deg;
+  return l < cnt ? pick : -1;
+}
+
+template <int LPS, bool REPLACE, int U>
 __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   constexpr int G = kSampleBlock / LPS;  // lane groups per block
   constexpr int kMaxTile = G * kMaxRowsPerGroup;
@@ -82,10 +112,12 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   const int tile = G * p.rows_per_group;
   const int64_t tile_base = static_cast<int64_t>(blockIdx.x) * tile;
   if (tile_base >= n) return;  // block-uniform
+  const uint64_t seed = p.seed_dev != nullptr ? *p.seed_dev : p.seed;
 
   const int tid = threadIdx.x;
   if (tid == 0) s_total = 0;
-  // Stage 1: one lane per row of the tile.
+  // Stage 1: one lane per row of the tile, so the dependent
+  // frontier -> (pos_map ->) indptr loads of the whole tile overlap.
   for (int t = tid; t < tile; t += kSampleBlock) {
     const int64_t gi = tile_base + t;
     const int64_t* nbrs = nullptr;
@@ -105,64 +137,92 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   const int l = tid % LPS;
   const int fanout = p.fanout;
   int64_t my_total = 0;
-  for (int s = 0; s < p.rows_per_group; ++s) {
-    const int t = s * G + grp;
-    const int64_t gi = tile_base + t;
-    if (gi >= n) break;  // group-uniform
-    const int64_t* nbrs = s_nbrs[t];
-    const int64_t deg = s_deg[t];
-    const int64_t node = s_node[t];
-    int64_t* o = p.out + gi * fanout;
-    int64_t cnt;
-    if (REPLACE) {
-      // reference :277-283
-      for (int i = l; i < fanout; i += LPS) {
-        int64_t val = -1;
-        if (deg > 0)
-          val = nbrs[bounded(draw64(p.seed, node, p.hop, static_cast<uint32_t>(i)),
-                             static_cast<uint64_t>(deg))];
-        o[i] = val;
+  if (fanout <= LPS) {
+    // U rows per group in flight: positions first, then the loads, then the
+    // stores.
+    for (int s0 = 0; s0 < p.rows_per_group; s0 += U) {
+      const int64_t* src[U];
+      int64_t pos[U];
+      int64_t gis[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = (s0 + u) * G + grp;
+        gis[u] = (s0 + u) < p.rows_per_group ? tile_base + t : n;
+        pos[u] = -1;
+        src[u] = nullptr;
+        if (gis[u] < n) {
+          const int64_t deg = s_deg[t];
+          src[u] = s_nbrs[t];
+          pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, s_node[t], seed, p.hop);
+          if (l == 0) {
+            const int64_t cnt = REPLACE ? (deg > 0 ? fanout : 0) : (deg < fanout ? deg : fanout);
+            if (p.counts != nullptr) p.counts[gis[u]] = cnt;
+            my_total += cnt;
+          }
+        }
       }
-      cnt = deg > 0 ? fanout : 0;
-    } else if (deg <= fanout) {
-      for (int i = l; i < fanout; i += LPS) o[i] = i < deg ? nbrs[i] : -1;
-      cnt = deg;
-    } else {
-      // Floyd: slot i draws t in [0, j], j = deg - fanout + i, and takes t
-      // unless an earlier slot already holds t, then it takes j.
-      int64_t* picks = s_picks + static_cast<size_t>(grp) * fanout;
-      for (int c0 = 0; c0 < fanout; c0 += LPS) {
-        const int i = c0 + l;
-        const bool active = i < fanout;
-        const int64_t j = deg - fanout + i;
-        int64_t tpos = -1 - l;  // inactive lanes never match a position
-        if (active)
-          tpos = static_cast<int64_t>(
-              bounded(draw64(p.seed, node, p.hop, static_cast<uint32_t>(i)),
-                      static_cast<uint64_t>(j + 1)));
-        bool coll = false;
-        if (LPS == kWave && c0 > 0) {
+      int64_t val[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) val[u] = pos[u] >= 0 ? src[u][pos[u]] : -1;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (gis[u] < n && l < fanout) p.out[gis[u] * fanout + l] = val[u];
+    }
+  } else {
+    // fanout wider than a group: slots are resolved LPS at a time and earlier
+    // chunks' picks are kept in LDS (whole-wave groups only).
+    for (int s = 0; s < p.rows_per_group; ++s) {
+      const int t = s * G + grp;
+      const int64_t gi = tile_base + t;
+      if (gi >= n) break;  // group-uniform
+      const int64_t* nbrs = s_nbrs[t];
+      const int64_t deg = s_deg[t];
+      const int64_t node = s_node[t];
+      int64_t* o = p.out + gi * fanout;
+      int64_t cnt;
+      if (REPLACE) {
+        for (int i = l; i < fanout; i += LPS) {
+          int64_t val = -1;
+          if (deg > 0)
+            val = nbrs[bounded(draw64(seed, node, p.hop, static_cast<uint32_t>(i)),
+                               static_cast<uint64_t>(deg))];
+          o[i] = val;
+        }
+        cnt = deg > 0 ? fanout : 0;
+      } else if (deg <= fanout) {
+        for (int i = l; i < fanout; i += LPS) o[i] = i < deg ? nbrs[i] : -1;
+        cnt = deg;
+      } else {
+        int64_t* picks = s_picks + static_cast<size_t>(grp) * fanout;
+        for (int c0 = 0; c0 < fanout; c0 += LPS) {
+          const int i = c0 + l;
+          const bool active = i < fanout;
+          const int64_t j = deg - fanout + i;
+          int64_t tpos = -1 - l;
+          if (active)
+            tpos = static_cast<int64_t>(bounded(draw64(seed, node, p.hop, static_cast<uint32_t>(i)),
+                                                static_cast<uint64_t>(j + 1)));
+          bool coll = false;
           for (int q = 0; q < c0; ++q) coll |= (picks[q] == tpos);
-        }
-        const int len = min(LPS, fanout - c0);
-        for (int q = 0; q + 1 < len; ++q) {
-          const int64_t mine = coll ? j : tpos;
-          const int64_t pq = __shfl(mine, q, LPS);
-          if (l > q && tpos == pq) coll = true;
-        }
-        const int64_t pick = coll ? j : tpos;
-        if (active) o[i] = nbrs[pick];
-        if (LPS == kWave && fanout > LPS) {
-          if (active) picks[i] = pick;
+          const int len = min(LPS, fanout - c0);
+          for (int q = 0; q + 1 < len; ++q) {
+            const int64_t pq = __shfl(coll ? j : tpos, q, LPS);
+            if (l > q && tpos == pq) coll = true;
+          }
+          const int64_t pick = coll ? j : tpos;
+          if (active) {
+            o[i] = nbrs[pick];
+            picks[i] = pick;
+          }
           __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
           __builtin_amdgcn_wave_barrier();
         }
+        cnt = fanout;
       }
-      cnt = fanout;
-    }
-    if (l == 0) {
-      if (p.counts != nullptr) p.counts[gi] = cnt;
-      my_total += cnt;
+      if (l == 0) {
+        if (p.counts != nullptr) p.counts[gi] = cnt;
+        my_total += cnt;
+      }
     }
   }
   if (p.total != nullptr) {
@@ -175,14 +235,17 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
 }
 
 template <int LPS>
-static int launch_sample(const SampleParams& p, bool replace, int64_t blocks,
-                         size_t dyn_lds, hipStream_t st) {
-  if (replace)
-    hipLaunchKernelGGL((sample_kernel<LPS, true>), dim3(static_cast<unsigned>(blocks)),
-                       dim3(kSampleBlock), dyn_lds, st, p);
-  else
-    hipLaunchKernelGGL((sample_kernel<LPS, false>), dim3(static_cast<unsigned>(blocks)),
-                       dim3(kSampleBlock), dyn_lds, st, p);
+static int launch_sample(const SampleParams& p, bool replace, int64_t blocks, size_t dyn_lds,
+                         hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>(blocks)), block(kSampleBlock);
+  const bool wide = p.rows_per_group >= 4;
+  if (replace) {
+    if (wide) hipLaunchKernelGGL((sample_kernel<LPS, true, 4>), grid, block, dyn_lds, st, p);
+    else hipLaunchKernelGGL((sample_kernel<LPS, true, 1>), grid, block, dyn_lds, st, p);
+  } else {
+    if (wide) hipLaunchKernelGGL((sample_kernel<LPS, false, 4>), grid, block, dyn_lds, st, p);
+    else hipLaunchKernelGGL((sample_kernel<LPS, false, 1>), grid, block, dyn_lds, st, p);
+  }
   APT_LAUNCH_CHECK("sample_kernel");
   return APT_OK;
 }
@@ -191,35 +254,33 @@ int tuning_sample_lanes();  // 0 = automatic
 
 }  // namespace apt
 
-extern "C" int apt_sample_neighbors(const apt_graph* graph, const int64_t* frontier,
-                                    int64_t num_frontier,
-                                    const int64_t* num_frontier_dev, int fanout,
-                                    int replace, uint64_t rng_seed, int hop,
-                                    int64_t* out_neighbors, int64_t* out_counts,
-                                    int64_t* out_total, void* stream) {
-  using namespace apt;
-  APT_REQUIRE(graph != nullptr, APT_EINVAL, "apt_sample_neighbors: graph is NULL");
-  APT_REQUIRE(num_frontier >= 0, APT_EINVAL,
-              "apt_sample_neighbors: num_frontier %lld < 0", (long long)num_frontier);
-  APT_REQUIRE(fanout > 0, APT_EINVAL, "apt_sample_neighbors: fanout %d must be > 0", fanout);
-  APT_REQUIRE(fanout <= kMaxFanout, APT_ELIMIT,
-              "apt_sample_neighbors: fanout %d exceeds the supported maximum %d", fanout,
-              kMaxFanout);
+namespace apt {
+
+// Shared by apt_sample_neighbors and the fused mini-batch driver.
+int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
+                  const int64_t* num_frontier_dev, int fanout, int replace, uint64_t rng_seed,
+                  const uint64_t* rng_seed_dev, int hop, int64_t* out_neighbors, int64_t* out_counts,
+                  int64_t* out_total, hipStream_t st, const char* who) {
+  APT_REQUIRE(graph != nullptr, APT_EINVAL, "%s: graph is NULL", who);
+  APT_REQUIRE(num_frontier >= 0, APT_EINVAL, "%s: num_frontier %lld < 0", who, (long long)num_frontier);
+  APT_REQUIRE(fanout > 0, APT_EINVAL, "%s: fanout %d must be > 0", who, fanout);
+  APT_REQUIRE(fanout <= kMaxFanout, APT_ELIMIT, "%s: fanout %d exceeds the supported maximum %d", who,
+              fanout, kMaxFanout);
   APT_REQUIRE(graph->num_rows >= 0 && graph->indptr != nullptr &&
                   (graph->indices != nullptr || graph->num_rows == 0),
-              APT_EINVAL, "apt_sample_neighbors: graph has no indptr/indices");
+              APT_EINVAL, "%s: graph has no indptr/indices", who);
   if (graph->adj_pos_map != nullptr) {
     APT_REQUIRE(graph->num_total_nodes >= 0, APT_EINVAL,
-                "apt_sample_neighbors: adj_pos_map given but num_total_nodes < 0");
+                "%s: adj_pos_map given but num_total_nodes < 0", who);
     APT_REQUIRE(graph->num_cached_rows == 0 ||
                     (graph->cached_indptr != nullptr && graph->cached_indices != nullptr),
-                APT_EINVAL, "apt_sample_neighbors: cached rows without cached tables");
+                APT_EINVAL, "%s: cached rows without cached tables", who);
   }
   if (num_frontier == 0) return APT_OK;
   APT_REQUIRE(frontier != nullptr && out_neighbors != nullptr, APT_EINVAL,
-              "apt_sample_neighbors: frontier/out_neighbors is NULL");
+              "%s: frontier/out_neighbors is NULL", who);
   APT_REQUIRE(num_frontier <= (INT64_MAX / 8) / fanout, APT_ELIMIT,
-              "apt_sample_neighbors: num_frontier * fanout overflows");
+              "%s: num_frontier * fanout overflows", who);
 
   SampleParams p;
   p.g = *graph;
@@ -228,34 +289,49 @@ extern "C" int apt_sample_neighbors(const apt_graph* graph, const int64_t* front
   p.n_dev = num_frontier_dev;
   p.fanout = fanout;
   p.seed = rng_seed;
+  p.seed_dev = rng_seed_dev;
   p.hop = hop;
   p.out = out_neighbors;
   p.counts = out_counts;
   p.total = out_total;
 
+  // Lanes per frontier row: the smallest power of two that holds the fanout
+  // (8..64).  One whole wavefront per row leaves most lanes idle at the usual
+  // fanouts (5..25) and costs more workgroups for the same rows.
   int lps = tuning_sample_lanes();
-  if (lps == 0) lps = kWave;  // one wavefront per frontier row
-  if (lps != 8 && lps != 16 && lps != 32 && lps != 64) lps = kWave;
+  if (lps != 8 && lps != 16 && lps != 32 && lps != 64) {
+    lps = 8;
+    while (lps < fanout && lps < kWave) lps <<= 1;
+  }
   if (!replace && fanout > lps) lps = kWave;  // chunked Floyd needs whole waves
   const int groups = kSampleBlock / lps;
-  // Enough blocks to cover 256 CUs several times over before rows are
+  // Enough workgroups to cover 256 CUs several times over before rows are
   // serialised inside a group.
-  int64_t rpg = num_frontier / (static_cast<int64_t>(groups) * 4096);
+  int64_t rpg = num_frontier / (static_cast<int64_t>(groups) * 2048);
   if (rpg < 1) rpg = 1;
   if (rpg > kMaxRowsPerGroup) rpg = kMaxRowsPerGroup;
   p.rows_per_group = static_cast<int>(rpg);
   const int64_t tile = static_cast<int64_t>(groups) * rpg;
   const int64_t blocks = ceil_div(num_frontier, tile);
-  APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT,
-              "apt_sample_neighbors: %lld rows need too many workgroups",
+  APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT, "%s: %lld rows need too many workgroups", who,
               (long long)num_frontier);
-  const size_t dyn =
-      (!replace && fanout > lps) ? sizeof(int64_t) * groups * (size_t)fanout : 0;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+  const size_t dyn = (!replace && fanout > lps) ? sizeof(int64_t) * groups * (size_t)fanout : 0;
   switch (lps) {
     case 8: return launch_sample<8>(p, replace != 0, blocks, dyn, st);
     case 16: return launch_sample<16>(p, replace != 0, blocks, dyn, st);
     case 32: return launch_sample<32>(p, replace != 0, blocks, dyn, st);
     default: return launch_sample<64>(p, replace != 0, blocks, dyn, st);
   }
+}
+
+}  // namespace apt
+
+extern "C" int apt_sample_neighbors(const apt_graph* graph, const int64_t* frontier,
+                                    int64_t num_frontier, const int64_t* num_frontier_dev,
+                                    int fanout, int replace, uint64_t rng_seed, int hop,
+                                    int64_t* out_neighbors, int64_t* out_counts,
+                                    int64_t* out_total, void* stream) {
+  return apt::sample_launch(graph, frontier, num_frontier, num_frontier_dev, fanout, replace,
+                            rng_seed, nullptr, hop, out_neighbors, out_counts, out_total,
+                            static_cast<hipStream_t>(stream), "apt_sample_neighbors");
 }

@@ -6,6 +6,14 @@ the unique count back on every hop.  Here every buffer is allocated once at its
 upper bound (hop h holds at most B * prod(1 + f_i) frontier rows), the counts
 stay in device memory and are read by the next kernel, and the host waits once
 per batch, when it wants the sizes.
+
+Two drivers give identical results:
+  fused=True   apt_minibatch_sample: one C call per batch, node-indexed rank
+               table for relabel (default);
+  fused=False  apt_sample_neighbors + apt_relabel per hop (hash-table relabel).
+With use_graph=True the fused batch (and the gather) is captured once into a
+HIP graph and replayed; seeds and the rng seed are read from fixed device
+buffers that are refreshed before each replay.
 """
 import torch
 
@@ -13,38 +21,53 @@ from . import capi
 
 
 class MiniBatchPipeline:
-    def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True):
+    def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
+                 use_graph=False):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
         --fan_out list reversed)."""
         self.graph, self.feat = graph, feat
         self.fanouts = [int(f) for f in hop_fanouts]
         self.replace = bool(replace)
+        self.fused = bool(fused)
         dev = graph.device
         self.device = dev
-        self.caps = [int(batch_size)]
-        for f in self.fanouts:
-            self.caps.append(self.caps[-1] * (1 + f))
+        H = len(self.fanouts)
         i64 = dict(dtype=torch.int64, device=dev)
-        self.neighbors = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
-        self.relabeled = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
-        self.counts = [torch.empty(self.caps[h], **i64) for h in range(len(self.fanouts))]
-        self.frontier = [None] + [torch.empty(self.caps[h + 1], **i64) for h in range(len(self.fanouts))]
-        # sizes[h] = rows of the frontier entering hop h; sizes[-1] = input nodes; then edge total
-        self.sizes = torch.zeros(len(self.fanouts) + 2, **i64)
-        self.workspace = torch.empty(capi.relabel_workspace_bytes(self.caps[-1]), dtype=torch.uint8,
-                                     device=dev)
+        if self.fused:
+            self.plan = capi.MinibatchPlan(graph, batch_size, self.fanouts, replace=replace)
+            self.caps = self.plan.caps
+            self.sizes = self.plan.sizes
+            self.neighbors, self.relabeled, self.counts = (self.plan.neighbors, self.plan.relabeled,
+                                                           self.plan.counts)
+            self.nodes = self.plan.nodes
+        else:
+            self.caps = [int(batch_size)]
+            for f in self.fanouts:
+                self.caps.append(self.caps[-1] * (1 + f))
+            self.neighbors = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
+            self.relabeled = [torch.empty(self.caps[h] * f, **i64) for h, f in enumerate(self.fanouts)]
+            self.counts = [torch.empty(self.caps[h], **i64) for h in range(H)]
+            self.frontier = [None] + [torch.empty(self.caps[h + 1], **i64) for h in range(H)]
+            # sizes[h] = rows of the frontier entering hop h; sizes[H] = input nodes; then edges
+            self.sizes = torch.zeros(H + 2, **i64)
+            self.workspace = torch.empty(capi.relabel_workspace_bytes(self.caps[-1]), dtype=torch.uint8,
+                                         device=dev)
         self.features = None
         if gather and feat is not None:
             self.features = torch.empty((self.caps[-1], feat.out_dim), dtype=feat.dtype, device=dev)
         self.misses = torch.zeros(1, **i64)
+        self.seeds = None
+        self.graph_exec = None
+        if use_graph:
+            if not self.fused:
+                raise ValueError("graph replay needs the fused driver")
+            self._capture()
 
+    # ------------------------------------------------------------ unfused
     def _size(self, h):
         return self.sizes[h:h + 1]
 
-    def sample(self, seeds, rng_seed):
-        """Sampling + relabel for every hop, asynchronous."""
-        if seeds.numel() != self.caps[0]:
-            raise ValueError(f"expected {self.caps[0]} seeds, got {seeds.numel()}")
+    def _sample_unfused(self, seeds, rng_seed):
         self.frontier[0] = seeds
         self.sizes.zero_()
         self.sizes[0:1].fill_(seeds.numel())
@@ -58,13 +81,46 @@ class MiniBatchPipeline:
                          unique=self.frontier[h + 1], relabeled=self.relabeled[h],
                          num_unique_dev=self._size(h + 1), workspace=self.workspace, sync=False)
 
+    # ------------------------------------------------------------ graph
+    def _capture(self):
+        self.static_seeds = torch.zeros(self.caps[0], dtype=torch.int64, device=self.device)
+        # run once eagerly so lazy initialisation happens outside the capture
+        self.plan.launch(self.static_seeds, rng_seed=None)
+        if self.features is not None:
+            self.gather()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.plan.launch(self.static_seeds, rng_seed=None)
+            if self.features is not None:
+                self.gather()
+        self.graph_exec = g
+
+    # ------------------------------------------------------------ public
+    def sample(self, seeds, rng_seed):
+        """Sampling + relabel for every hop, asynchronous."""
+        if seeds.numel() != self.caps[0]:
+            raise ValueError(f"expected {self.caps[0]} seeds, got {seeds.numel()}")
+        self.seeds = seeds
+        if self.fused:
+            self.plan.launch(seeds, rng_seed)
+        else:
+            self._sample_unfused(seeds, rng_seed)
+
     def gather(self):
         """Features of the input nodes (the last hop's unique ids), asynchronous."""
         H = len(self.fanouts)
-        capi.gather_rows(self.feat, self.frontier[H], num_index_dev=self._size(H), out=self.features,
+        index = self.nodes if self.fused else self.frontier[H]
+        capi.gather_rows(self.feat, index, num_index_dev=self._size(H), out=self.features,
                          miss_count=self.misses)
 
     def run(self, seeds, rng_seed):
+        if self.graph_exec is not None:
+            self.static_seeds.copy_(seeds)
+            self.plan.rng_seed_dev.fill_(int(rng_seed) & 0x7FFFFFFFFFFFFFFF)
+            self.seeds = self.static_seeds
+            self.graph_exec.replay()
+            return
         self.sample(seeds, rng_seed)
         if self.features is not None:
             self.gather()
@@ -77,9 +133,15 @@ class MiniBatchPipeline:
         blocks = []
         for h, f in enumerate(self.fanouts):
             n = sizes[h]
-            blocks.insert(0, dict(seeds=self.frontier[h][:n], neighbors=self.neighbors[h][:n * f],
+            if self.fused:
+                src = self.seeds if h == 0 else self.nodes[:n]
+                uniq = self.nodes[:sizes[h + 1]]
+            else:
+                src, uniq = self.frontier[h][:n], self.frontier[h + 1][:sizes[h + 1]]
+            blocks.insert(0, dict(seeds=src, neighbors=self.neighbors[h][:n * f],
                                   relabeled=self.relabeled[h][:n * f], counts=self.counts[h][:n],
-                                  unique=self.frontier[h + 1][:sizes[h + 1]], fanout=f))
+                                  unique=uniq, fanout=f))
         feats = None if self.features is None else self.features[:sizes[H]]
-        return dict(input_nodes=self.frontier[H][:sizes[H]], blocks=blocks, features=feats,
-                    num_edges=sizes[-1], sizes=sizes[:-1])
+        inp = self.nodes[:sizes[H]] if self.fused else self.frontier[H][:sizes[H]]
+        return dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],
+                    sizes=sizes[:-1])

@@ -36,6 +36,7 @@ extern "C" {
 #define APT_EWORKSPACE (-3) /* workspace too small */
 #define APT_EHIP (-4)    /* a HIP runtime call failed */
 
+#define APT_MAX_HOPS 8
 #define APT_MAX_BUCKETS 64 /* reference: MAX_NUM_DEVICES 33 (src/cuda/npc_kernel.h:13) */
 
 const char* apt_last_error(void);
@@ -218,6 +219,49 @@ int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* feat_pos_map,
                      int64_t* bucket_offset, int64_t* sorted_ids,
                      int64_t* permutation, void* workspace,
                      size_t workspace_bytes, void* stream);
+
+/* Whole multi-hop mini-batch in one call: for every hop, sample the current
+ * frontier, relabel, and make the unique node list the next frontier.
+ * Replaces the DP branch of MixedPSNeighborSampler.sample
+ * (python/npc/sampler.py:187-203,358-364) with its per-hop
+ * local_sample_one_layer + relabel_csc calls; results are identical to calling
+ * apt_sample_neighbors (hop index = position in hop_fanouts) and apt_relabel
+ * hop by hop.  Nothing is read back to the host.
+ *
+ *   hop_fanouts     host int[num_hops], from the seeds outward (the reference's
+ *                   --fan_out list reversed, python/npc/sampler.py:191)
+ *   rng_seed_dev    optional device uint64[1] overriding rng_seed (lets a
+ *                   captured HIP graph be replayed with a new seed)
+ *   rank_table      device uint32[rank_table_len], rank_table_len >= every node
+ *                   id of the graph; apt_rank_table_bytes / apt_rank_table_init
+ *                   size and initialise it once, every call leaves it
+ *                   initialised again.  A node id outside [0, rank_table_len)
+ *                   is treated like padding (no edge, not in the node list).
+ *   nodes           device int64[capacity(num_hops)]: the unique node list;
+ *                   its first sizes[h] entries are the frontier of hop h and
+ *                   the source nodes of hop h-1's block, its first
+ *                   sizes[num_hops] entries the input nodes of the batch
+ *   neighbors[h], relabeled[h]   host arrays of device int64[capacity(h) *
+ *                   hop_fanouts[h]]: sampled ids (-1 padded) and their compact
+ *                   ids (= index into nodes)
+ *   counts[h]       optional (counts or counts[h] may be NULL) device
+ *                   int64[capacity(h)]
+ *   sizes           device int64[num_hops + 2]: sizes[h] = frontier rows
+ *                   entering hop h (sizes[0] = batch), sizes[num_hops] = input
+ *                   nodes, sizes[num_hops + 1] = sampled edges of the batch
+ *   capacity(h)     apt_minibatch_capacity: batch * prod_{i<h}(1 + fanout_i)
+ */
+size_t apt_rank_table_bytes(int64_t num_total_nodes);
+int apt_rank_table_init(void* table, size_t table_bytes, void* stream);
+size_t apt_minibatch_workspace_bytes(int64_t batch, const int* hop_fanouts, int num_hops);
+int64_t apt_minibatch_capacity(int64_t batch, const int* hop_fanouts, int num_hops, int hop);
+int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                         const int* hop_fanouts, int num_hops, int replace,
+                         uint64_t rng_seed, const uint64_t* rng_seed_dev,
+                         void* rank_table, int64_t rank_table_len, int64_t* nodes,
+                         int64_t* const* neighbors, int64_t* const* relabeled,
+                         int64_t* const* counts, int64_t* sizes, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -19,18 +19,22 @@ def _setup(orc, capi, n=30000, deg=14, dim=100, seed=21):
     return indptr, indices, feats
 
 
+@pytest.mark.parametrize("mode", ["fused", "graph", "unfused"])
 @pytest.mark.parametrize("replace", [False, True])
-def test_pipeline_matches_oracle_driver(orc, capi, replace):
+def test_pipeline_matches_oracle_driver(orc, capi, replace, mode):
     from apt_amd.pipeline import MiniBatchPipeline
     indptr, indices, feats = _setup(orc, capi)
     og = orc.Graph(indptr, indices)
     dg = capi.Graph(dev(indptr), dev(indices))
     fs = capi.FeatStore(dev(feats))
     hops = [5, 10, 15]
-    pipe = MiniBatchPipeline(dg, fs, 512, hops, replace=replace)
+    pipe = MiniBatchPipeline(dg, fs, 512, hops, replace=replace, fused=mode != "unfused",
+                             use_graph=mode == "graph")
     rng = np.random.default_rng(0)
-    for batch in range(3):                                   # buffers are reused across batches
+    for batch in range(4):                                   # buffers (and the graph) are reused
         seeds = rng.permutation(len(indptr) - 1)[:512]
+        if batch == 2:
+            seeds[100:200] = seeds[0:100]                    # repeated seeds are legal
         pipe.run(dev(seeds), 1000 + batch)
         res = pipe.result()
         want_in, want_blocks = orc.sample_blocks(og, seeds, hops, replace, 1000 + batch)
@@ -43,7 +47,29 @@ def test_pipeline_matches_oracle_driver(orc, capi, replace):
         assert miss == 0 and int(pipe.misses.item()) == 0
         assert np.array_equal(res["features"].cpu().numpy(), want_f)
         # structure (reference sampler.py:358-364): dst nodes are a prefix of src nodes
-        assert np.array_equal(want_in[:512], seeds)
+        if batch != 2:
+            assert np.array_equal(want_in[:512], seeds)
+        if mode != "unfused":                                # the rank table is clean again
+            assert bool((pipe.plan.table.view(torch.int32) == -1).all())
+
+
+def test_fused_driver_edge_cases(orc, capi):
+    from apt_amd.pipeline import MiniBatchPipeline
+    from helpers import special_graph
+    indptr, indices, degs = special_graph()
+    og = orc.Graph(indptr, indices)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    for hops, replace in [([5], False), ([16, 3], False), ([2, 2, 2, 2], True), ([64], False)]:
+        seeds = np.array([0, 1, 2, 3, 4, 5, 6, 6, 7, 8, 9, 10, 11, 5, -1, 3])
+        pipe = MiniBatchPipeline(dg, None, len(seeds), hops, replace=replace, gather=False)
+        pipe.run(dev(seeds), 77)
+        res = pipe.result()
+        want_in, want_blocks = orc.sample_blocks(og, seeds, hops, replace, 77)
+        assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+        for got, want in zip(res["blocks"], want_blocks):
+            for k in ("neighbors", "relabeled", "counts", "unique"):
+                assert np.array_equal(got[k].cpu().numpy(), want[k]), (hops, k)
+        assert bool((pipe.plan.table.view(torch.int32) == -1).all())
 
 
 def test_operator_layer_dp_sampler(orc, capi):
