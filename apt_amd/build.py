@@ -11,6 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libapt_hip.so")
+NPC_LIB = os.path.join(HERE, "libnpc.so")
 SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "minibatch.hip", "synth.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -54,7 +55,27 @@ def build(force=True, verbose=False):
             print(text, file=sys.stderr)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     subprocess.check_call(cmd)
+    build_torch_binding(verbose=verbose)
     return LIB
+
+
+def build_torch_binding(verbose=False):
+    """Compile libnpc.so: TORCH_LIBRARY(npc) over the C ABI (host code only)."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           os.path.join(CSRC, "torch_bind.cc"), "-o", NPC_LIB,
+           *[f"-I{p}" for p in ce.include_paths()], "-I/opt/rocm/include",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-L{tlib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           f"-L{HERE}", "-lapt_hip", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"]
+    if verbose:
+        print(" ".join(cmd), file=sys.stderr)
+    subprocess.check_call(cmd)
+    return NPC_LIB
 
 
 if __name__ == "__main__":

@@ -14,6 +14,7 @@
 namespace apt {
 
 constexpr int kGatherBlock = 256;
+constexpr int kGatherPersistentBlocks = 16384;
 
 struct GatherParams {
   const char* local_table;
@@ -116,15 +117,21 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
               static_cast<unsigned long long>(misses));
 }
 
-int tuning_gather_rows();  // 0 = default
+int tuning_gather_rows();        // 0 = default
+int tuning_gather_max_blocks();  // 0 = default
 
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int R = tuning_gather_rows();
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = 4;
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
   const int groups = kGatherBlock / LPR;
+  // With a device-side count the host size is only an upper bound: a capped
+  // grid that strides over the rows avoids dispatching workgroups that would
+  // find nothing to do.
+  int64_t max_blocks = tuning_gather_max_blocks();
+  if (max_blocks <= 0) max_blocks = p.n_dev != nullptr ? kGatherPersistentBlocks : (1 << 20);
   int64_t blocks = ceil_div(p.n, static_cast<int64_t>(groups) * R);
-  if (blocks > (1 << 20)) blocks = 1 << 20;
+  if (blocks > max_blocks) blocks = max_blocks;
   const dim3 grid(static_cast<unsigned>(blocks)), block(kGatherBlock);
   switch (R) {
     case 1: hipLaunchKernelGGL((gather_kernel<V, LPR, 1>), grid, block, 0, st, p); break;

@@ -13,9 +13,11 @@ char* last_error_buf() {
 
 static int g_sample_lanes = 0;
 static int g_gather_rows = 0;
+static int g_gather_max_blocks = 0;
 
 int tuning_sample_lanes() { return g_sample_lanes; }
 int tuning_gather_rows() { return g_gather_rows; }
+int tuning_gather_max_blocks() { return g_gather_max_blocks; }
 
 }  // namespace apt
 
@@ -35,6 +37,11 @@ extern "C" int apt_set_tuning(const char* key, int value) {
     if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
       return apt::fail(APT_EINVAL, "apt_set_tuning: gather_rows_in_flight must be 0, 1, 2, 4 or 8");
     apt::g_gather_rows = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "gather_max_blocks") == 0) {
+    if (value < 0) return apt::fail(APT_EINVAL, "apt_set_tuning: gather_max_blocks must be >= 0");
+    apt::g_gather_max_blocks = value;
     return APT_OK;
   }
   return apt::fail(APT_EINVAL, "apt_set_tuning: unknown key '%s'", key);

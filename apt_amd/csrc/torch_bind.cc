@@ -1,0 +1,411 @@
+// libnpc.so: the `npc` operator library for PyTorch-ROCm.
+//
+// Registers the hot-path operators under the names and C++ signatures the
+// reference binds with TORCH_LIBRARY(npc, m) in src/pybind.cc:18-48, so that
+// torch.ops.npc.<name>(...) keeps working.  Every operator is a thin host
+// wrapper: it checks its tensors, allocates outputs with torch, and calls the
+// C ABI of libapt_hip.so (include/apt_amd.h) on the current HIP stream.
+// Operators whose reference implementation exchanges data with other GPUs
+// over NCCL are registered too, and raise.
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+#include <torch/torch.h>
+
+#include <tuple>
+#include <vector>
+
+#include "../../include/apt_amd.h"
+
+namespace npc {
+
+using torch::Tensor;
+using IdType = int64_t;  // reference src/utils.h:14
+
+namespace {
+
+struct State {  // counterpart of NPCState, reference src/state.h:32-63
+  int64_t rank = 0, local_rank = 0, world_size = 1, node_size = 1;
+  // graph (reference GraphStorage, state.h:18-23)
+  bool has_graph = false;
+  Tensor indptr, indices, cached_indptr, cached_indices, adj_pos_map;
+  apt_graph graph{};
+  // features (reference FeatStorage, state.h:10-16)
+  bool has_feat = false;
+  Tensor local_feats, cache_feats, feat_pos_map, cpu_feat_pos_map;
+  bool identity_map = false;
+  apt_feat_store feat{};
+  // bucketing
+  Tensor shuffle_min_vids, remote_worker_map;
+  int64_t shuffle_id_offset = 0, num_remote_workers = 0;
+  // sampling
+  uint64_t rng_seed = 7777777;  // reference src/cuda/npc_kernel.cu:292
+  int64_t sample_calls = 0;
+  bool strict = true;
+};
+
+State& S() {
+  static State s;
+  return s;
+}
+
+void check(int status) {
+  TORCH_CHECK(status == APT_OK, "npc: ", apt_last_error(), " (status ", status, ")");
+}
+
+void* stream() { return static_cast<void*>(c10::hip::getCurrentHIPStream().stream()); }
+
+c10::Device device() {
+  TORCH_CHECK(torch::cuda::is_available(), "npc: no GPU; the operators have no CPU implementation");
+  return c10::Device(c10::kCUDA, c10::hip::current_device());
+}
+
+Tensor ids_on_device(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.scalar_type() == torch::kInt64, "npc: ", name, " must be int64");
+  TORCH_CHECK(t.dim() == 1, "npc: ", name, " must be 1-D");
+  return t.to(device()).contiguous();
+}
+
+const int64_t* i64(const Tensor& t) { return t.defined() && t.numel() ? t.data_ptr<int64_t>() : nullptr; }
+
+torch::TensorOptions i64_opts() { return torch::TensorOptions().dtype(torch::kInt64).device(device()); }
+
+}  // namespace
+
+// ---------------------------------------------------------------- registries
+void SetTopology(IdType rank, IdType world_size, IdType node_size) {
+  TORCH_CHECK(world_size >= 1 && world_size <= APT_MAX_BUCKETS && rank >= 0 && rank < world_size &&
+                  node_size >= 1,
+              "npc: bad topology");
+  S().rank = rank;
+  S().world_size = world_size;
+  S().node_size = node_size;
+  S().local_rank = rank % node_size;
+}
+
+void SetRngSeed(IdType seed) {
+  S().rng_seed = static_cast<uint64_t>(seed);
+  S().sample_calls = 0;
+}
+
+void SetStrict(bool strict) { S().strict = strict; }
+
+// reference src/cache_feats.cc:14-61
+void CacheFeatsShared(IdType num_total_nodes, Tensor localnode_feats, Tensor cached_feats,
+                      Tensor cached_idx, Tensor localnode_idx, IdType feat_dim_offset) {
+  auto& s = S();
+  TORCH_CHECK(localnode_feats.dim() == 2, "npc: localnode_feats must be [num_local, feat_dim]");
+  TORCH_CHECK(localnode_feats.element_size() == 2 || localnode_feats.element_size() == 4,
+              "npc: features must have 2- or 4-byte elements");
+  const int64_t n_local = localnode_feats.size(0), feat_dim = localnode_feats.size(1);
+  const int64_t n_cached = cached_feats.dim() == 2 ? cached_feats.size(0) : 0;
+  auto local_idx = ids_on_device(localnode_idx, "localnode_idx");
+  auto cache_idx = ids_on_device(cached_idx, "cached_idx");
+  TORCH_CHECK(local_idx.numel() == n_local, "npc: localnode_idx must name every local row");
+  TORCH_CHECK(cache_idx.numel() == n_cached, "npc: cached_idx must name every cached row");
+  if (n_local)
+    TORCH_CHECK(local_idx.min().item<int64_t>() >= 0 && local_idx.max().item<int64_t>() < num_total_nodes,
+                "npc: localnode_idx out of range");
+  if (n_cached)
+    TORCH_CHECK(cache_idx.min().item<int64_t>() >= 0 && cache_idx.max().item<int64_t>() < num_total_nodes,
+                "npc: cached_idx out of range");
+  const int64_t rank_dim = n_cached ? cached_feats.size(1) : feat_dim - feat_dim_offset;
+  TORCH_CHECK(feat_dim_offset >= 0 && feat_dim_offset + rank_dim <= feat_dim,
+              "npc: feat_dim_offset + cached width exceeds the local feature width");
+  s.local_feats = localnode_feats.to(device()).contiguous();
+  auto pos = torch::full({num_total_nodes}, -1, i64_opts());  // FEAT_NOT_EXIST, src/utils.h:20
+  pos.index_put_({local_idx}, -torch::arange(n_local, i64_opts()) - 2);  // ENCODE_ID, src/utils.h:17
+  s.cpu_feat_pos_map = pos.cpu();  // without cache entries, src/cache_feats.cc:52
+  s.cache_feats = Tensor();
+  if (n_cached) {
+    TORCH_CHECK(cached_feats.scalar_type() == localnode_feats.scalar_type(),
+                "npc: cached_feats dtype differs from localnode_feats");
+    s.cache_feats = cached_feats.to(device()).contiguous();
+    pos.index_put_({cache_idx}, torch::arange(n_cached, i64_opts()));  // the cache wins, :53-55
+  }
+  s.feat_pos_map = pos;
+  s.identity_map = n_cached == 0 && n_local == num_total_nodes &&
+                   torch::equal(local_idx, torch::arange(n_local, i64_opts()));
+  s.feat.local_table = s.local_feats.data_ptr();
+  s.feat.num_local_rows = n_local;
+  s.feat.local_dim = feat_dim;
+  s.feat.cache_table = n_cached ? s.cache_feats.data_ptr() : nullptr;
+  s.feat.num_cache_rows = n_cached;
+  s.feat.pos_map = s.identity_map ? nullptr : pos.data_ptr<int64_t>();
+  s.feat.num_total_nodes = num_total_nodes;
+  s.feat.col_offset = feat_dim_offset;
+  s.feat.out_dim = rank_dim;
+  s.feat.elem_size = static_cast<int>(localnode_feats.element_size());
+  s.has_feat = true;
+}
+
+// reference src/cache_graphs.cc:12-49
+void MixCacheGraphs(IdType num_cached_nodes, Tensor cached_node_idx, Tensor cached_indptr,
+                    Tensor cached_indices, Tensor global_indptr, Tensor global_indices) {
+  auto& s = S();
+  TORCH_CHECK(num_cached_nodes == cached_node_idx.numel(),
+              "npc: num_cached_nodes != cached_node_idx.numel()");  // reference CHECK :19
+  s.indptr = ids_on_device(global_indptr, "global_indptr");
+  s.indices = ids_on_device(global_indices, "global_indices");
+  const int64_t total = s.indptr.numel() - 1;
+  TORCH_CHECK(total >= 0, "npc: global_indptr is empty");
+  s.graph = apt_graph{};
+  s.graph.indptr = s.indptr.data_ptr<int64_t>();
+  s.graph.indices = i64(s.indices);
+  s.graph.row_begin = 0;
+  s.graph.num_rows = total;
+  s.graph.num_total_nodes = total;
+  s.adj_pos_map = Tensor();
+  if (num_cached_nodes > 0) {
+    auto idx = ids_on_device(cached_node_idx, "cached_node_idx");
+    s.cached_indptr = ids_on_device(cached_indptr, "cached_indptr");
+    s.cached_indices = ids_on_device(cached_indices, "cached_indices");
+    TORCH_CHECK(s.cached_indptr.numel() == num_cached_nodes + 1,
+                "npc: cached_indptr must have num_cached_nodes + 1 entries");
+    TORCH_CHECK(idx.min().item<int64_t>() >= 0 && idx.max().item<int64_t>() < total,
+                "npc: cached_node_idx out of range");
+    s.adj_pos_map = -torch::arange(total, i64_opts()) - 2;  // ENCODE_ID(v), :37-40
+    s.adj_pos_map.index_put_({idx}, torch::arange(num_cached_nodes, i64_opts()));
+    s.graph.cached_indptr = s.cached_indptr.data_ptr<int64_t>();
+    s.graph.cached_indices = i64(s.cached_indices);
+    s.graph.num_cached_rows = num_cached_nodes;
+    s.graph.adj_pos_map = s.adj_pos_map.data_ptr<int64_t>();
+  }
+  s.has_graph = true;
+}
+
+// A contiguous-range partition: nodes outside [row_begin, row_begin + rows)
+// have no adjacency.  No counterpart in the reference.
+void RegisterGraphPartition(Tensor indptr, Tensor indices, IdType row_begin, IdType num_total_nodes) {
+  auto& s = S();
+  s.indptr = ids_on_device(indptr, "indptr");
+  s.indices = ids_on_device(indices, "indices");
+  TORCH_CHECK(s.indptr.numel() >= 1, "npc: indptr is empty");
+  s.adj_pos_map = Tensor();
+  s.graph = apt_graph{};
+  s.graph.indptr = s.indptr.data_ptr<int64_t>();
+  s.graph.indices = i64(s.indices);
+  s.graph.row_begin = row_begin;
+  s.graph.num_rows = s.indptr.numel() - 1;
+  s.graph.num_total_nodes = num_total_nodes;
+  s.has_graph = true;
+}
+
+// reference src/core.cc:102-108
+void RegisterMinVids(Tensor shuffle_min_vids, IdType shuffle_id_offset) {
+  S().shuffle_min_vids = ids_on_device(shuffle_min_vids, "shuffle_min_vids");
+  S().shuffle_id_offset = shuffle_id_offset;
+}
+
+// reference src/core.cc:110-125 (state only)
+void RegisterMultiMachinesScheme(Tensor remote_worker_map, Tensor remote_worker_id) {
+  S().remote_worker_map = ids_on_device(remote_worker_map, "remote_worker_map");
+  S().num_remote_workers = remote_worker_id.numel();
+}
+
+// ---------------------------------------------------------------- hot path
+std::tuple<Tensor, Tensor> SampleNeighbors(Tensor seeds, IdType fanout, bool replace, IdType rng_seed,
+                                           IdType hop) {
+  auto& s = S();
+  TORCH_CHECK(s.has_graph, "npc: no graph registered (mix_cache_graphs)");
+  TORCH_CHECK(fanout > 0, "npc: fanout must be > 0");
+  auto f = ids_on_device(seeds, "seeds");
+  auto out = torch::empty({f.numel() * fanout}, i64_opts());
+  auto cnt = torch::empty({f.numel()}, i64_opts());
+  check(apt_sample_neighbors(&s.graph, i64(f), f.numel(), nullptr, static_cast<int>(fanout), replace,
+                             static_cast<uint64_t>(rng_seed), static_cast<int>(hop),
+                             out.data_ptr<int64_t>(), cnt.data_ptr<int64_t>(), nullptr, stream()));
+  return {out, cnt};
+}
+
+// reference src/sampling.cc:13-17
+std::vector<Tensor> LocalSamplingNeibhorsOneLayer(Tensor seeds, IdType fanout) {
+  auto& s = S();
+  TORCH_CHECK(s.has_graph, "npc: no graph registered (mix_cache_graphs)");
+  TORCH_CHECK(fanout > 0, "npc: fanout must be > 0");
+  auto f = ids_on_device(seeds, "seeds");
+  auto out = torch::empty({f.numel() * fanout}, i64_opts());
+  check(apt_sample_neighbors(&s.graph, i64(f), f.numel(), nullptr, static_cast<int>(fanout), 1,
+                             s.rng_seed, static_cast<int>(s.sample_calls), out.data_ptr<int64_t>(),
+                             nullptr, nullptr, stream()));
+  s.sample_calls += 1;
+  return {f, out};
+}
+
+// reference src/relabel.cc:9-15
+std::vector<Tensor> RelabelCSC(Tensor seeds, Tensor neighbors) {
+  auto sd = ids_on_device(seeds, "seeds");
+  auto nb = ids_on_device(neighbors, "neighbors");
+  const int64_t items = sd.numel() + nb.numel();
+  const size_t need = apt_relabel_workspace_bytes(items);
+  TORCH_CHECK(need > 0, "npc: relabel_csc: ", items, " items exceed the supported maximum");
+  auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
+  auto unique = torch::empty({items}, i64_opts());
+  auto relabeled = torch::empty({nb.numel()}, i64_opts());
+  auto count = torch::empty({1}, i64_opts());
+  int64_t host_count = -1;
+  check(apt_relabel(i64(sd), sd.numel(), nullptr, i64(nb), nb.numel(), 0, unique.data_ptr<int64_t>(),
+                    relabeled.data_ptr<int64_t>(), count.data_ptr<int64_t>(), &host_count,
+                    ws.data_ptr(), need, stream()));
+  return {unique.narrow(0, 0, host_count), relabeled};
+}
+
+// reference src/load_subtensor.cc:19-40
+Tensor LoadSubtensor(Tensor node_id) {
+  auto& s = S();
+  TORCH_CHECK(s.has_feat, "npc: no features registered (cache_feats_shared)");
+  auto idx = ids_on_device(node_id, "node_id");
+  auto out = torch::empty({idx.numel(), s.feat.out_dim}, s.local_feats.options());
+  Tensor miss;
+  if (s.strict) miss = torch::zeros({1}, i64_opts());
+  check(apt_gather_rows(&s.feat, i64(idx), idx.numel(), nullptr, out.data_ptr(),
+                        s.strict ? miss.data_ptr<int64_t>() : nullptr, stream()));
+  if (s.strict) {
+    const int64_t m = miss.item<int64_t>();
+    TORCH_CHECK_INDEX(m == 0, "npc: load_subtensor: ", m,
+                      " requested node(s) have no feature row on this GPU");
+  }
+  return out;
+}
+
+// reference src/load_subtensor.cc:10-17
+Tensor CPULoadSubtensor(Tensor node_id) {
+  auto& s = S();
+  TORCH_CHECK(s.has_feat, "npc: no features registered (cache_feats_shared)");
+  auto pos = -s.cpu_feat_pos_map.index_select(0, node_id.cpu()) - 2;
+  return s.local_feats.index_select(0, pos.to(s.local_feats.device()));
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> ClusterAndPermuteLocal(Tensor seeds) {
+  auto& s = S();
+  TORCH_CHECK(s.shuffle_min_vids.defined(), "npc: register_min_vids has not been called");
+  TORCH_CHECK(s.shuffle_min_vids.numel() >= s.world_size + 1, "npc: min_vids shorter than world_size + 1");
+  auto ids = ids_on_device(seeds, "seeds");
+  const int W = static_cast<int>(s.world_size);
+  const int node_beg = static_cast<int>(s.rank - (s.rank % s.node_size));  // src/sampling.cc:168-169
+  auto size = torch::empty({W}, i64_opts()), offset = torch::empty({W}, i64_opts());
+  auto sorted = torch::empty({ids.numel()}, i64_opts()), perm = torch::empty({ids.numel()}, i64_opts());
+  const size_t need = apt_bucket_workspace_bytes(ids.numel(), W);
+  TORCH_CHECK(need > 0, "npc: bucketing: unsupported size");
+  auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
+  check(apt_cluster_permute(i64(ids), ids.numel(), s.shuffle_min_vids.data_ptr<int64_t>(), W,
+                            s.shuffle_id_offset, static_cast<int>(s.rank), node_beg,
+                            node_beg + static_cast<int>(s.node_size), size.data_ptr<int64_t>(),
+                            offset.data_ptr<int64_t>(), sorted.data_ptr<int64_t>(),
+                            perm.data_ptr<int64_t>(), ws.data_ptr(), need, stream()));
+  return {size, offset, sorted, perm};
+}
+
+// reference src/sampling.cc:159-193; with one GPU both all-to-alls are identity copies
+std::tuple<Tensor, Tensor, Tensor, Tensor> ShuffleSeeds(Tensor seeds) {
+  TORCH_CHECK(S().world_size == 1,
+              "npc: shuffle_seeds exchanges ids between GPUs; only world_size 1 is available "
+              "(cluster_and_permute gives the local half)");
+  auto r = ClusterAndPermuteLocal(seeds);
+  auto off = std::get<1>(r).cpu();
+  return {std::get<2>(r), std::get<3>(r), off.clone(), off};
+}
+
+// reference src/load_subtensor.cc:83-86
+std::tuple<Tensor, Tensor, Tensor> ClusterReqs(Tensor node_id) {
+  auto& s = S();
+  TORCH_CHECK(s.has_feat && s.remote_worker_map.defined() && s.shuffle_min_vids.defined(),
+              "npc: cluster_reqs needs cache_feats_shared, register_min_vids and "
+              "register_multi_machines_scheme");
+  TORCH_CHECK(s.shuffle_min_vids.numel() >= s.world_size + 1 && s.remote_worker_map.numel() >= s.world_size,
+              "npc: min_vids / remote_worker_map shorter than world_size");
+  auto ids = ids_on_device(node_id, "node_id");
+  const int R = static_cast<int>(s.num_remote_workers);
+  auto size = torch::empty({R}, i64_opts());
+  auto sorted = torch::empty({ids.numel()}, i64_opts()), perm = torch::empty({ids.numel()}, i64_opts());
+  const size_t need = apt_bucket_workspace_bytes(ids.numel(), R);
+  TORCH_CHECK(need > 0, "npc: bucketing: unsupported size");
+  auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
+  check(apt_cluster_reqs(i64(ids), ids.numel(), s.feat_pos_map.data_ptr<int64_t>(),
+                         s.feat_pos_map.numel(), s.remote_worker_map.data_ptr<int64_t>(),
+                         s.shuffle_min_vids.data_ptr<int64_t>(), static_cast<int>(s.world_size), R,
+                         size.data_ptr<int64_t>(), nullptr, sorted.data_ptr<int64_t>(),
+                         perm.data_ptr<int64_t>(), ws.data_ptr(), need, stream()));
+  return {size, sorted, perm};
+}
+
+// reference src/feat_shuffle.cc:9-30 with one GPU
+Tensor FeatShuffle(Tensor inputs, Tensor send_offset, Tensor recv_offset, Tensor permutation,
+                   IdType feat_dim, IdType fwd_flag) {
+  TORCH_CHECK(S().world_size == 1,
+              "npc: feat_shuffle exchanges rows between GPUs; only world_size 1 is available");
+  TORCH_CHECK(inputs.is_cuda() && (inputs.element_size() == 2 || inputs.element_size() == 4),
+              "npc: feat_shuffle needs a GPU tensor with 2- or 4-byte elements");
+  auto x = inputs.reshape({-1, feat_dim}).contiguous();
+  auto perm = ids_on_device(permutation, "permutation");
+  const int64_t n_out = recv_offset.index({-1}).item<int64_t>();
+  if (fwd_flag) {
+    TORCH_CHECK(x.size(0) == n_out, "npc: with one GPU the received row count equals the sent one");
+    auto out = torch::empty({perm.numel(), feat_dim}, x.options());
+    check(apt_permute_rows(x.data_ptr(), x.size(0), i64(perm), perm.numel(), feat_dim,
+                           static_cast<int>(x.element_size()), out.data_ptr(), stream()));
+    return out;
+  }
+  TORCH_CHECK(perm.numel() == x.size(0), "npc: permutation must name every input row");
+  auto out = torch::zeros({n_out, feat_dim}, x.options());
+  check(apt_scatter_rows(x.data_ptr(), i64(perm), perm.numel(), feat_dim,
+                         static_cast<int>(x.element_size()), out.data_ptr(), n_out, stream()));
+  return out;
+}
+
+// ---------------------------------------------------------------- peers only
+#define NPC_NEEDS_PEERS(name)                                                              \
+  TORCH_CHECK(false, "npc." name " talks to other GPUs over NCCL in the reference; this " \
+                     "library builds one GPU's share only")
+
+Tensor NCCLGetUniqueId() { NPC_NEEDS_PEERS("nccl_get_unique_id"); }
+void Initialize(IdType, IdType, IdType, Tensor, IdType) { NPC_NEEDS_PEERS("init"); }
+void AlltoAll(Tensor, Tensor, Tensor, Tensor, IdType, IdType) { NPC_NEEDS_PEERS("alltoall"); }
+Tensor CrossMachineLoadSubtensor(Tensor) { NPC_NEEDS_PEERS("crossmachine_load_subtensor"); }
+Tensor SrcDsttoVir(IdType, Tensor, Tensor) { NPC_NEEDS_PEERS("srcdst_to_vir"); }
+Tensor SrcToVir(IdType, IdType, Tensor) { NPC_NEEDS_PEERS("src_to_vir"); }
+std::vector<Tensor> NPSampleAndShuffle(Tensor, IdType) { NPC_NEEDS_PEERS("np_sample_and_shuffle"); }
+std::vector<Tensor> SPSampleAndShuffle(IdType, Tensor, Tensor, Tensor, IdType) {
+  NPC_NEEDS_PEERS("sp_sample_and_shuffle");
+}
+std::vector<Tensor> SPSampleShuffleSrc(Tensor) { NPC_NEEDS_PEERS("sp_sample_shuffle_src"); }
+std::vector<Tensor> MPSampleShuffle(Tensor, Tensor, Tensor) { NPC_NEEDS_PEERS("mp_sample_shuffle"); }
+Tensor SPFeatShuffle(Tensor, Tensor, Tensor, IdType, IdType, IdType) { NPC_NEEDS_PEERS("sp_feat_shuffle"); }
+Tensor MPFeatShuffleFwd(Tensor, Tensor, Tensor, IdType) { NPC_NEEDS_PEERS("mp_feat_shuffle_fwd"); }
+Tensor MPFeatShuffleBwd(Tensor, Tensor, Tensor, IdType) { NPC_NEEDS_PEERS("mp_feat_shuffle_bwd"); }
+
+TORCH_LIBRARY(npc, m) {
+  // same names and order as the reference's src/pybind.cc:18-48
+  m.def("nccl_get_unique_id", &NCCLGetUniqueId)
+      .def("init", &Initialize)
+      .def("alltoall", &AlltoAll)
+      .def("cache_feats_shared", &CacheFeatsShared)
+      .def("mix_cache_graphs", &MixCacheGraphs)
+      .def("register_min_vids", &RegisterMinVids)
+      .def("register_multi_machines_scheme", &RegisterMultiMachinesScheme)
+      .def("cpu_load_subtensor", &CPULoadSubtensor)
+      .def("load_subtensor", &LoadSubtensor)
+      .def("crossmachine_load_subtensor", &CrossMachineLoadSubtensor)
+      .def("cluster_reqs", &ClusterReqs)
+      .def("local_sample_one_layer", &LocalSamplingNeibhorsOneLayer)
+      .def("srcdst_to_vir", &SrcDsttoVir)
+      .def("src_to_vir", &SrcToVir)
+      .def("np_sample_and_shuffle", &NPSampleAndShuffle)
+      .def("sp_sample_and_shuffle", &SPSampleAndShuffle)
+      .def("sp_sample_shuffle_src", &SPSampleShuffleSrc)
+      .def("mp_sample_shuffle", &MPSampleShuffle)
+      .def("feat_shuffle", &FeatShuffle)
+      .def("sp_feat_shuffle", &SPFeatShuffle)
+      .def("mp_feat_shuffle_fwd", &MPFeatShuffleFwd)
+      .def("mp_feat_shuffle_bwd", &MPFeatShuffleBwd)
+      .def("shuffle_seeds", &ShuffleSeeds)
+      .def("relabel_csc", &RelabelCSC)
+      // additions (no counterpart in the reference)
+      .def("sample_neighbors", &SampleNeighbors)
+      .def("cluster_and_permute", &ClusterAndPermuteLocal)
+      .def("register_graph_partition", &RegisterGraphPartition)
+      .def("set_topology", &SetTopology)
+      .def("set_rng_seed", &SetRngSeed)
+      .def("set_strict", &SetStrict);
+}
+
+}  // namespace npc

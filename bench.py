@@ -40,9 +40,13 @@ def parse_args():
     ap.add_argument("--fan_out", type=str, default=None,
                     help="comma list, k-hop..1-hop as in the reference (the seeds use the last entry)")
     ap.add_argument("--replace", action="store_true", help="sample with replacement (reference semantics)")
-    ap.add_argument("--cpu_batches", type=int, default=None, help="batches timed on the CPU oracle (0 = skip)")
+    ap.add_argument("--cpu_seconds", type=float, default=12.0,
+                    help="seconds of CPU-oracle work for the cpu_baseline leg (0 = skip)")
     ap.add_argument("--cpu_threads", type=int, default=None)
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused"],
+                    help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
+                         "unfused: per-hop sample + hash relabel calls")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
@@ -88,7 +92,11 @@ def main():
 
     graph = capi.Graph(indptr, indices)
     store = capi.FeatStore(feats)
-    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace)
+    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace,
+                             fused=args.driver != "unfused", use_graph=args.driver == "graph")
+    # the per-stage pass brackets stages with events, which a graph replay does not allow
+    stage_pipe = pipe if args.driver != "graph" else MiniBatchPipeline(
+        graph, store, B, hops, replace=args.replace, fused=True, use_graph=False)
 
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.seed + 2)
@@ -121,29 +129,26 @@ def main():
     for i in range(K):
         e0, e1, e2 = ev(), ev(), ev()
         e0.record()
-        pipe.sample(seed_sets[W + i], args.seed + 100 + W + i)
+        stage_pipe.sample(seed_sets[W + i], args.seed + 100 + W + i)
         e1.record()
-        pipe.gather()
+        stage_pipe.gather()
         e2.record()
         torch.cuda.synchronize()
         t_sample += e0.elapsed_time(e1)
         t_gather += e1.elapsed_time(e2)
-        sizes = pipe.sizes.cpu().tolist()
+        sizes = stage_pipe.sizes.cpu().tolist()
         edges += sizes[-1]
         rows += sizes[len(hops)]
         hop_sizes.append(sizes[:-1])
-    assert int(pipe.misses.item()) == 0
+    assert int(pipe.misses.item()) == 0 and int(stage_pipe.misses.item()) == 0
     bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
 
     # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
     cpu = None
-    n_cpu = args.cpu_batches
-    if n_cpu is None:
-        n_cpu = {"full": 6, "medium": 20, "small": 40}[args.workload]
-    n_cpu = min(n_cpu, K)
-    if n_cpu > 0:
+    budget = args.cpu_seconds
+    if budget > 0:
         import numpy as np
 
         import oracle as orc
@@ -157,19 +162,24 @@ def main():
             h_feats = feats.cpu().numpy()
         og = orc.Graph(h_indptr, h_indices)
         ofs = orc.FeatStore(h_feats)
-        cpu_edges = 0
+        h_seeds = [s.cpu().numpy() for s in seed_sets[W:]]
+        cpu_edges = cpu_batches = 0
         tc = 0.0
-        for i in range(n_cpu):
-            s = seed_sets[W + i].cpu().numpy()
+        while tc < budget:
+            # the timed batches, cycled with fresh rng keys once they are used up
+            s = h_seeds[cpu_batches % K]
+            key = args.seed + 100 + W + cpu_batches
             t1 = time.perf_counter()
-            inp, blocks = orc.sample_blocks(og, s, hops, args.replace, args.seed + 100 + W + i)
+            inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
             orc.gather_rows(ofs, inp)
             tc += time.perf_counter() - t1
             cpu_edges += sum(int(b["counts"].sum()) for b in blocks)
+            cpu_batches += 1
         cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
-                   sample=f"{n_cpu} of the {K} timed batches (same seeds and rng keys): sampling and "
-                          f"gather on {threads} OpenMP threads, relabel on 1; {tc:.1f} s of CPU work")
-        del h_indices, h_feats
+                   sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
+                          f"with fresh rng keys) in {tc:.1f} s: sampling and gather on {threads} "
+                          f"OpenMP threads, relabel on 1 thread")
+        del h_indices, h_feats, og, ofs
 
     out = {
         "metric": "sampled edges/s (3-hop 15,10,5) + feature-gather GB/s as % of HBM peak",
@@ -190,7 +200,7 @@ def main():
                         f"fan_out {w['fan_out']} (hops from the seeds: {hops}), "
                         f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
                         f"gather of all input nodes",
-            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"],
+            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver,
         },
         "roofline": {
             "bound": "hbm", "kernel": "gather_kernel",

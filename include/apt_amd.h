@@ -46,7 +46,8 @@ int apt_abi_version(void);
  * counterpart in the reference whose launch shapes are compile-time constants,
  * src/cuda/npc_kernel.h:10-14).  value 0 restores the default.
  *   "sample_lanes_per_row"   8|16|32|64 lanes of a wavefront per frontier row
- *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing */
+ *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing
+ *   "gather_max_blocks"      cap on the gather grid (rows are strided over) */
 int apt_set_tuning(const char* key, int value);
 
 /* A CSR (CSC in the reference's naming: row v lists the in-neighbours of v)

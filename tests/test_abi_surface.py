@@ -1,0 +1,95 @@
+"""No-GPU checks of the drop-in boundary: the C-ABI library exports every
+symbol the headers declare, and the torch operator library registers the
+operator names (and inferred schemas) the reference binds."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    names = []
+    for hdr in ("apt_amd.h", "apt_synth.h"):
+        text = open(os.path.join(ROOT, "include", hdr)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(apt_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from apt_amd import capi
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    declared = _declared_functions()
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
+        assert name in capi.SYMBOLS, f"{name} has no ctypes prototype in capi.SYMBOLS"
+    assert capi.lib().apt_abi_version() == 1
+
+
+def test_argument_checks_need_no_gpu():
+    """Host-side validation runs before anything touches the device."""
+    from apt_amd import capi
+    L = capi.lib()
+    g = capi.CGraph()
+    assert L.apt_sample_neighbors(ctypes.byref(g), None, -1, None, 5, 0, 1, 0, None, None, None, None) != 0
+    assert b"num_frontier" in L.apt_last_error()
+    assert L.apt_sample_neighbors(ctypes.byref(g), None, 4, None, 0, 0, 1, 0, None, None, None, None) != 0
+    assert b"fanout" in L.apt_last_error()
+    assert L.apt_relabel(None, -1, None, None, 0, 0, None, None, None, None, None, 0, None) != 0
+    assert L.apt_relabel_workspace_bytes(1 << 40) == 0
+    assert L.apt_relabel_workspace_bytes(1000) > 0
+    assert L.apt_bucket_workspace_bytes(10, 0) == 0 and L.apt_bucket_workspace_bytes(10, 8) > 0
+    assert L.apt_set_tuning(b"no_such_knob", 1) != 0
+    fan = (ctypes.c_int * 3)(5, 10, 15)
+    assert L.apt_minibatch_capacity(4096, fan, 3, 3) == 4096 * 6 * 11 * 16
+    assert L.apt_minibatch_capacity(1 << 28, fan, 3, 3) == -1          # ids would not fit 32 bits
+    assert L.apt_rank_table_bytes(111_059_956) >= 4 * 111_059_956
+
+
+REFERENCE_OPS = {   # reference src/pybind.cc:19-47 with the schemas torch infers from the C++ types
+    "nccl_get_unique_id": "() -> Tensor",
+    "init": "(int _0, int _1, int _2, Tensor _3, int _4) -> ()",
+    "cache_feats_shared": "(int _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, int _5) -> ()",
+    "mix_cache_graphs": "(int _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, Tensor _5) -> ()",
+    "register_min_vids": "(Tensor _0, int _1) -> ()",
+    "register_multi_machines_scheme": "(Tensor _0, Tensor _1) -> ()",
+    "cpu_load_subtensor": "(Tensor _0) -> Tensor",
+    "load_subtensor": "(Tensor _0) -> Tensor",
+    "crossmachine_load_subtensor": "(Tensor _0) -> Tensor",
+    "cluster_reqs": "(Tensor _0) -> (Tensor, Tensor, Tensor)",
+    "local_sample_one_layer": "(Tensor _0, int _1) -> Tensor[]",
+    "np_sample_and_shuffle": "(Tensor _0, int _1) -> Tensor[]",
+    "feat_shuffle": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, int _4, int _5) -> Tensor",
+    "shuffle_seeds": "(Tensor _0) -> (Tensor, Tensor, Tensor, Tensor)",
+    "relabel_csc": "(Tensor _0, Tensor _1) -> Tensor[]",
+    "alltoall": None, "srcdst_to_vir": None, "src_to_vir": None, "sp_sample_and_shuffle": None,
+    "sp_sample_shuffle_src": None, "mp_sample_shuffle": None, "sp_feat_shuffle": None,
+    "mp_feat_shuffle_fwd": None, "mp_feat_shuffle_bwd": None,
+}
+
+
+def test_operator_names_and_schemas():
+    import torch
+
+    import apt_amd  # noqa: F401  (loads libnpc.so)
+    for name, schema in REFERENCE_OPS.items():
+        got = torch._C._jit_get_schemas_for_operator(f"npc::{name}")
+        assert len(got) == 1, name
+        if schema is not None:
+            text = re.sub(r" _\d+(?=[,)]|$)", "", str(got[0]).replace(f"npc::{name}", ""))
+            want = re.sub(r" _\d+(?=[,)]|$)", "", schema)
+            assert text == want, (name, text, want)
+
+
+def test_peer_operators_raise():
+    import torch
+
+    import apt_amd  # noqa: F401
+    with pytest.raises(RuntimeError, match="other GPUs"):
+        torch.ops.npc.np_sample_and_shuffle(torch.arange(4), 3)
+    with pytest.raises(RuntimeError, match="other GPUs"):
+        torch.ops.npc.nccl_get_unique_id()

@@ -74,10 +74,9 @@ def test_fused_driver_edge_cases(orc, capi):
 
 def test_operator_layer_dp_sampler(orc, capi):
     import apt_amd as npc
-    from apt_amd.state import STATE
     indptr, indices, feats = _setup(orc, capi, n=8000, dim=32, seed=5)
     n = len(indptr) - 1
-    STATE.reset()
+    npc.set_topology(0, 1)
     e = torch.empty(0, dtype=torch.int64)
     npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
     npc.cache_feats_shared(n, torch.from_numpy(feats), torch.empty(0, 32), e, torch.arange(n), 0)
@@ -104,18 +103,19 @@ def test_operator_layer_dp_sampler(orc, capi):
     assert np.array_equal(npc.cpu_load_subtensor(input_nodes.cpu()).cpu().numpy(), feats[frontier])
     with pytest.raises(IndexError):
         npc.load_subtensor(torch.tensor([0, n + 5]))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError):
         npc.np_sample_and_shuffle(dev(seeds), 5)
-    STATE.reset()
+    # the operators are reachable under the reference's names
+    u, r = torch.ops.npc.relabel_csc(dev(seeds), dev(seeds[::-1].copy()))
+    assert np.array_equal(u.cpu().numpy(), seeds)
 
 
 def test_operator_layer_caches_and_buckets(orc, capi):
     import apt_amd as npc
-    from apt_amd.state import STATE
     indptr, indices, feats = _setup(orc, capi, n=6000, dim=24, seed=6)
     n = len(indptr) - 1
     rng = np.random.default_rng(2)
-    STATE.reset()
+    npc.set_topology(0, 1)
     # graph cache: rows of the 500 highest-degree nodes in a second table
     deg = np.diff(indptr)
     hot = np.argsort(-deg, kind="stable")[:500]
@@ -155,6 +155,8 @@ def test_operator_layer_caches_and_buckets(orc, capi):
         assert np.array_equal(g.cpu().numpy(), w)
     rwm = np.array([0, 1, 1, 2, 2, 3, 3, 3])
     npc.register_multi_machines_scheme(torch.from_numpy(rwm), torch.arange(4))
+    with pytest.raises(RuntimeError):
+        npc.shuffle_seeds(dev(ids))                             # world_size 8 needs peers
     got = npc.cluster_reqs(dev(ids))
     want = orc.cluster_reqs(ids, pos, rwm, min_vids, 8, 4)
     assert np.array_equal(got[0].cpu().numpy(), want[0])
@@ -171,4 +173,3 @@ def test_operator_layer_caches_and_buckets(orc, capi):
     assert torch.equal(fwd, h[perm])
     bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm, 16, 0)
     assert torch.equal(bwd, h)                                  # pack undoes unpack
-    STATE.reset()
