@@ -60,6 +60,7 @@ SYMBOLS = {
                                   _SZ, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
+    "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
 }
 
 
@@ -381,3 +382,12 @@ class MinibatchPlan:
             _ptr(self.rng_seed_dev) if rng_seed is None else None, _ptr(self.table), self.table_len,
             _ptr(self.nodes), self._nb, self._rl, self._ct, _ptr(self.sizes), _ptr(self.workspace),
             self.workspace.numel(), _stream()))
+
+
+def synth_copy(src, dst):
+    """dst := src with the plain copy kernel (counter calibration)."""
+    nbytes = src.numel() * src.element_size()
+    if dst.numel() * dst.element_size() != nbytes:
+        raise AptError("synth_copy: size mismatch")
+    check(lib().apt_synth_copy(_ptr(src), _ptr(dst), nbytes, _stream()))
+    return dst

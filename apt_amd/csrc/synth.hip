@@ -67,7 +67,31 @@ __global__ __launch_bounds__(kSynBlock) void rmat_fill_kernel(
   }
 }
 
+// Plain streaming copy in 16-byte vectors: the known-size reference for
+// scaling hardware traffic counters.
+__global__ __launch_bounds__(kSynBlock) void copy_kernel(const uint4* __restrict__ src,
+                                                         uint4* __restrict__ dst, int64_t vecs) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kSynBlock + threadIdx.x; i < vecs;
+       i += static_cast<int64_t>(gridDim.x) * kSynBlock)
+    dst[i] = src[i];
+}
+
 }  // namespace apt
+
+extern "C" int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(bytes >= 0 && bytes % 16 == 0, APT_EINVAL, "apt_synth_copy: bytes must be a multiple of 16");
+  if (bytes == 0) return APT_OK;
+  APT_REQUIRE(src != nullptr && dst != nullptr &&
+                  ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
+              APT_EINVAL, "apt_synth_copy: src/dst must be 16-byte aligned");
+  const int64_t vecs = bytes / 16;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(vecs, kSynBlock), 16384));
+  hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(kSynBlock), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(src), static_cast<uint4*>(dst), vecs);
+  APT_LAUNCH_CHECK("copy_kernel");
+  return APT_OK;
+}
 
 extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_edges,
                                    int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,

@@ -17,6 +17,9 @@ import sys
 import time
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes the gather kernel moves per gathered row, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this script (profiles/gather_kernel_full_pmc.txt); None where it has not been measured.
+MEASURED_GATHER_TRAFFIC_PER_ROW = {"full": 520.0}
 
 WORKLOADS = {
     # BASELINE.json configs[3]: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
@@ -47,6 +50,11 @@ def parse_args():
     ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused"],
                     help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
                          "unfused: per-hop sample + hash relabel calls")
+    ap.add_argument("--inflight", type=int, default=3,
+                    help="batches in flight: N pipelines on N HIP streams, batches dealt round-robin")
+    ap.add_argument("--calibration_copy_mib", type=int, default=0,
+                    help="also launch the plain copy kernel once on this many MiB (for scaling "
+                         "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
@@ -108,18 +116,45 @@ def main():
         seed_sets = [torch.randperm(w["nodes"], generator=gen, device=dev)[:B].contiguous()
                      for _ in range(K + W)]
 
+    # N batches in flight: each pipeline owns its buffers, rank table and stream
+    pipes, streams = [pipe], [torch.cuda.current_stream()]
+    for _ in range(1, max(1, args.inflight)):
+        pipes.append(MiniBatchPipeline(graph, store, B, hops, replace=args.replace,
+                                       fused=args.driver != "unfused", use_graph=args.driver == "graph"))
+        streams.append(torch.cuda.Stream())
+    torch.cuda.synchronize()
+
+    def run_batches(first, count):
+        for i in range(count):
+            k = i % len(pipes)
+            with torch.cuda.stream(streams[k]):
+                pipes[k].run(seed_sets[first + i], args.seed + 100 + first + i)
+
     # ---- warm-up
-    for i in range(W):
-        pipe.run(seed_sets[i], args.seed + 100 + i)
+    run_batches(0, W)
     torch.cuda.synchronize()
 
     # ---- timed region: exactly K steps
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    run_batches(W, K)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    if args.calibration_copy_mib > 0:
+        a = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        capi.synth_copy(a, b)
+        torch.cuda.synchronize()
+        del a, b
+
+    # ---- the same K steps on one stream (latency of a batch when nothing overlaps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
     for i in range(K):
         pipe.run(seed_sets[W + i], args.seed + 100 + W + i)
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    single_stream_ms = (time.perf_counter() - t0) / K * 1e3
 
     # ---- per-stage pass over the same K batches (HIP events on the launch stream)
     ev = lambda: torch.cuda.Event(enable_timing=True)
@@ -140,7 +175,7 @@ def main():
         edges += sizes[-1]
         rows += sizes[len(hops)]
         hop_sizes.append(sizes[:-1])
-    assert int(pipe.misses.item()) == 0 and int(stage_pipe.misses.item()) == 0
+    assert all(int(p.misses.item()) == 0 for p in pipes) and int(stage_pipe.misses.item()) == 0
     bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
@@ -200,17 +235,22 @@ def main():
                         f"fan_out {w['fan_out']} (hops from the seeds: {hops}), "
                         f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
                         f"gather of all input nodes",
-            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver,
+            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver, "batches_in_flight": len(pipes),
         },
         "roofline": {
             "bound": "hbm", "kernel": "gather_kernel",
             "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": gather_gbps / HBM_PEAK_GBPS, "traffic": None,
+            "frac": gather_gbps / HBM_PEAK_GBPS,
+            "traffic": (MEASURED_GATHER_TRAFFIC_PER_ROW[args.workload] * rows / K
+                        if args.workload in MEASURED_GATHER_TRAFFIC_PER_ROW and not args.fan_out
+                        and not args.batch_size else None),
+            "algorithmic_bytes_per_launch": bytes_per_row * rows / K,
             "bytes_per_row": bytes_per_row, "rows_per_launch": rows / K,
             "avg_launch_us": t_gather / K * 1e3,
         },
         "cpu_baseline": cpu,
         "stages": {
+            "single_stream_ms_per_step": single_stream_ms,
             "edges_per_step": edges / K,
             "input_nodes_per_step": rows / K,
             "sample_relabel_ms": t_sample / K,

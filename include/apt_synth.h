@@ -25,6 +25,11 @@ int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_ed
                         int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
                         int64_t* indices, void* stream);
 
+/* Plain device-to-device copy of `bytes` (multiple of 16) with a known
+ * traffic of `bytes` read + `bytes` written: the reference point for scaling
+ * the FETCH_SIZE / WRITE_SIZE hardware counters. */
+int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
