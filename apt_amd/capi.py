@@ -49,8 +49,8 @@ SYMBOLS = {
     "apt_permute_rows": (_I, [_P, _I64, _P, _I64, _I64, _I, _P, _P]),
     "apt_scatter_rows": (_I, [_P, _P, _I64, _I64, _I, _P, _I64, _P]),
     "apt_bucket_workspace_bytes": (_SZ, [_I64, _I]),
-    "apt_cluster_permute": (_I, [_P, _I64, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
-    "apt_cluster_reqs": (_I, [_P, _I64, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_cluster_permute": (_I, [_P, _I64, _P, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_cluster_reqs": (_I, [_P, _I64, _P, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_rank_table_bytes": (_SZ, [_I64]),
     "apt_rank_table_init": (_I, [_P, _SZ, _P]),
     "apt_minibatch_workspace_bytes": (_SZ, [_I64, C.POINTER(C.c_int), _I]),
@@ -59,7 +59,7 @@ SYMBOLS = {
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                   _SZ, _P]),
     # include/apt_synth.h
-    "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
+    "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
 }
 
@@ -272,7 +272,8 @@ def scatter_rows(table, perm, num_out_rows=None, out=None):
     return out
 
 
-def cluster_permute(ids, min_vids, num_buckets, id_offset=0, rank=0, node_beg=0, node_end=None):
+def cluster_permute(ids, min_vids, num_buckets, id_offset=0, rank=0, node_beg=0, node_end=None,
+                    n_dev=None):
     """-> (bucket_size, bucket_offset, sorted_ids, permutation), all on the GPU."""
     ids = _dev_i64(ids, "ids")
     min_vids = _dev_i64(min_vids, "min_vids")
@@ -289,14 +290,16 @@ def cluster_permute(ids, min_vids, num_buckets, id_offset=0, rank=0, node_beg=0,
     if need == 0:
         raise AptError(f"cluster_permute: unsupported size (n={n}, buckets={num_buckets})")
     ws = torch.empty(need, dtype=torch.uint8, device=dev)
-    check(lib().apt_cluster_permute(_ptr(ids), n, _ptr(min_vids), int(num_buckets), int(id_offset),
+    check(lib().apt_cluster_permute(_ptr(ids), n, _ptr(n_dev), _ptr(min_vids), int(num_buckets), int(id_offset),
                                     int(rank), int(node_beg), int(node_end), _ptr(bs), _ptr(bo),
                                     _ptr(so), _ptr(pm), _ptr(ws), ws.numel(), _stream()))
     return bs, bo, so, pm
 
 
-def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num_remote_workers):
-    """-> (bucket_size, bucket_offset, sorted_ids, permutation), all on the GPU."""
+def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num_remote_workers,
+                 n_dev=None, out=None, workspace=None):
+    """-> (bucket_size, bucket_offset, sorted_ids, permutation), all on the GPU.
+    `out` / `workspace` let a caller reuse buffers across batches."""
     ids = _dev_i64(ids, "ids")
     feat_pos_map = _dev_i64(feat_pos_map, "feat_pos_map")
     remote_worker_map = _dev_i64(remote_worker_map, "remote_worker_map")
@@ -304,27 +307,32 @@ def cluster_reqs(ids, feat_pos_map, remote_worker_map, min_vids, world_size, num
     if min_vids.numel() < world_size + 1 or remote_worker_map.numel() < world_size:
         raise AptError("cluster_reqs: min_vids / remote_worker_map shorter than world_size")
     dev, n = ids.device, ids.numel()
-    bs = torch.empty(num_remote_workers, dtype=torch.int64, device=dev)
-    bo = torch.empty(num_remote_workers, dtype=torch.int64, device=dev)
-    so = torch.empty(n, dtype=torch.int64, device=dev)
-    pm = torch.empty(n, dtype=torch.int64, device=dev)
+    if out is None:
+        out = (torch.empty(num_remote_workers, dtype=torch.int64, device=dev),
+               torch.empty(num_remote_workers, dtype=torch.int64, device=dev),
+               torch.empty(n, dtype=torch.int64, device=dev),
+               torch.empty(n, dtype=torch.int64, device=dev))
+    bs, bo, so, pm = out
     need = int(lib().apt_bucket_workspace_bytes(n, int(num_remote_workers)))
     if need == 0:
         raise AptError(f"cluster_reqs: unsupported size (n={n}, buckets={num_remote_workers})")
-    ws = torch.empty(need, dtype=torch.uint8, device=dev)
-    check(lib().apt_cluster_reqs(_ptr(ids), n, _ptr(feat_pos_map), feat_pos_map.numel(),
+    ws = workspace if workspace is not None else torch.empty(need, dtype=torch.uint8, device=dev)
+    if ws.numel() < need:
+        raise AptError("cluster_reqs: workspace too small")
+    check(lib().apt_cluster_reqs(_ptr(ids), n, _ptr(n_dev), _ptr(feat_pos_map), feat_pos_map.numel(),
                                  _ptr(remote_worker_map), _ptr(min_vids), int(world_size),
                                  int(num_remote_workers), _ptr(bs), _ptr(bo), _ptr(so), _ptr(pm),
                                  _ptr(ws), ws.numel(), _stream()))
     return bs, bo, so, pm
 
 
-def synth_rmat_fill(indptr, num_nodes, num_edges, levels, seed, thr0, thr1, indices):
+def synth_rmat_fill(indptr, row_begin, num_nodes, num_edges, levels, seed, thr0, thr1, indices):
     indptr = _dev_i64(indptr, "indptr")
     indices = _dev_i64(indices, "indices")
-    if indices.numel() < num_edges or indptr.numel() != num_nodes + 1:
+    if indices.numel() < num_edges:
         raise AptError("synth_rmat_fill: buffer sizes do not match")
-    check(lib().apt_synth_rmat_fill(_ptr(indptr), int(num_nodes), int(num_edges), int(levels),
+    check(lib().apt_synth_rmat_fill(_ptr(indptr), indptr.numel() - 1, int(row_begin), int(num_nodes),
+                                    int(num_edges), int(levels),
                                     int(seed) & 0xFFFFFFFFFFFFFFFF, int(thr0), int(thr1),
                                     _ptr(indices), _stream()))
     return indices

@@ -20,7 +20,8 @@ constexpr int kBktWaves = kBktBlock / kWave;
 
 struct BucketParams {
   const int64_t* ids;
-  int64_t n;
+  int64_t n;                 // host-side count (upper bound when n_dev != NULL)
+  const int64_t* n_dev;
   const int64_t* min_vids;   // [world + 1]
   int world;                 // entries scanned in min_vids
   int num_buckets;           // output buckets
@@ -48,10 +49,11 @@ __global__ __launch_bounds__(kBktBlock) void bucket_classify_kernel(BucketParams
   if (p.feat_pos_map != nullptr && tid < p.world) s_map[tid] = p.remote_worker_map[tid];
   if (tid < APT_MAX_BUCKETS) s_hist[tid] = 0;
   __syncthreads();
+  const int64_t n = actual_count(p.n, p.n_dev);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kBktTile;
   for (int it = 0; it < kBktIters; ++it) {
     const int64_t i = base + it * kBktBlock + tid;
-    if (i < p.n) {
+    if (i < n) {
       const int64_t v = p.ids[i];
       int64_t d;
       if (p.feat_pos_map == nullptr) {
@@ -120,6 +122,7 @@ __global__ __launch_bounds__(kBktBlock) void bucket_place_kernel(BucketParams p)
   const int lane = lane_id();
   const int wave = tid / kWave;
   const int nb = p.num_buckets;
+  const int64_t n = actual_count(p.n, p.n_dev);
   if (tid == 0) {
     int64_t acc = 0;
     for (int w = 0; w < nb; ++w) {
@@ -133,13 +136,13 @@ __global__ __launch_bounds__(kBktBlock) void bucket_place_kernel(BucketParams p)
     }
   }
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kBktTile;
-  if (base >= p.n) return;  // block-uniform (only block 0 when n == 0)
+  if (base >= n) return;  // block-uniform
   int mine[kBktIters];
   uint32_t rank_in_wave[kBktIters];
 #pragma unroll
   for (int it = 0; it < kBktIters; ++it) {
     const int64_t i = base + it * kBktBlock + tid;
-    mine[it] = i < p.n ? static_cast<int>(p.bucket_of[i]) : -1;
+    mine[it] = i < n ? static_cast<int>(p.bucket_of[i]) : -1;
     rank_in_wave[it] = 0;
     for (int w = 0; w < nb; ++w) {
       const uint64_t m = ballot(mine[it] == w);
@@ -218,7 +221,8 @@ extern "C" size_t apt_bucket_workspace_bytes(int64_t n, int num_buckets) {
   return apt::bucket_layout(n, num_buckets).total;
 }
 
-extern "C" int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* min_vids,
+extern "C" int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* n_dev,
+                                   const int64_t* min_vids,
                                    int num_buckets, int64_t id_offset, int rank, int node_beg,
                                    int node_end, int64_t* bucket_size, int64_t* bucket_offset,
                                    int64_t* sorted_ids, int64_t* permutation, void* workspace,
@@ -242,6 +246,7 @@ extern "C" int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t*
   BucketParams p{};
   p.ids = ids;
   p.n = n;
+  p.n_dev = n_dev;
   p.min_vids = min_vids;
   p.world = num_buckets;
   p.num_buckets = num_buckets;
@@ -258,7 +263,8 @@ extern "C" int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t*
                        "apt_cluster_permute");
 }
 
-extern "C" int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* feat_pos_map,
+extern "C" int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_dev,
+                                const int64_t* feat_pos_map,
                                 int64_t num_total_nodes, const int64_t* remote_worker_map,
                                 const int64_t* min_vids, int world_size, int num_remote_workers,
                                 int64_t* bucket_size, int64_t* bucket_offset,
@@ -282,6 +288,7 @@ extern "C" int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* fe
   BucketParams p{};
   p.ids = ids;
   p.n = n;
+  p.n_dev = n_dev;
   p.min_vids = min_vids;
   p.world = world_size;
   p.num_buckets = num_remote_workers;

@@ -20,27 +20,32 @@ __device__ __forceinline__ int64_t row_of_edge(const int64_t* indptr, int64_t lo
 }
 
 __global__ __launch_bounds__(kSynBlock) void rmat_fill_kernel(
-    const int64_t* __restrict__ indptr, int64_t num_nodes, int64_t num_edges, int levels,
-    uint64_t seed, uint32_t thr0, uint32_t thr1, int64_t* __restrict__ indices) {
+    const int64_t* __restrict__ indptr, int64_t num_rows, int64_t row_begin, int64_t num_nodes,
+    int64_t num_edges, int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
+    int64_t* __restrict__ indices) {
   __shared__ int64_t s_lo, s_hi;
   const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kSynEdgesPerBlock;
   if (e0 >= num_edges) return;
   const int64_t e1 = min(e0 + kSynEdgesPerBlock, num_edges) - 1;
-  if (threadIdx.x == 0) s_lo = row_of_edge(indptr, 0, num_nodes - 1, e0);
-  if (threadIdx.x == 1) s_hi = row_of_edge(indptr, 0, num_nodes - 1, e1);
+  if (threadIdx.x == 0) s_lo = row_of_edge(indptr, 0, num_rows - 1, e0);
+  if (threadIdx.x == 1) s_hi = row_of_edge(indptr, 0, num_rows - 1, e1);
   __syncthreads();
   const int64_t lo = s_lo, hi = s_hi;
   for (int64_t e = e0 + threadIdx.x; e <= e1; e += kSynBlock) {
-    const int64_t u = row_of_edge(indptr, lo, hi, e);
+    const int64_t u = row_begin + row_of_edge(indptr, lo, hi, e);
+    // Slots are keyed by (row id, slot inside the row) so that a partition of
+    // the rows generates exactly the rows of the whole graph.
+    const uint64_t ekey = static_cast<uint64_t>(e - indptr[u - row_begin]);
     int64_t v = 0;
     for (uint32_t attempt = 0; attempt < 32; ++attempt) {
       v = 0;
       for (int l0 = 0; l0 < levels; l0 += 8) {
         uint32_t w[4];
         {
-          uint32_t c0 = static_cast<uint32_t>(static_cast<uint64_t>(e));
-          uint32_t c1 = static_cast<uint32_t>(static_cast<uint64_t>(e) >> 32);
-          uint32_t c2 = static_cast<uint32_t>(l0), c3 = attempt;
+          uint32_t c0 = static_cast<uint32_t>(static_cast<uint64_t>(u));
+          uint32_t c1 = static_cast<uint32_t>(static_cast<uint64_t>(u) >> 32) ^
+                        (static_cast<uint32_t>(l0) << 16) ^ (attempt << 24);
+          uint32_t c2 = static_cast<uint32_t>(ekey), c3 = static_cast<uint32_t>(ekey >> 32);
           uint32_t k0 = static_cast<uint32_t>(seed), k1 = static_cast<uint32_t>(seed >> 32);
 #pragma unroll
           for (int r = 0; r < 10; ++r) {
@@ -93,11 +98,13 @@ extern "C" int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* s
   return APT_OK;
 }
 
-extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_edges,
-                                   int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
-                                   int64_t* indices, void* stream) {
+extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_rows, int64_t row_begin,
+                                   int64_t num_nodes, int64_t num_edges, int levels, uint64_t seed,
+                                   uint32_t thr0, uint32_t thr1, int64_t* indices, void* stream) {
   using namespace apt;
-  APT_REQUIRE(num_nodes > 0 && num_edges >= 0, APT_EINVAL, "apt_synth_rmat_fill: bad sizes");
+  APT_REQUIRE(num_nodes > 0 && num_edges >= 0 && num_rows > 0 && row_begin >= 0 &&
+                  row_begin + num_rows <= num_nodes,
+              APT_EINVAL, "apt_synth_rmat_fill: bad sizes");
   APT_REQUIRE(levels >= 1 && levels <= 40 && (num_nodes - 1) >> levels == 0, APT_EINVAL,
               "apt_synth_rmat_fill: %d levels do not cover %lld nodes", levels, (long long)num_nodes);
   APT_REQUIRE(thr0 <= 65536 && thr1 <= 65536, APT_EINVAL, "apt_synth_rmat_fill: bad thresholds");
@@ -107,8 +114,8 @@ extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int
   const int64_t blocks = ceil_div(num_edges, kSynEdgesPerBlock);
   APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT, "apt_synth_rmat_fill: too many edges");
   hipLaunchKernelGGL(rmat_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kSynBlock), 0,
-                     static_cast<hipStream_t>(stream), indptr, num_nodes, num_edges, levels, seed,
-                     thr0, thr1, indices);
+                     static_cast<hipStream_t>(stream), indptr, num_rows, row_begin, num_nodes,
+                     num_edges, levels, seed, thr0, thr1, indices);
   APT_LAUNCH_CHECK("rmat_fill_kernel");
   return APT_OK;
 }

@@ -287,7 +287,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> ClusterAndPermuteLocal(Tensor seeds) 
   const size_t need = apt_bucket_workspace_bytes(ids.numel(), W);
   TORCH_CHECK(need > 0, "npc: bucketing: unsupported size");
   auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
-  check(apt_cluster_permute(i64(ids), ids.numel(), s.shuffle_min_vids.data_ptr<int64_t>(), W,
+  check(apt_cluster_permute(i64(ids), ids.numel(), nullptr, s.shuffle_min_vids.data_ptr<int64_t>(), W,
                             s.shuffle_id_offset, static_cast<int>(s.rank), node_beg,
                             node_beg + static_cast<int>(s.node_size), size.data_ptr<int64_t>(),
                             offset.data_ptr<int64_t>(), sorted.data_ptr<int64_t>(),
@@ -320,7 +320,7 @@ std::tuple<Tensor, Tensor, Tensor> ClusterReqs(Tensor node_id) {
   const size_t need = apt_bucket_workspace_bytes(ids.numel(), R);
   TORCH_CHECK(need > 0, "npc: bucketing: unsupported size");
   auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
-  check(apt_cluster_reqs(i64(ids), ids.numel(), s.feat_pos_map.data_ptr<int64_t>(),
+  check(apt_cluster_reqs(i64(ids), ids.numel(), nullptr, s.feat_pos_map.data_ptr<int64_t>(),
                          s.feat_pos_map.numel(), s.remote_worker_map.data_ptr<int64_t>(),
                          s.shuffle_min_vids.data_ptr<int64_t>(), static_cast<int>(s.world_size), R,
                          size.data_ptr<int64_t>(), nullptr, sorted.data_ptr<int64_t>(),

@@ -22,9 +22,17 @@ from . import capi
 
 class MiniBatchPipeline:
     def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
-                 use_graph=False):
+                 use_graph=False, requests=None):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
-        --fan_out list reversed)."""
+        --fan_out list reversed).
+
+        requests: dict(feat_pos_map, remote_worker_map, min_vids, world_size,
+        num_remote_workers) for a partitioned feature store.  The input nodes
+        are then bucketed as cluster_reqs does (reference
+        src/load_subtensor.cc:41-56,83-86): bucket 0 = rows present on this GPU,
+        which are gathered; the other buckets are the per-owner request lists
+        that the reference would send (left in `request_ids`, grouped by
+        bucket, sizes in `request_sizes`)."""
         self.graph, self.feat = graph, feat
         self.fanouts = [int(f) for f in hop_fanouts]
         self.replace = bool(replace)
@@ -56,6 +64,15 @@ class MiniBatchPipeline:
         if gather and feat is not None:
             self.features = torch.empty((self.caps[-1], feat.out_dim), dtype=feat.dtype, device=dev)
         self.misses = torch.zeros(1, **i64)
+        self.requests = requests
+        if requests is not None:
+            R = int(requests["num_remote_workers"])
+            self.request_sizes = torch.zeros(R, **i64)
+            self.request_offsets = torch.zeros(R, **i64)
+            self.request_ids = torch.empty(self.caps[-1], **i64)
+            self.request_perm = torch.empty(self.caps[-1], **i64)
+            need = int(capi.lib().apt_bucket_workspace_bytes(self.caps[-1], R))
+            self.request_ws = torch.empty(need, dtype=torch.uint8, device=dev)
         self.seeds = None
         self.graph_exec = None
         if use_graph:
@@ -111,8 +128,18 @@ class MiniBatchPipeline:
         """Features of the input nodes (the last hop's unique ids), asynchronous."""
         H = len(self.fanouts)
         index = self.nodes if self.fused else self.frontier[H]
-        capi.gather_rows(self.feat, index, num_index_dev=self._size(H), out=self.features,
-                         miss_count=self.misses)
+        if self.requests is None:
+            capi.gather_rows(self.feat, index, num_index_dev=self._size(H), out=self.features,
+                             miss_count=self.misses)
+            return
+        rq = self.requests
+        capi.cluster_reqs(index, rq["feat_pos_map"], rq["remote_worker_map"], rq["min_vids"],
+                          rq["world_size"], rq["num_remote_workers"], n_dev=self._size(H),
+                          out=(self.request_sizes, self.request_offsets, self.request_ids,
+                               self.request_perm), workspace=self.request_ws)
+        # rows that are here: features[k] belongs to request_ids[k], k < request_sizes[0]
+        capi.gather_rows(self.feat, self.request_ids, num_index_dev=self.request_sizes[0:1],
+                         out=self.features, miss_count=self.misses)
 
     def run(self, seeds, rng_seed):
         if self.graph_exec is not None:
@@ -143,5 +170,11 @@ class MiniBatchPipeline:
                                   unique=uniq, fanout=f))
         feats = None if self.features is None else self.features[:sizes[H]]
         inp = self.nodes[:sizes[H]] if self.fused else self.frontier[H][:sizes[H]]
-        return dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],
-                    sizes=sizes[:-1])
+        out = dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],
+                   sizes=sizes[:-1])
+        if self.requests is not None:
+            rs = self.request_sizes.cpu().tolist()
+            out.update(request_sizes=rs, request_ids=self.request_ids[:sizes[H]],
+                       request_perm=self.request_perm[:sizes[H]],
+                       features=None if self.features is None else self.features[:rs[0]])
+        return out

@@ -61,7 +61,44 @@ def rmat_csr_numpy(num_nodes, num_edges, seed):
     return csr_from_edges(num_nodes, row, col)
 
 
-def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B, c=RMAT_C):
+def _rmat_log_row_prob(lo, hi, levels, device, a, b, c):
+    """log of the unnormalised R-MAT row probability of ids [lo, hi): every 0
+    bit contributes a+b, every 1 bit c+d."""
+    import math
+
+    import torch
+
+    d = 1.0 - a - b - c
+    u = torch.arange(lo, hi, dtype=torch.int64, device=device)
+    pc = torch.zeros_like(u)
+    for bit in range(levels):
+        pc += (u >> bit) & 1
+    return (levels - pc).to(torch.float64) * math.log(a + b) + pc.to(torch.float64) * math.log(c + d)
+
+
+def rmat_expected_degree(num_nodes, num_edges, device="cuda:0", a=RMAT_A, b=RMAT_B, c=RMAT_C,
+                         lo=0, hi=None):
+    """Expected row degree E * p_u / Z of ids [lo, hi) (float32 tensor)."""
+    import math
+
+    import torch
+
+    levels = max(1, int(math.ceil(math.log2(max(num_nodes, 2)))))
+    chunk = 1 << 24
+    z = 0.0
+    for s in range(0, num_nodes, chunk):
+        z += float(torch.exp(_rmat_log_row_prob(s, min(s + chunk, num_nodes), levels, device, a, b, c)).sum())
+    hi = num_nodes if hi is None else hi
+    scale = math.log(num_edges) - math.log(z)
+    out = torch.empty(hi - lo, dtype=torch.float32, device=device)
+    for s in range(lo, hi, chunk):
+        e = min(s + chunk, hi)
+        out[s - lo:e - lo] = torch.exp(_rmat_log_row_prob(s, e, levels, device, a, b, c) + scale).to(torch.float32)
+    return out
+
+
+def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B, c=RMAT_C,
+                 row_begin=0, num_rows=None):
     """Large R-MAT graph built directly in CSR on the GPU, without a sort.
 
     R-MAT's recursive quadrant choice factorises over bits: row id u has
@@ -70,9 +107,10 @@ def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B
     Poisson(E * p_u / Z) (ids >= num_nodes excluded, i.e. rejected) and every
     neighbour slot is then filled independently by apt_synth_rmat_fill.
     Neighbour lists are unsorted and may repeat an id (multigraph), which the
-    samplers treat as distinct positions.
+    samplers treat as distinct positions.  row_begin / num_rows build only the
+    rows of a contiguous-range partition (neighbour ids stay global).
 
-    -> (indptr int64[num_nodes+1], indices int64[E'], E' ~ num_edges)
+    -> (indptr int64[rows+1], indices int64[E'], E' ~ num_edges * row mass)
     """
     import math
 
@@ -81,37 +119,24 @@ def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B
     from . import capi
 
     d = 1.0 - a - b - c
+    if num_rows is None:
+        num_rows = num_nodes - row_begin
     levels = max(1, int(math.ceil(math.log2(max(num_nodes, 2)))))
     gen = torch.Generator(device=device)
-    gen.manual_seed(int(seed))
-    l0, l1 = math.log(a + b), math.log(c + d)
-    indptr = torch.zeros(num_nodes + 1, dtype=torch.int64, device=device)
+    gen.manual_seed(int(seed) * 1000003 + int(row_begin))
+    rate = rmat_expected_degree(num_nodes, num_edges, device, a, b, c, row_begin, row_begin + num_rows)
+    indptr = torch.zeros(num_rows + 1, dtype=torch.int64, device=device)
     chunk = 1 << 24
-    # normaliser over ids < num_nodes, in float64
-    z = 0.0
-    logp_chunks = []
-    for s in range(0, num_nodes, chunk):
-        u = torch.arange(s, min(s + chunk, num_nodes), dtype=torch.int64, device=device)
-        pc = torch.zeros_like(u)
-        for bit in range(levels):
-            pc += (u >> bit) & 1
-        logp = (levels - pc).to(torch.float64) * l0 + pc.to(torch.float64) * l1
-        z += float(torch.exp(logp).sum().item())
-        logp_chunks.append((s, logp.to(torch.float32)))
-        del u, pc, logp
-    scale = math.log(num_edges) - math.log(z)
-    for s, logp in logp_chunks:
-        rate = torch.exp(logp.to(torch.float64) + scale).to(torch.float32)
-        deg = torch.poisson(rate, generator=gen).to(torch.int64)
-        indptr[s + 1:s + 1 + deg.numel()] = deg
-        del rate, deg
-    del logp_chunks
+    for s in range(0, num_rows, chunk):
+        e = min(s + chunk, num_rows)
+        indptr[s + 1:e + 1] = torch.poisson(rate[s:e], generator=gen).to(torch.int64)
+    del rate
     torch.cumsum(indptr, 0, out=indptr)
     total = int(indptr[-1].item())
     indices = torch.empty(total, dtype=torch.int64, device=device)
     thr0 = int(round(65536 * b / (a + b)))
     thr1 = int(round(65536 * d / (c + d)))
-    capi.synth_rmat_fill(indptr, num_nodes, total, levels, seed, thr0, thr1, indices)
+    capi.synth_rmat_fill(indptr, row_begin, num_nodes, total, levels, seed, thr0, thr1, indices)
     return indptr, indices
 
 

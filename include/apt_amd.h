@@ -195,11 +195,14 @@ int apt_scatter_rows(const void* in, const int64_t* perm, int64_t n,
  *   sorted_ids[n] (ids grouped by bucket, input order kept inside a bucket —
  *   the reference's order inside a bucket is whatever its atomics produce),
  *   permutation[n] (slot of ids[i] in sorted_ids).
+ *   n_dev        optional device int64[1] (as in apt_sample_neighbors); outputs
+ *                beyond the actual count are not written
  *   min_vids     device int64[num_buckets + 1]
  *   workspace    device scratch, apt_bucket_workspace_bytes(n, num_buckets)
  */
 size_t apt_bucket_workspace_bytes(int64_t n, int num_buckets);
-int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* min_vids,
+int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* n_dev,
+                        const int64_t* min_vids,
                         int num_buckets, int64_t id_offset, int rank,
                         int node_beg, int node_end, int64_t* bucket_size,
                         int64_t* bucket_offset, int64_t* sorted_ids,
@@ -213,7 +216,8 @@ int apt_cluster_permute(const int64_t* ids, int64_t n, const int64_t* min_vids,
  *   bucket(v) = feat_pos_map[v] != -1 ? 0 : remote_worker_map[owner(v)]
  *   with owner(v) the min_vids scan above started at 0 and no rank override.
  *   bucket_offset is optional (NULL to skip). */
-int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* feat_pos_map,
+int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_dev,
+                     const int64_t* feat_pos_map,
                      int64_t num_total_nodes, const int64_t* remote_worker_map,
                      const int64_t* min_vids, int world_size,
                      int num_remote_workers, int64_t* bucket_size,

@@ -12,18 +12,19 @@
 extern "C" {
 #endif
 
-/* Fill the neighbour lists of an R-MAT graph whose row degrees are already
- * fixed by indptr (device int64[num_nodes + 1]).  R-MAT factorises: given the
+/* Fill the neighbour lists of rows [row_begin, row_begin + num_rows) of an
+ * R-MAT graph over num_nodes ids whose row degrees are already fixed by indptr
+ * (device int64[num_rows + 1]).  R-MAT factorises: given the
  * bits of the row id u, each bit of a neighbour is an independent Bernoulli
  * draw with P(1 | row bit 0) = b/(a+b) and P(1 | row bit 1) = d/(c+d), so the
- * neighbour of edge slot e is drawn from Philox keyed by (seed, e) with no
- * sort or transpose.  Candidates >= num_nodes are redrawn.
+ * neighbour in slot k of row u is drawn from Philox keyed by (seed, u, k) with
+ * no sort or transpose.  Candidates >= num_nodes are redrawn.
  *   thr0, thr1   the two probabilities scaled to [0, 65536]
- *   indices      device int64[indptr[num_nodes]] (output)
+ *   indices      device int64[indptr[num_rows]] (output)
  */
-int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_nodes, int64_t num_edges,
-                        int levels, uint64_t seed, uint32_t thr0, uint32_t thr1,
-                        int64_t* indices, void* stream);
+int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_rows, int64_t row_begin,
+                        int64_t num_nodes, int64_t num_edges, int levels, uint64_t seed,
+                        uint32_t thr0, uint32_t thr1, int64_t* indices, void* stream);
 
 /* Plain device-to-device copy of `bytes` (multiple of 16) with a known
  * traffic of `bytes` read + `bytes` written: the reference point for scaling

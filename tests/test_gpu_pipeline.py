@@ -173,3 +173,53 @@ def test_operator_layer_caches_and_buckets(orc, capi):
     assert torch.equal(fwd, h[perm])
     bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm, 16, 0)
     assert torch.equal(bwd, h)                                  # pack undoes unpack
+
+
+def test_partitioned_store_pipeline(orc, capi):
+    """One GPU's share: rows [lo, hi) of the graph are here, features of the
+    local nodes plus a cache of hot remote nodes; input nodes are bucketed into
+    "here" + per-owner request lists and the rows that are here are gathered."""
+    from apt_amd.pipeline import MiniBatchPipeline
+    indptr, indices, feats = _setup(orc, capi, n=40000, deg=12, dim=64, seed=31)
+    n, W = 40000, 8
+    lo, hi = 15000, 20000
+    p_indptr = indptr[lo:hi + 1] - indptr[lo]
+    p_indices = indices[indptr[lo]:indptr[hi]]
+    og = orc.Graph(p_indptr, p_indices, row_begin=lo, num_total_nodes=n)
+    dg = capi.Graph(dev(p_indptr), dev(p_indices), row_begin=lo, num_total_nodes=n)
+    deg = np.diff(indptr)
+    remote = np.setdiff1d(np.arange(n), np.arange(lo, hi))
+    hot = remote[np.argsort(-deg[remote], kind="stable")[:7000]]            # 20% of the remote nodes
+    pos = np.full(n, -1, dtype=np.int64)
+    pos[lo:hi] = -np.arange(hi - lo) - 2
+    pos[hot] = np.arange(len(hot))
+    local_t, cache_t = feats[lo:hi], feats[hot]
+    ofs = orc.FeatStore(local_t, cache_t, pos)
+    dfs = capi.FeatStore(dev(local_t), dev(cache_t), dev(pos))
+    min_vids = np.arange(W + 1) * (n // W)
+    rwm = np.arange(W)
+    rq = dict(feat_pos_map=dev(pos), remote_worker_map=dev(rwm), min_vids=dev(min_vids), world_size=W,
+              num_remote_workers=W)
+    hops = [5, 10, 15]
+    pipe = MiniBatchPipeline(dg, dfs, 256, hops, replace=False, requests=rq)
+    rng = np.random.default_rng(3)
+    for batch in range(2):
+        seeds = lo + rng.permutation(hi - lo)[:256]
+        pipe.run(dev(seeds), 500 + batch)
+        res = pipe.result()
+        want_in, want_blocks = orc.sample_blocks(og, seeds, hops, False, 500 + batch)
+        assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+        for got, want in zip(res["blocks"], want_blocks):
+            assert np.array_equal(got["relabeled"].cpu().numpy(), want["relabeled"])
+        bs, bo, so, pm = orc.cluster_reqs(want_in, pos, rwm, min_vids, W, W)
+        assert res["request_sizes"] == bs.tolist()
+        assert np.array_equal(res["request_ids"].cpu().numpy(), so)
+        assert np.array_equal(res["request_perm"].cpu().numpy(), pm)
+        here = so[:bs[0]]
+        want_f, _ = orc.gather_rows(ofs, here)
+        assert np.array_equal(res["features"].cpu().numpy(), want_f)
+        assert bs[1:].sum() > 0 and bs[0] > 0
+        # frontier nodes outside the partition have no adjacency here
+        outer = want_blocks[0]
+        outside = (outer["seeds"] < lo) | (outer["seeds"] >= hi)
+        assert outside.any() and np.all(outer["counts"][outside] == 0)
