@@ -28,6 +28,10 @@ WORKLOADS = {
     # configs[1]: products-sized, 62M edges, 100 x fp32, batch 1024
     "medium": dict(nodes=2_449_029, edges=62_000_000, dim=100, dtype="fp32", batch=1024,
                    fan_out=[15, 10, 5]),
+    # configs[2]: one GPU's share of the full graph: a contiguous 1/8 of the rows, local features plus a
+    # cache of the 20% hottest remote rows, misses bucketed into 8 owner request lists
+    "partition": dict(nodes=111_059_956, edges=3_200_000_000, dim=128, dtype="fp32", batch=1024,
+                      fan_out=[15, 10, 5], parts=8, part=3, cache_ratio=0.2),
     # configs[0]: CPU-runnable plumbing case
     "small": dict(nodes=100_000, edges=1_500_000, dim=128, dtype="fp32", batch=1024, fan_out=[10, 5]),
 }
@@ -91,36 +95,73 @@ def main():
     B, K, W = w["batch"], args.steps, args.warmup
 
     t0 = time.time()
-    indptr, indices = synth.rmat_csr_gpu(w["nodes"], w["edges"], args.seed, dev)
-    feats = synth.random_features(w["nodes"], w["dim"], dtype, args.seed + 1, dev)
+    N = w["nodes"]
+    requests = None
+    part_note = ""
+    if "parts" in w:
+        P = w["parts"]
+        lo, hi = N * w["part"] // P, N * (w["part"] + 1) // P
+        indptr, indices = synth.rmat_csr_gpu(N, w["edges"], args.seed, dev, row_begin=lo, num_rows=hi - lo)
+        graph = capi.Graph(indptr, indices, row_begin=lo, num_total_nodes=N)
+        feats = synth.random_features(hi - lo, w["dim"], dtype, args.seed + 1, dev)
+        # hot-node cache: the remote nodes with the largest expected degree
+        exp_deg = synth.rmat_expected_degree(N, w["edges"], dev)
+        exp_deg[lo:hi] = -1.0
+        n_cache = int((N - (hi - lo)) * w["cache_ratio"])
+        hot = torch.sort(exp_deg, descending=True, stable=True).indices[:n_cache].contiguous()
+        del exp_deg
+        cache = synth.random_features(n_cache, w["dim"], dtype, args.seed + 3, dev)
+        pos_map = torch.full((N,), -1, dtype=torch.int64, device=dev)
+        pos_map[lo:hi] = -torch.arange(hi - lo, dtype=torch.int64, device=dev) - 2
+        pos_map[hot] = torch.arange(n_cache, dtype=torch.int64, device=dev)
+        store = capi.FeatStore(feats, cache, pos_map)
+        min_vids = torch.tensor([N * k // P for k in range(P + 1)], dtype=torch.int64, device=dev)
+        # bucket 0 is this GPU (reference src/cuda/npc_kernel.cu:398-408): the own part maps to 0,
+        # the other owners to 1..P-1
+        rwm = [0] * P
+        nxt = 1
+        for k in range(P):
+            if k != w["part"]:
+                rwm[k] = nxt
+                nxt += 1
+        requests = dict(feat_pos_map=pos_map, remote_worker_map=torch.tensor(rwm, dtype=torch.int64, device=dev),
+                        min_vids=min_vids, world_size=P, num_remote_workers=P)
+        seed_lo, seed_n = lo, hi - lo
+        part_note = (f", rows [{lo}, {hi}) of {P} contiguous parts held here, cache of the {n_cache} "
+                     f"hottest remote rows, misses bucketed into {P} owner lists")
+    else:
+        indptr, indices = synth.rmat_csr_gpu(N, w["edges"], args.seed, dev)
+        feats = synth.random_features(N, w["dim"], dtype, args.seed + 1, dev)
+        graph = capi.Graph(indptr, indices)
+        store = capi.FeatStore(feats)
+        seed_lo, seed_n = 0, N
     torch.cuda.synchronize()
     t_setup = time.time() - t0
     num_edges_graph = int(indices.numel())
     max_deg = int((indptr[1:] - indptr[:-1]).max().item())
 
-    graph = capi.Graph(indptr, indices)
-    store = capi.FeatStore(feats)
-    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace,
-                             fused=args.driver != "unfused", use_graph=args.driver == "graph")
+    def make_pipe(use_graph):
+        return MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused",
+                                 use_graph=use_graph, requests=requests)
+
+    pipe = make_pipe(args.driver == "graph")
     # the per-stage pass brackets stages with events, which a graph replay does not allow
-    stage_pipe = pipe if args.driver != "graph" else MiniBatchPipeline(
-        graph, store, B, hops, replace=args.replace, fused=True, use_graph=False)
+    stage_pipe = pipe if args.driver != "graph" else make_pipe(False)
 
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.seed + 2)
     need = (K + W) * B
-    if need <= w["nodes"]:
-        pool = torch.randperm(w["nodes"], generator=gen, device=dev)[:need]
+    if need <= seed_n:
+        pool = seed_lo + torch.randperm(seed_n, generator=gen, device=dev)[:need]
         seed_sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(K + W)]
     else:   # more seeds than nodes: each batch still without repetition
-        seed_sets = [torch.randperm(w["nodes"], generator=gen, device=dev)[:B].contiguous()
+        seed_sets = [(seed_lo + torch.randperm(seed_n, generator=gen, device=dev)[:B]).contiguous()
                      for _ in range(K + W)]
 
     # N batches in flight: each pipeline owns its buffers, rank table and stream
     pipes, streams = [pipe], [torch.cuda.current_stream()]
     for _ in range(1, max(1, args.inflight)):
-        pipes.append(MiniBatchPipeline(graph, store, B, hops, replace=args.replace,
-                                       fused=args.driver != "unfused", use_graph=args.driver == "graph"))
+        pipes.append(make_pipe(args.driver == "graph"))
         streams.append(torch.cuda.Stream())
     torch.cuda.synchronize()
 
@@ -173,9 +214,10 @@ def main():
         t_gather += e1.elapsed_time(e2)
         sizes = stage_pipe.sizes.cpu().tolist()
         edges += sizes[-1]
-        rows += sizes[len(hops)]
+        rows += sizes[len(hops)] if requests is None else int(stage_pipe.request_sizes[0].item())
         hop_sizes.append(sizes[:-1])
     assert all(int(p.misses.item()) == 0 for p in pipes) and int(stage_pipe.misses.item()) == 0
+    request_sizes = None if requests is None else stage_pipe.request_sizes.cpu().tolist()
     bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
@@ -195,8 +237,16 @@ def main():
             h_feats = feats.view(torch.int16).cpu().numpy().view(np.uint16)
         else:
             h_feats = feats.cpu().numpy()
-        og = orc.Graph(h_indptr, h_indices)
-        ofs = orc.FeatStore(h_feats)
+        to_np = lambda t: (t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype == torch.bfloat16
+                           else t.cpu().numpy())
+        if requests is None:
+            og = orc.Graph(h_indptr, h_indices)
+            ofs = orc.FeatStore(h_feats)
+        else:
+            h_pos = pos_map.cpu().numpy()
+            og = orc.Graph(h_indptr, h_indices, row_begin=lo, num_total_nodes=N)
+            ofs = orc.FeatStore(h_feats, to_np(cache), h_pos)
+            h_mv, h_rw = min_vids.cpu().numpy(), requests["remote_worker_map"].cpu().numpy()
         h_seeds = [s.cpu().numpy() for s in seed_sets[W:]]
         cpu_edges = cpu_batches = 0
         tc = 0.0
@@ -206,7 +256,11 @@ def main():
             key = args.seed + 100 + W + cpu_batches
             t1 = time.perf_counter()
             inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
-            orc.gather_rows(ofs, inp)
+            if requests is None:
+                orc.gather_rows(ofs, inp)
+            else:
+                bs, _, so, _ = orc.cluster_reqs(inp, h_pos, h_rw, h_mv, P, P)
+                orc.gather_rows(ofs, so[:bs[0]])
             tc += time.perf_counter() - t1
             cpu_edges += sum(int(b["counts"].sum()) for b in blocks)
             cpu_batches += 1
@@ -234,7 +288,7 @@ def main():
                         f"(max degree {max_deg}), features {w['dim']} x {w['dtype']}, batch {B}, "
                         f"fan_out {w['fan_out']} (hops from the seeds: {hops}), "
                         f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
-                        f"gather of all input nodes",
+                        f"gather of all input nodes" + part_note,
             "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver, "batches_in_flight": len(pipes),
         },
         "roofline": {
@@ -257,6 +311,7 @@ def main():
             "gather_ms": t_gather / K,
             "sample_relabel_edges_per_s": edges / (t_sample * 1e-3),
             "frontier_sizes_last_step": hop_sizes[-1],
+            "request_bucket_sizes_last_step": request_sizes,
             "setup_s": t_setup,
         },
     }
