@@ -58,6 +58,8 @@ SYMBOLS = {
     "apt_minibatch_sample": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                   _SZ, _P]),
+    "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
+    "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
@@ -399,3 +401,51 @@ def synth_copy(src, dst):
         raise AptError("synth_copy: size mismatch")
     check(lib().apt_synth_copy(_ptr(src), _ptr(dst), nbytes, _stream()))
     return dst
+
+
+def _feat2d(t, name):
+    if not (t.is_cuda and t.is_contiguous() and t.dim() == 2 and t.dtype in (torch.float32, torch.bfloat16)):
+        raise TypeError(f"{name} must be a contiguous 2-D fp32 or bf16 GPU tensor")
+    return t
+
+
+def _segments(coo_offset, num_edges, device):
+    if coo_offset is None:
+        coo_offset = torch.tensor([0, num_edges], dtype=torch.int64, device=device)
+    return _dev_i64(coo_offset, "coo_offset")
+
+
+def spmm_sum(mode, row, col, x, num_out, edata=None, coo_offset=None, input_offset=None,
+             output_offset=None):
+    """mode 0 copy_u, 1 copy_e, 2 u_mul_e -> fp32 [num_out, dim] (see apt_spmm_sum)."""
+    row, col, x = _dev_i64(row, "row"), _dev_i64(col, "col"), _feat2d(x, "input")
+    if edata is not None:
+        edata = _feat2d(edata, "edata")
+        if edata.dtype != x.dtype or edata.shape != (row.numel(), x.shape[1]):
+            raise AptError("spmm_sum: edata must be [E, dim] of the input dtype")
+    if mode == 1 and x.shape[0] != row.numel():
+        raise AptError("spmm_sum: copy_e needs one input row per edge")
+    if row.numel() != col.numel():
+        raise AptError("spmm_sum: row and col differ in length")
+    coo = _segments(coo_offset, row.numel(), x.device)
+    out = torch.zeros((num_out, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().apt_spmm_sum(int(mode), _ptr(row), _ptr(col), row.numel(), _ptr(x), x.shape[0], _ptr(edata),
+                             x.shape[1], x.element_size(), _ptr(coo), _ptr(_dev_i64(input_offset, "input_offset")),
+                             _ptr(_dev_i64(output_offset, "output_offset")), coo.numel() - 1, _ptr(out),
+                             int(num_out), _stream()))
+    return out
+
+
+def sddmm(op, row, col, lhs, rhs, coo_offset=None, lhs_offset=None, rhs_offset=None):
+    """op 0 u_add_v, 1 u_mul_v -> fp32 [E, dim] (see apt_sddmm)."""
+    row, col = _dev_i64(row, "row"), _dev_i64(col, "col")
+    lhs, rhs = _feat2d(lhs, "lhs"), _feat2d(rhs, "rhs")
+    if lhs.dtype != rhs.dtype or lhs.shape[1] != rhs.shape[1] or row.numel() != col.numel():
+        raise AptError("sddmm: lhs/rhs dtype or width mismatch")
+    coo = _segments(coo_offset, row.numel(), lhs.device)
+    out = torch.empty((row.numel(), lhs.shape[1]), dtype=torch.float32, device=lhs.device)
+    check(lib().apt_sddmm(int(op), _ptr(row), _ptr(col), row.numel(), _ptr(lhs), lhs.shape[0], _ptr(rhs),
+                          rhs.shape[0], lhs.shape[1], lhs.element_size(), _ptr(coo),
+                          _ptr(_dev_i64(lhs_offset, "lhs_offset")), _ptr(_dev_i64(rhs_offset, "rhs_offset")),
+                          coo.numel() - 1, _ptr(out), _stream()))
+    return out

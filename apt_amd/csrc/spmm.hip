@@ -1,0 +1,267 @@
+// Aggregation on sampled blocks: SpMM (sum over in-edges) and SDDMM
+// (per-edge element-wise combine) over COO.
+//
+// Replaces CopyUSumKernel / CopyESumKernel / UMulESumKernel (reference
+// src/cuda/spmm.cu:8-148) and UAddVKernel / UMulVKernel (src/cuda/sddmm.cu:8-103).
+// The reference launches a 2-D grid with one fp32 atomicAdd per (edge,
+// feature) and a binary search of coo_off per edge.  Here a wavefront owns a
+// run of consecutive edges and keeps the running sum of a destination row in
+// registers; it touches memory only when the destination changes, so for the
+// sampler's blocks (edges grouped by destination) a row is written by at most
+// two wavefronts and the result does not depend on scheduling; for arbitrary
+// edge order it degrades to the reference's atomic-per-edge behaviour.
+// u_mul_e multiplies (the reference's kernel adds, src/cuda/spmm.cu:78, and
+// has no caller).
+#include "common.hpp"
+
+namespace apt {
+
+constexpr int kAggBlock = 256;
+constexpr int kAggWaves = kAggBlock / kWave;
+constexpr int kEdgesPerWave = 64;
+constexpr int kMaxSegments = APT_MAX_BUCKETS + 1;
+
+struct AggParams {
+  const int64_t* row;       // source index per edge
+  const int64_t* col;       // destination index per edge
+  int64_t num_edges;
+  const void* in;           // [*, D] (copy_u / u_mul_e / sddmm lhs) or [E, D] (copy_e)
+  const void* edata;        // [E, D] (u_mul_e) / sddmm rhs [*, D]
+  float* out;               // spmm: [num_out, D] fp32, zero-filled; sddmm: [E, D]
+  const int64_t* coo_off;   // [num_seg + 1]
+  const int64_t* in_off;    // [num_seg] or NULL
+  const int64_t* out_off;   // [num_seg] (sddmm: rhs offsets) or NULL
+  int num_seg;
+  int64_t dim;
+  int64_t num_in_rows, num_e_rows, num_out_rows;
+};
+
+template <typename T> __device__ __forceinline__ float to_float(T v);
+template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_float<uint16_t>(uint16_t v) {  // bf16 bits
+  return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+
+// Segment of edge e: last k with coo_off[k] <= e (reference: cub::UpperBound - 1).
+__device__ __forceinline__ int segment_of(const int64_t* s_off, int num_seg, int64_t e) {
+  int k = 0;
+  while (k + 1 < num_seg && s_off[k + 1] <= e) ++k;
+  return k;
+}
+
+template <typename T, int VEC> struct Pack;
+template <> struct Pack<float, 4> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct Pack<float, 1> { typedef float type; };
+template <> struct Pack<uint16_t, 4> { typedef uint16_t type __attribute__((ext_vector_type(4))); };
+template <> struct Pack<uint16_t, 1> { typedef uint16_t type; };
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const T* base, int64_t elem, float (&v)[VEC]) {
+  using P = typename Pack<T, VEC>::type;
+  const P raw = *reinterpret_cast<const P*>(base + elem);
+  if constexpr (VEC == 1) {
+    v[0] = to_float<T>(raw);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = to_float<T>(raw[i]);
+  }
+}
+
+// MODE 0: copy_u  acc += in[in_off + src]
+// MODE 1: copy_e  acc += in[e]
+// MODE 2: u_mul_e acc += in[in_off + src] * edata[e]
+// A lane owns VEC consecutive features; kUnroll edges are loaded before they
+// are accumulated.
+template <typename T, int MODE, int VEC>
+__global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
+  constexpr int kUnroll = 4;
+  __shared__ int64_t s_off[kMaxSegments + 1];
+  __shared__ int64_t s_in[kMaxSegments], s_out[kMaxSegments];
+  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off[threadIdx.x];
+  if (threadIdx.x < p.num_seg) {
+    s_in[threadIdx.x] = p.in_off != nullptr ? p.in_off[threadIdx.x] : 0;
+    s_out[threadIdx.x] = p.out_off != nullptr ? p.out_off[threadIdx.x] : 0;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x % kWave;
+  const int64_t wave = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave;
+  const int64_t e0 = wave * kEdgesPerWave;
+  if (e0 >= p.num_edges) return;
+  const int64_t e1 = min(e0 + kEdgesPerWave, p.num_edges);
+  const T* in = static_cast<const T*>(p.in);
+  const T* ed = static_cast<const T*>(p.edata);
+  for (int64_t d0 = 0; d0 < p.dim; d0 += kWave * VEC) {
+    const int64_t d = d0 + static_cast<int64_t>(lane) * VEC;
+    const bool live = d < p.dim;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    int64_t cur = -1;
+    auto flush = [&]() {
+      if (cur >= 0 && cur < p.num_out_rows && live) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) atomicAdd(&p.out[cur * p.dim + d + i], acc[i]);
+      }
+    };
+    for (int64_t eb = e0; eb < e1; eb += kUnroll) {
+      float v[kUnroll][VEC];
+      int64_t dst[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int64_t e = eb + u;
+        dst[u] = -1;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[u][i] = 0.f;
+        if (e < e1) {
+          const int k = segment_of(s_off, p.num_seg, e);
+          dst[u] = s_out[k] + p.col[e];
+          if (live) {
+            if (MODE == 1) {
+              load_vec<T, VEC>(in, e * p.dim + d, v[u]);
+            } else {
+              const int64_t src = s_in[k] + p.row[e];
+              if (src >= 0 && src < p.num_in_rows) load_vec<T, VEC>(in, src * p.dim + d, v[u]);
+              if (MODE == 2) {
+                float w[VEC];
+                load_vec<T, VEC>(ed, e * p.dim + d, w);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) v[u][i] *= w[i];
+              }
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        if (eb + u < e1) {
+          if (dst[u] != cur) {
+            flush();
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+            cur = dst[u];
+          }
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) acc[i] += v[u][i];
+        }
+      }
+    }
+    flush();
+  }
+}
+
+// OP 0: lhs[src] + rhs[dst]; OP 1: lhs[src] * rhs[dst]  -> out[e]
+template <typename T, int OP>
+__global__ __launch_bounds__(kAggBlock) void sddmm_kernel(AggParams p) {
+  __shared__ int64_t s_off[kMaxSegments + 1];
+  __shared__ int64_t s_l[kMaxSegments], s_r[kMaxSegments];
+  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off[threadIdx.x];
+  if (threadIdx.x < p.num_seg) {
+    s_l[threadIdx.x] = p.in_off != nullptr ? p.in_off[threadIdx.x] : 0;
+    s_r[threadIdx.x] = p.out_off != nullptr ? p.out_off[threadIdx.x] : 0;
+  }
+  __syncthreads();
+  const T* lhs = static_cast<const T*>(p.in);
+  const T* rhs = static_cast<const T*>(p.edata);
+  const int lane = threadIdx.x % kWave;
+  const int64_t waves = static_cast<int64_t>(gridDim.x) * kAggWaves;
+  for (int64_t e = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave; e < p.num_edges;
+       e += waves) {
+    const int k = segment_of(s_off, p.num_seg, e);
+    const int64_t src = s_l[k] + p.row[e];
+    const int64_t dst = s_r[k] + p.col[e];
+    const bool ok = src >= 0 && src < p.num_in_rows && dst >= 0 && dst < p.num_e_rows;
+    for (int64_t d = lane; d < p.dim; d += kWave) {
+      float v = 0.f;
+      if (ok) {
+        const float a = to_float<T>(lhs[src * p.dim + d]);
+        const float b = to_float<T>(rhs[dst * p.dim + d]);
+        v = OP == 0 ? a + b : a * b;
+      }
+      p.out[e * p.dim + d] = v;
+    }
+  }
+}
+
+static int agg_check(const char* who, const int64_t* row, const int64_t* col, int64_t E, const void* in,
+                     float* out, const int64_t* coo_off, int num_seg, int64_t dim, int elem_size) {
+  APT_REQUIRE(E >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (E %lld, dim %lld)", who, (long long)E,
+              (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "%s: elem_size %d (4 = fp32, 2 = bf16)", who,
+              elem_size);
+  APT_REQUIRE(num_seg >= 1 && num_seg <= kMaxSegments - 1, APT_ELIMIT, "%s: %d segments outside [1, %d]",
+              who, num_seg, kMaxSegments - 1);
+  APT_REQUIRE(coo_off != nullptr, APT_EINVAL, "%s: coo_offset is NULL", who);
+  APT_REQUIRE(E == 0 || (row != nullptr && col != nullptr && in != nullptr && out != nullptr), APT_EINVAL,
+              "%s: a tensor is NULL", who);
+  return APT_OK;
+}
+
+}  // namespace apt
+
+extern "C" int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+                            const void* input, int64_t num_in_rows, const void* edata, int64_t dim,
+                            int elem_size, const int64_t* coo_offset, const int64_t* input_offset,
+                            const int64_t* output_offset, int num_segments, float* out,
+                            int64_t num_out_rows, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(mode >= 0 && mode <= 2, APT_EINVAL, "apt_spmm_sum: mode %d (0 copy_u, 1 copy_e, 2 u_mul_e)", mode);
+  int rc = agg_check("apt_spmm_sum", coo_row, coo_col, num_edges, input, out, coo_offset, num_segments, dim,
+                     elem_size);
+  if (rc != APT_OK) return rc;
+  APT_REQUIRE(mode != 2 || edata != nullptr || num_edges == 0, APT_EINVAL, "apt_spmm_sum: edata is NULL");
+  APT_REQUIRE(num_out_rows >= 0 && num_in_rows >= 0, APT_EINVAL, "apt_spmm_sum: negative row count");
+  if (num_edges == 0) return APT_OK;
+  AggParams p{};
+  p.row = coo_row; p.col = coo_col; p.num_edges = num_edges; p.in = input; p.edata = edata; p.out = out;
+  p.coo_off = coo_offset; p.in_off = input_offset; p.out_off = output_offset; p.num_seg = num_segments;
+  p.dim = dim; p.num_in_rows = num_in_rows; p.num_e_rows = num_edges; p.num_out_rows = num_out_rows;
+  const int64_t waves = ceil_div(num_edges, kEdgesPerWave);
+  const dim3 grid(static_cast<unsigned>(ceil_div(waves, kAggWaves))), block(kAggBlock);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // 4 features per lane when rows are 4-element aligned
+  const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(input) & 15) == 0 &&
+                    (edata == nullptr || (reinterpret_cast<uintptr_t>(edata) & 15) == 0);
+#define APT_SPMM_LAUNCH(T, V)                                                            \
+  switch (mode) {                                                                         \
+    case 0: hipLaunchKernelGGL((spmm_kernel<T, 0, V>), grid, block, 0, st, p); break;      \
+    case 1: hipLaunchKernelGGL((spmm_kernel<T, 1, V>), grid, block, 0, st, p); break;      \
+    default: hipLaunchKernelGGL((spmm_kernel<T, 2, V>), grid, block, 0, st, p); break;     \
+  }
+  if (elem_size == 4) {
+    if (vec4) { APT_SPMM_LAUNCH(float, 4) } else { APT_SPMM_LAUNCH(float, 1) }
+  } else {
+    if (vec4) { APT_SPMM_LAUNCH(uint16_t, 4) } else { APT_SPMM_LAUNCH(uint16_t, 1) }
+  }
+#undef APT_SPMM_LAUNCH
+  APT_LAUNCH_CHECK("spmm_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_sddmm(int op, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+                         const void* lhs, int64_t num_lhs_rows, const void* rhs, int64_t num_rhs_rows,
+                         int64_t dim, int elem_size, const int64_t* coo_offset, const int64_t* lhs_offset,
+                         const int64_t* rhs_offset, int num_segments, float* out, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(op == 0 || op == 1, APT_EINVAL, "apt_sddmm: op %d (0 u_add_v, 1 u_mul_v)", op);
+  int rc = agg_check("apt_sddmm", coo_row, coo_col, num_edges, lhs, out, coo_offset, num_segments, dim,
+                     elem_size);
+  if (rc != APT_OK) return rc;
+  APT_REQUIRE(rhs != nullptr || num_edges == 0, APT_EINVAL, "apt_sddmm: rhs is NULL");
+  if (num_edges == 0) return APT_OK;
+  AggParams p{};
+  p.row = coo_row; p.col = coo_col; p.num_edges = num_edges; p.in = lhs; p.edata = rhs; p.out = out;
+  p.coo_off = coo_offset; p.in_off = lhs_offset; p.out_off = rhs_offset; p.num_seg = num_segments;
+  p.dim = dim; p.num_in_rows = num_lhs_rows; p.num_e_rows = num_rhs_rows; p.num_out_rows = 0;
+  const dim3 grid(static_cast<unsigned>(std::min<int64_t>(ceil_div(num_edges, kAggWaves), 1 << 16))),
+      block(kAggBlock);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (elem_size == 4) {
+    if (op == 0) hipLaunchKernelGGL((sddmm_kernel<float, 0>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sddmm_kernel<float, 1>), grid, block, 0, st, p);
+  } else {
+    if (op == 0) hipLaunchKernelGGL((sddmm_kernel<uint16_t, 0>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sddmm_kernel<uint16_t, 1>), grid, block, 0, st, p);
+  }
+  APT_LAUNCH_CHECK("sddmm_kernel");
+  return APT_OK;
+}

@@ -352,6 +352,84 @@ Tensor FeatShuffle(Tensor inputs, Tensor send_offset, Tensor recv_offset, Tensor
   return out;
 }
 
+// ---------------------------------------------------------------- aggregation
+namespace {
+
+Tensor feat2d(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 &&
+                  (t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kBFloat16),
+              "npc: ", name, " must be a 2-D fp32 or bf16 GPU tensor");
+  return t.contiguous();
+}
+
+// out_num = output_offset[-1] is read on the host, as in the reference (src/spmm.cc:13).
+Tensor spmm(int mode, Tensor coo_row, Tensor coo_col, Tensor input, const Tensor* edata, Tensor coo_offset,
+            const Tensor* input_offset, Tensor output_offset) {
+  auto row = ids_on_device(coo_row, "coo_row"), col = ids_on_device(coo_col, "coo_col");
+  auto x = feat2d(input, "input");
+  auto coo = ids_on_device(coo_offset, "coo_offset");
+  auto oo = ids_on_device(output_offset, "output_offset");
+  TORCH_CHECK(coo.numel() >= 2 && oo.numel() >= coo.numel() - 1 && row.numel() == col.numel(),
+              "npc: spmm: bad offsets or edge lists");
+  const int nseg = static_cast<int>(coo.numel() - 1);
+  const int64_t out_num = oo.index({-1}).item<int64_t>();
+  Tensor io, ed;
+  if (input_offset) io = ids_on_device(*input_offset, "input_offset");
+  if (edata) {
+    ed = feat2d(*edata, "edata");
+    TORCH_CHECK(ed.scalar_type() == x.scalar_type() && ed.size(0) == row.numel() && ed.size(1) == x.size(1),
+                "npc: spmm: edata must be [E, dim] of the input dtype");
+  }
+  if (mode == 1) TORCH_CHECK(x.size(0) == row.numel(), "npc: spmm_copy_e_sum needs one input row per edge");
+  auto out = torch::zeros({out_num, x.size(1)}, x.options().dtype(torch::kFloat32));
+  check(apt_spmm_sum(mode, i64(row), i64(col), row.numel(), x.data_ptr(), x.size(0),
+                     edata ? ed.data_ptr() : nullptr, x.size(1), static_cast<int>(x.element_size()),
+                     i64(coo), input_offset ? i64(io) : nullptr, i64(oo), nseg, out.data_ptr<float>(),
+                     out_num, stream()));
+  return out.to(x.scalar_type());
+}
+
+Tensor sddmm(int op, Tensor coo_row, Tensor coo_col, Tensor lhs, Tensor rhs, Tensor coo_offset,
+             Tensor lhs_offset, Tensor rhs_offset) {
+  auto row = ids_on_device(coo_row, "coo_row"), col = ids_on_device(coo_col, "coo_col");
+  auto l = feat2d(lhs, "lhs"), r = feat2d(rhs, "rhs");
+  TORCH_CHECK(l.scalar_type() == r.scalar_type() && l.size(1) == r.size(1) && row.numel() == col.numel(),
+              "npc: sddmm: lhs/rhs mismatch");
+  auto coo = ids_on_device(coo_offset, "coo_offset");
+  auto lo = ids_on_device(lhs_offset, "lhs_offset"), ro = ids_on_device(rhs_offset, "rhs_offset");
+  TORCH_CHECK(coo.numel() >= 2 && lo.numel() >= coo.numel() - 1 && ro.numel() >= coo.numel() - 1,
+              "npc: sddmm: bad offsets");
+  auto out = torch::empty({row.numel(), l.size(1)}, l.options().dtype(torch::kFloat32));
+  check(apt_sddmm(op, i64(row), i64(col), row.numel(), l.data_ptr(), l.size(0), r.data_ptr(), r.size(0),
+                  l.size(1), static_cast<int>(l.element_size()), i64(coo), i64(lo), i64(ro),
+                  static_cast<int>(coo.numel() - 1), out.data_ptr<float>(), stream()));
+  return out.to(l.scalar_type());
+}
+
+}  // namespace
+
+// reference src/spmm.cc:9-42
+Tensor CopyUSum(Tensor coo_row, Tensor coo_col, Tensor input, Tensor coo_offset, Tensor input_offset,
+                Tensor output_offset) {
+  return spmm(0, coo_row, coo_col, input, nullptr, coo_offset, &input_offset, output_offset);
+}
+Tensor CopyESum(Tensor coo_row, Tensor coo_col, Tensor input, Tensor coo_offset, Tensor output_offset) {
+  return spmm(1, coo_row, coo_col, input, nullptr, coo_offset, nullptr, output_offset);
+}
+Tensor UMulESum(Tensor coo_row, Tensor coo_col, Tensor input, Tensor edata, Tensor coo_offset,
+                Tensor input_offset, Tensor output_offset) {
+  return spmm(2, coo_row, coo_col, input, &edata, coo_offset, &input_offset, output_offset);
+}
+// reference src/sddmm.cc:9-31
+Tensor UAddV(Tensor coo_row, Tensor coo_col, Tensor lhs, Tensor rhs, Tensor coo_offset, Tensor lhs_offset,
+             Tensor rhs_offset) {
+  return sddmm(0, coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset);
+}
+Tensor UMulV(Tensor coo_row, Tensor coo_col, Tensor lhs, Tensor rhs, Tensor coo_offset, Tensor lhs_offset,
+             Tensor rhs_offset) {
+  return sddmm(1, coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset);
+}
+
 // ---------------------------------------------------------------- peers only
 #define NPC_NEEDS_PEERS(name)                                                              \
   TORCH_CHECK(false, "npc." name " talks to other GPUs over NCCL in the reference; this " \
@@ -399,6 +477,11 @@ TORCH_LIBRARY(npc, m) {
       .def("mp_feat_shuffle_bwd", &MPFeatShuffleBwd)
       .def("shuffle_seeds", &ShuffleSeeds)
       .def("relabel_csc", &RelabelCSC)
+      .def("spmm_copy_u_sum", &CopyUSum)
+      .def("spmm_copy_e_sum", &CopyESum)
+      .def("spmm_u_mul_e_sum", &UMulESum)
+      .def("sddmm_u_add_v", &UAddV)
+      .def("sddmm_u_mul_v", &UMulV)
       // additions (no counterpart in the reference)
       .def("sample_neighbors", &SampleNeighbors)
       .def("cluster_and_permute", &ClusterAndPermuteLocal)

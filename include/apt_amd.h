@@ -268,6 +268,36 @@ int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t b
                          int64_t* const* counts, int64_t* sizes, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/* Aggregation over the COO edges of sampled blocks (optional stage).
+ * Replaces CopyUSum / CopyESum / UMulESum (src/spmm.cc:9-42, src/cuda/spmm.cu:8-148)
+ * and UAddV / UMulV (src/sddmm.cc:9-31, src/cuda/sddmm.cu:8-103).
+ *
+ * Edge e belongs to segment k = last k with coo_offset[k] <= e (the reference
+ * concatenates the blocks of several ranks; one segment = plain COO):
+ *   apt_spmm_sum  out[output_offset[k] + col[e], :] += x_e, x_e =
+ *                   mode 0 (copy_u)  input[input_offset[k] + row[e], :]
+ *                   mode 1 (copy_e)  input[e, :]
+ *                   mode 2 (u_mul_e) input[input_offset[k] + row[e], :] * edata[e, :]
+ *                 (the reference's u_mul_e kernel adds instead of multiplying,
+ *                 src/cuda/spmm.cu:78, and has no caller; the product is
+ *                 implemented).  `out` is fp32 [num_out_rows, dim] and must be
+ *                 zero on entry.
+ *   apt_sddmm     out[e, :] = lhs[lhs_offset[k] + row[e], :] (+|*) rhs[rhs_offset[k] + col[e], :]
+ *                 op 0 = u_add_v, 1 = u_mul_v; out is fp32 [num_edges, dim].
+ * elem_size 4 = fp32 inputs (the reference), 2 = bf16 inputs; accumulation and
+ * outputs are fp32.  All pointers device memory; the offset arrays have
+ * num_segments (+1 for coo_offset) entries and may be NULL for "all zero"
+ * (not coo_offset). */
+int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+                 const void* input, int64_t num_in_rows, const void* edata, int64_t dim,
+                 int elem_size, const int64_t* coo_offset, const int64_t* input_offset,
+                 const int64_t* output_offset, int num_segments, float* out,
+                 int64_t num_out_rows, void* stream);
+int apt_sddmm(int op, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+              const void* lhs, int64_t num_lhs_rows, const void* rhs, int64_t num_rhs_rows,
+              int64_t dim, int elem_size, const int64_t* coo_offset, const int64_t* lhs_offset,
+              const int64_t* rhs_offset, int num_segments, float* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

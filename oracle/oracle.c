@@ -24,6 +24,9 @@
  *   orc_cluster_*       numpy searchsorted + stable argsort closed form; the
  *                       inputs of tests/test_shuffle_seeds.cc:19-26.
  *   orc_permute/scatter numpy take / put.
+ *   orc_spmm_sum/sddmm  numpy closed forms (np.add.at over fancy-indexed rows,
+ *                       in float64); a sum over a row of ones equals its
+ *                       in-degree.
  *
  * Build: make -C oracle   (gcc -O3 -fopenmp -shared -fPIC)
  */
@@ -392,4 +395,53 @@ void orc_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* feat_pos_map
   stable_place(ids, n, bucket, num_remote_workers, bucket_size, bucket_offset,
                sorted_ids, permutation);
   free(bucket);
+}
+
+/* ------------------------------------------------------------------ */
+/* Aggregation: src/cuda/spmm.cu:8-83 (COO SpMM; segment of an edge by  */
+/* upper bound in coo_off, :21,:47,:72) and src/cuda/sddmm.cu:8-59.     */
+/* Sums are accumulated in double and rounded once, so the result is    */
+/* the correctly rounded reference for the 1e-5 tolerance; u_mul_e      */
+/* multiplies (the reference adds, spmm.cu:78; no caller).              */
+/* Pinned by numpy closed forms (np.add.at on fancy-indexed rows).      */
+/* ------------------------------------------------------------------ */
+static inline int seg_of(const int64_t* coo_off, int num_seg, int64_t e) {
+  int k = 0;
+  while (k + 1 < num_seg && coo_off[k + 1] <= e) ++k;
+  return k;
+}
+
+void orc_spmm_sum(int mode, const int64_t* row, const int64_t* col, int64_t E, const float* in,
+                  const float* edata, int64_t dim, const int64_t* coo_off, const int64_t* in_off,
+                  const int64_t* out_off, int num_seg, float* out, int64_t num_out) {
+  double* acc = (double*)calloc((size_t)(num_out > 0 ? num_out : 1) * (size_t)dim, sizeof(double));
+  for (int64_t e = 0; e < E; ++e) {
+    int k = seg_of(coo_off, num_seg, e);
+    int64_t dst = (out_off ? out_off[k] : 0) + col[e];
+    int64_t src = (in_off ? in_off[k] : 0) + row[e];
+    for (int64_t d = 0; d < dim; ++d) {
+      double v;
+      if (mode == 1) v = in[e * dim + d];
+      else if (mode == 2) v = (double)in[src * dim + d] * (double)edata[e * dim + d];
+      else v = in[src * dim + d];
+      acc[dst * dim + d] += v;
+    }
+  }
+  for (int64_t i = 0; i < num_out * dim; ++i) out[i] = (float)acc[i];
+  free(acc);
+}
+
+void orc_sddmm(int op, const int64_t* row, const int64_t* col, int64_t E, const float* lhs,
+               const float* rhs, int64_t dim, const int64_t* coo_off, const int64_t* lhs_off,
+               const int64_t* rhs_off, int num_seg, float* out) {
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+  for (int64_t e = 0; e < E; ++e) {
+    int k = seg_of(coo_off, num_seg, e);
+    int64_t src = (lhs_off ? lhs_off[k] : 0) + row[e];
+    int64_t dst = (rhs_off ? rhs_off[k] : 0) + col[e];
+    for (int64_t d = 0; d < dim; ++d) {
+      float a = lhs[src * dim + d], b = rhs[dst * dim + d];
+      out[e * dim + d] = op == 0 ? a + b : a * b;
+    }
+  }
 }

@@ -16,7 +16,7 @@ __all__ = [
     "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
     "sample_neighbors", "sample_positions", "relabel", "gather_rows",
     "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
-    "set_threads", "max_threads", "sample_blocks",
+    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm",
 ]
 
 
@@ -257,3 +257,36 @@ def sample_blocks(graph, seeds, hop_fanouts, replace, rng_seed):
                               relabeled=rel, fanout=f))
         frontier = uniq
     return frontier, blocks
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def spmm_sum(mode, row, col, x, num_out, edata=None, coo_offset=None, input_offset=None,
+             output_offset=None):
+    """mode 0 copy_u, 1 copy_e, 2 u_mul_e -> float32 [num_out, dim]."""
+    row, col, x = _i64(row), _i64(col), _f32(x)
+    E, dim = len(row), x.shape[1]
+    coo = _i64([0, E] if coo_offset is None else coo_offset)
+    nseg = len(coo) - 1
+    io = None if input_offset is None else _i64(input_offset)
+    oo = None if output_offset is None else _i64(output_offset)
+    ed = None if edata is None else _f32(edata)
+    out = np.zeros((num_out, dim), dtype=np.float32)
+    lib().orc_spmm_sum(C.c_int(mode), _p(row), _p(col), C.c_int64(E), _p(x), _p(ed), C.c_int64(dim),
+                       _p(coo), _p(io), _p(oo), C.c_int(nseg), _p(out), C.c_int64(num_out))
+    return out
+
+
+def sddmm(op, row, col, lhs, rhs, coo_offset=None, lhs_offset=None, rhs_offset=None):
+    """op 0 u_add_v, 1 u_mul_v -> float32 [E, dim]."""
+    row, col, lhs, rhs = _i64(row), _i64(col), _f32(lhs), _f32(rhs)
+    E, dim = len(row), lhs.shape[1]
+    coo = _i64([0, E] if coo_offset is None else coo_offset)
+    lo = None if lhs_offset is None else _i64(lhs_offset)
+    ro = None if rhs_offset is None else _i64(rhs_offset)
+    out = np.zeros((E, dim), dtype=np.float32)
+    lib().orc_sddmm(C.c_int(op), _p(row), _p(col), C.c_int64(E), _p(lhs), _p(rhs), C.c_int64(dim),
+                    _p(coo), _p(lo), _p(ro), C.c_int(len(coo) - 1), _p(out))
+    return out
