@@ -59,6 +59,7 @@ SYMBOLS = {
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                   _SZ, _P]),
     "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
+    "apt_spmm_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I64, _I, _I, _P, _P]),
     "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
@@ -448,4 +449,19 @@ def sddmm(op, row, col, lhs, rhs, coo_offset=None, lhs_offset=None, rhs_offset=N
                           rhs.shape[0], lhs.shape[1], lhs.element_size(), _ptr(coo),
                           _ptr(_dev_i64(lhs_offset, "lhs_offset")), _ptr(_dev_i64(rhs_offset, "rhs_offset")),
                           coo.numel() - 1, _ptr(out), _stream()))
+    return out
+
+
+def spmm_block(neighbors, num_dst, fanout, x, mean=False, num_dst_dev=None, out=None):
+    """Sum (or mean) of x rows over a sampled block in its fixed-stride layout
+    (see apt_spmm_block) -> fp32 [num_dst, dim]."""
+    neighbors = _dev_i64(neighbors, "neighbors")
+    x = _feat2d(x, "input")
+    if neighbors.numel() < num_dst * fanout:
+        raise AptError("spmm_block: neighbors shorter than num_dst * fanout")
+    if out is None:
+        out = torch.empty((num_dst, x.shape[1]), dtype=torch.float32, device=x.device)
+    check(lib().apt_spmm_block(_ptr(neighbors), int(num_dst), _ptr(num_dst_dev), int(fanout), _ptr(x),
+                               x.shape[0], x.shape[1], x.element_size(), int(bool(mean)), _ptr(out),
+                               _stream()))
     return out

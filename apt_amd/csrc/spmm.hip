@@ -182,6 +182,70 @@ __global__ __launch_bounds__(kAggBlock) void sddmm_kernel(AggParams p) {
   }
 }
 
+// Fixed-stride ("ELL") SpMM over a sampled block as the sampler emits it:
+// destination i owns slots [i*fanout, (i+1)*fanout) of `nbr`, negative = no
+// edge.  A lane group owns a destination row, so there are no atomics, no
+// zero-fill and the sum order is fixed.  LPR lanes x VEC features cover `dim`.
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kAggBlock) void spmm_ell_kernel(const int64_t* __restrict__ nbr,
+                                                             int64_t num_dst, const int64_t* num_dst_dev,
+                                                             int fanout, const T* __restrict__ x,
+                                                             int64_t num_src, int64_t dim,
+                                                             float* __restrict__ out, int mean) {
+  constexpr int kGroups = kAggBlock / LPR;
+  constexpr int kUnroll = 5;
+  const int64_t n = actual_count(num_dst, num_dst_dev);
+  const int grp = threadIdx.x / LPR, l = threadIdx.x % LPR;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kGroups + grp; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kGroups) {
+    const int64_t* ids = nbr + i * fanout;
+    for (int64_t d = static_cast<int64_t>(l) * VEC; d < dim; d += LPR * VEC) {
+      float acc[VEC];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
+      int cnt = 0;
+      for (int s0 = 0; s0 < fanout; s0 += kUnroll) {
+        float v[kUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) v[u][k] = 0.f;
+          if (s0 + u < fanout) {
+            const int64_t src = ids[s0 + u];
+            if (src >= 0 && src < num_src) {
+              load_vec<T, VEC>(x, src * dim + d, v[u]);
+              ++cnt;
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) acc[k] += v[u][k];
+      }
+      const float scale = (mean && cnt > 0) ? 1.0f / static_cast<float>(cnt) : 1.0f;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) out[i * dim + d + k] = acc[k] * scale;
+    }
+  }
+}
+
+template <typename T, int VEC>
+static void launch_ell(const int64_t* nbr, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+                       const void* x, int64_t num_src, int64_t dim, float* out, int mean, hipStream_t st) {
+  const int64_t per_row = ceil_div(dim, VEC);
+  const T* xt = static_cast<const T*>(x);
+#define APT_ELL(LPR)                                                                                 \
+  hipLaunchKernelGGL((spmm_ell_kernel<T, VEC, LPR>),                                                  \
+                     dim3(static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst, kAggBlock / LPR), 1 << 20))), \
+                     dim3(kAggBlock), 0, st, nbr, num_dst, num_dst_dev, fanout, xt, num_src, dim, out, mean)
+  if (per_row <= 8) APT_ELL(8);
+  else if (per_row <= 16) APT_ELL(16);
+  else if (per_row <= 32) APT_ELL(32);
+  else APT_ELL(64);
+#undef APT_ELL
+}
+
 static int agg_check(const char* who, const int64_t* row, const int64_t* col, int64_t E, const void* in,
                      float* out, const int64_t* coo_off, int num_seg, int64_t dim, int elem_size) {
   APT_REQUIRE(E >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (E %lld, dim %lld)", who, (long long)E,
@@ -263,5 +327,31 @@ extern "C" int apt_sddmm(int op, const int64_t* coo_row, const int64_t* coo_col,
     else hipLaunchKernelGGL((sddmm_kernel<uint16_t, 1>), grid, block, 0, st, p);
   }
   APT_LAUNCH_CHECK("sddmm_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_spmm_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_dst_dev,
+                              int fanout, const void* input, int64_t num_src, int64_t dim, int elem_size,
+                              int mean, float* out, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_dst >= 0 && fanout > 0 && dim > 0 && num_src >= 0, APT_EINVAL,
+              "apt_spmm_block: bad shape (num_dst %lld, fanout %d, dim %lld)", (long long)num_dst, fanout,
+              (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_spmm_block: elem_size %d (4 = fp32, 2 = bf16)",
+              elem_size);
+  if (num_dst == 0) return APT_OK;
+  APT_REQUIRE(neighbors != nullptr && out != nullptr && (input != nullptr || num_src == 0), APT_EINVAL,
+              "apt_spmm_block: a tensor is NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(input) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (elem_size == 4) {
+    if (vec4) launch_ell<float, 4>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+    else launch_ell<float, 1>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+  } else {
+    if (vec4) launch_ell<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+    else launch_ell<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+  }
+  APT_LAUNCH_CHECK("spmm_ell_kernel");
   return APT_OK;
 }

@@ -128,5 +128,27 @@ class NPFeatureShuffle(torch.autograd.Function):
                                   fsi.permutation, fsi.feat_dim, 0)
 
 
+# ---------------------------------------------------------------- aggregation
+def spmm_copy_u_sum(coo_row, coo_col, input, coo_offset, input_offset, output_offset):
+    """reference src/spmm.cc:9-19 (python/npc/model/sageconv.py:105)"""
+    return _npc.spmm_copy_u_sum(coo_row, coo_col, input, coo_offset, input_offset, output_offset)
+
+
+def spmm_copy_e_sum(coo_row, coo_col, input, coo_offset, output_offset):
+    return _npc.spmm_copy_e_sum(coo_row, coo_col, input, coo_offset, output_offset)
+
+
+def spmm_u_mul_e_sum(coo_row, coo_col, input, edata, coo_offset, input_offset, output_offset):
+    return _npc.spmm_u_mul_e_sum(coo_row, coo_col, input, edata, coo_offset, input_offset, output_offset)
+
+
+def sddmm_u_add_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset):
+    return _npc.sddmm_u_add_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset)
+
+
+def sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset):
+    return _npc.sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset)
+
+
 def np_sample_and_shuffle(seeds, fanout):
     return _npc.np_sample_and_shuffle(seeds, fanout)

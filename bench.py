@@ -59,6 +59,9 @@ def parse_args():
     ap.add_argument("--calibration_copy_mib", type=int, default=0,
                     help="also launch the plain copy kernel once on this many MiB (for scaling "
                          "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
+    ap.add_argument("--aggregation", action="store_true",
+                    help="also time GraphSAGE-style SpMM (hidden 256, fp32 and bf16) and SDDMM on the "
+                         "outermost sampled block of the last batch")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
@@ -222,6 +225,63 @@ def main():
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
 
+    # ---- optional aggregation stage on the outermost block of the last batch
+    agg = None
+    if args.aggregation:
+        res = stage_pipe.result()
+        blk = res["blocks"][0]
+        rel = blk["relabeled"]
+        f = blk["fanout"]
+        col_all = torch.arange(blk["seeds"].numel(), device=dev).repeat_interleave(f)
+        keep = rel >= 0
+        row_e, col_e = rel[keep].contiguous(), col_all[keep].contiguous()
+        n_src, n_dst, E, hid = blk["unique"].numel(), blk["seeds"].numel(), int(keep.sum()), 256
+        agg = {"edges": E, "num_src": n_src, "num_dst": n_dst, "hidden": hid}
+        for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+            h = synth.random_features(n_src, hid, dt, args.seed + 7, dev)
+            fn = lambda: capi.spmm_sum(0, row_e, col_e, h, n_dst)
+            for _ in range(3):
+                fn()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(10):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) / 10 * 1e-3
+            nbytes = E * hid * es + 2 * n_dst * hid * 4 + 16 * E   # rows read, zero-fill + sums written, ids
+            agg[f"spmm_copy_u_sum_{name}_us"] = t * 1e6
+            agg[f"spmm_copy_u_sum_{name}_GBps"] = nbytes / t / 1e9
+            # the same sum (as a mean) straight from the sampler's fixed-stride block layout
+            fn = lambda: capi.spmm_block(rel, n_dst, f, h, mean=True)
+            for _ in range(3):
+                fn()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(10):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) / 10 * 1e-3
+            nbytes = E * hid * es + n_dst * hid * 4 + 8 * n_dst * f
+            agg[f"spmm_block_mean_{name}_us"] = t * 1e6
+            agg[f"spmm_block_mean_{name}_GBps"] = nbytes / t / 1e9
+        hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
+        h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)
+        fn = lambda: capi.sddmm(0, row_e, col_e, h, hd)
+        for _ in range(3):
+            fn()
+        e0, e1 = ev(), ev()
+        e0.record()
+        for _ in range(10):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / 10 * 1e-3
+        agg["sddmm_u_add_v_fp32_us"] = t * 1e6
+        agg["sddmm_u_add_v_fp32_GBps"] = (3 * E * hid * 4 + 16 * E) / t / 1e9
+        del h, hd
+
     # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
     cpu = None
     budget = args.cpu_seconds
@@ -303,6 +363,7 @@ def main():
             "avg_launch_us": t_gather / K * 1e3,
         },
         "cpu_baseline": cpu,
+        "aggregation": agg,
         "stages": {
             "single_stream_ms_per_step": single_stream_ms,
             "edges_per_step": edges / K,

@@ -293,6 +293,17 @@ int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo_col, int64
                  int elem_size, const int64_t* coo_offset, const int64_t* input_offset,
                  const int64_t* output_offset, int num_segments, float* out,
                  int64_t num_out_rows, void* stream);
+/* SpMM over a sampled block in the layout the sampler and relabel emit
+ * (apt_sample_neighbors / apt_relabel / apt_minibatch_sample): destination i
+ * owns slots [i * fanout, (i+1) * fanout) of `neighbors` (compact source ids,
+ * negative = no edge).  out[i, :] = sum (mean != 0: mean over the valid slots)
+ * of input[neighbors[slot], :].  Same result as apt_spmm_sum mode 0 on the
+ * block's COO (reference CopyUSum + the division by the fanout that
+ * python/npc/model/sageconv.py:173-174 does), without atomics or zero-fill.
+ * num_dst_dev: optional device int64[1] (as in apt_sample_neighbors). */
+int apt_spmm_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_dst_dev,
+                   int fanout, const void* input, int64_t num_src, int64_t dim, int elem_size,
+                   int mean, float* out, void* stream);
 int apt_sddmm(int op, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
               const void* lhs, int64_t num_lhs_rows, const void* rhs, int64_t num_rhs_rows,
               int64_t dim, int elem_size, const int64_t* coo_offset, const int64_t* lhs_offset,

@@ -102,3 +102,26 @@ def test_aggregation_operators(orc, capi):
     assert _close(out.cpu().numpy(), orc.spmm_sum(0, row, col, x, 1000), 1e-5)
     out = torch.ops.npc.sddmm_u_add_v(dev(row), dev(col), dev(x), dev(y), coo, zero, zero)
     assert np.array_equal(out.cpu().numpy(), orc.sddmm(0, row, col, x, y))
+
+
+@pytest.mark.parametrize("dim,dtype", [(256, torch.float32), (256, torch.bfloat16), (64, torch.float32),
+                                       (100, torch.float32), (7, torch.float32), (1000, torch.float32)])
+def test_spmm_block_layout(orc, capi, dim, dtype):
+    """The sampler's padded block layout, sum and mean, vs the COO oracle."""
+    rng = np.random.default_rng(dim)
+    n_dst, n_src, f = 3000, 20000, 15
+    nbr = rng.integers(0, n_src, size=(n_dst, f))
+    cnt = rng.integers(0, f + 1, size=n_dst)
+    nbr[np.arange(f)[None, :] >= cnt[:, None]] = -1                  # ragged rows, some empty
+    x = torch.from_numpy(rng.standard_normal((n_src, dim)).astype(np.float32)).to(DEV).to(dtype)
+    xh = x.float().cpu().numpy()
+    col = np.repeat(np.arange(n_dst), f)
+    keep = nbr.reshape(-1) >= 0
+    want = orc.spmm_sum(0, nbr.reshape(-1)[keep], col[keep], xh, n_dst)
+    got = capi.spmm_block(dev(nbr.reshape(-1)), n_dst, f, x)
+    assert _close(got.cpu().numpy(), want, 1e-5)
+    got_mean = capi.spmm_block(dev(nbr.reshape(-1)), n_dst, f, x, mean=True)
+    assert _close(got_mean.cpu().numpy(), want / np.maximum(cnt, 1)[:, None], 1e-5)
+    assert np.all(got.cpu().numpy()[cnt == 0] == 0)
+    a = capi.spmm_block(dev(nbr.reshape(-1)), n_dst, f, x)
+    assert torch.equal(a, got)                                       # fixed summation order
