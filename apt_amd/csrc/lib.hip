@@ -14,10 +14,14 @@ char* last_error_buf() {
 static int g_sample_lanes = 0;
 static int g_gather_rows = 0;
 static int g_gather_max_blocks = 0;
+static int g_fuse_mark = 1;
+static int g_payload_bits = 0;
 
 int tuning_sample_lanes() { return g_sample_lanes; }
 int tuning_gather_rows() { return g_gather_rows; }
 int tuning_gather_max_blocks() { return g_gather_max_blocks; }
+int tuning_fuse_mark() { return g_fuse_mark; }
+int tuning_payload_bits() { return g_payload_bits; }
 
 }  // namespace apt
 
@@ -37,6 +41,15 @@ extern "C" int apt_set_tuning(const char* key, int value) {
     if (value != 0 && value != 1 && value != 2 && value != 4 && value != 8)
       return apt::fail(APT_EINVAL, "apt_set_tuning: gather_rows_in_flight must be 0, 1, 2, 4 or 8");
     apt::g_gather_rows = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "minibatch_payload_bits") == 0) {
+    if (value < 0 || value > 31) return apt::fail(APT_EINVAL, "apt_set_tuning: minibatch_payload_bits must be 0..31");
+    apt::g_payload_bits = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "minibatch_fuse_mark") == 0) {
+    apt::g_fuse_mark = value != 0;
     return APT_OK;
   }
   if (std::strcmp(key, "gather_max_blocks") == 0) {

@@ -22,16 +22,33 @@
 // Random atomics are the scarcest resource on this GPU (~20 G/s against
 // ~45 G/s random loads), which is why the table is indexed directly (no CAS
 // to claim a slot, no probing) and why nodes already present never touch one.
-// The table is restored to all-0xFFFFFFFF before the call returns control of
-// the stream, by walking the final node list.
+// Nothing is ever cleared per batch: an entry is (epoch << P) | payload, P =
+// bits needed for the largest id of the plan, and every call uses the next
+// lower epoch, so the entries of earlier batches (larger epochs, or the
+// all-ones fill) compare greater than anything the current batch writes and an
+// atomicMin overrides them without being told.  The epoch lives in device
+// memory next to the table, so a captured HIP graph replays correctly; when
+// the epochs run out (every 2^(32-P) - 1 calls) the table is refilled.
+// On the last hop the owners' ids are not even written to the table: the few
+// slots that lost a race fetch the id from the winner's output slot instead.
 #include "common.hpp"
 
 namespace apt {
 
+struct SampleMark {  // fused relabel marking inside the sampling kernel (sample.hip)
+  uint32_t* table;
+  int64_t table_len;
+  const uint32_t* state;
+  int64_t* relabeled;
+  int first_hop;
+};
+
 int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
                   const int64_t* num_frontier_dev, int fanout, int replace, uint64_t rng_seed,
                   const uint64_t* rng_seed_dev, int hop, int64_t* out_neighbors, int64_t* out_counts,
-                  int64_t* out_total, hipStream_t st, const char* who);
+                  int64_t* out_total, hipStream_t st, const char* who, const SampleMark* mark);
+
+int tuning_fuse_mark();  // 1 (default) = mark inside the sampling kernel
 
 constexpr int kMbBlock = 256;
 constexpr int kMbIters = 4;
@@ -50,6 +67,8 @@ struct HopParams {
   int64_t* relabeled;        // [ns_cap * fanout]
   uint32_t* table;
   int64_t table_len;
+  const uint32_t* state;     // [0] epoch, [1] payload bits, [2] refill request
+  int last;                  // last hop: ids are not written back to the table
   int64_t* nodes;            // growing unique list
   int64_t* n_next;           // receives the size of the list after this hop
   uint64_t* flags;           // owner bit per item, one word per wavefront-load
@@ -71,6 +90,36 @@ __device__ __forceinline__ bool in_table(const HopParams& p, int64_t v) {
   return v >= 0 && v < p.table_len;
 }
 
+// Smallest table value of the current batch: (epoch << payload bits).
+__device__ __forceinline__ uint32_t table_base(const uint32_t* state) {
+  return state[0] << state[1];
+}
+
+// One thread: next epoch, or a refill request when the epochs are used up or
+// the table was last used with another payload width.
+__global__ void mb_begin_kernel(uint32_t* state, uint32_t payload_bits) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const uint32_t top = (1u << (32 - payload_bits)) - 1;  // all-ones epoch = the fill value
+  if (state[1] != payload_bits || state[0] == 0 || state[0] > top - 1) {
+    state[0] = top - 1;
+    state[1] = payload_bits;
+    state[2] = 1;
+  } else {
+    state[0] -= 1;
+    state[2] = 0;
+  }
+}
+
+// Refill, only when mb_begin_kernel asked for it.
+__global__ __launch_bounds__(kMbBlock) void mb_refill_kernel(uint4* table, int64_t vecs,
+                                                             const uint32_t* state) {
+  if (state[2] == 0) return;
+  const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
+       i += static_cast<int64_t>(gridDim.x) * kMbBlock)
+    table[i] = ones;
+}
+
 // First hop only: seeds may repeat, so they race like everything else; the
 // smallest seed index owns the node.  Also clears the per-batch counters.
 __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, int64_t* sizes,
@@ -79,7 +128,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, in
   if (i < num_sizes) sizes[i] = i == 0 ? p.ns_cap : 0;
   if (i < p.ns_cap) {
     const int64_t v = p.seeds[i];
-    if (in_table(p, v)) atomicMin(&p.table[v], static_cast<uint32_t>(i));
+    if (in_table(p, v)) atomicMin(&p.table[v], table_base(p.state) + static_cast<uint32_t>(i));
   }
 }
 
@@ -89,6 +138,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, in
 template <bool FIRST>
 __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p) {
   const HopSizes s = hop_sizes(p);
+  const uint32_t tb = table_base(p.state);
   for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < s.nn;
        j += static_cast<int64_t>(gridDim.x) * kMbBlock) {
     const int64_t v = p.neighbors[j];
@@ -96,10 +146,10 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p
     if (!in_table(p, v)) {
       out = v < 0 ? v : -1;  // padding, or an id the table cannot hold: no edge
     } else {
-      const uint32_t bid = static_cast<uint32_t>(s.ns + j);
+      const uint32_t bid = tb + static_cast<uint32_t>(s.ns + j);
       // Values only decrease, so a stale read can only cause a redundant atomic.
       const uint32_t cur = p.table[v];
-      if (!FIRST && cur < static_cast<uint32_t>(s.ns)) out = cur;
+      if (!FIRST && cur < tb + static_cast<uint32_t>(s.ns)) out = cur - tb;
       else if (cur > bid) atomicMin(&p.table[v], bid);
     }
     p.relabeled[j] = out;
@@ -123,7 +173,7 @@ __device__ __forceinline__ bool mb_is_owner(const HopParams& p, const HopSizes& 
     v = p.neighbors[i];
     bid = static_cast<uint32_t>(s.ns + i);
   }
-  return p.table[v] == bid;
+  return p.table[v] == table_base(p.state) + bid;
 }
 
 template <bool FIRST>
@@ -206,7 +256,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
         p.relabeled[i] = id;
       }
       p.nodes[id] = v;
-      p.table[v] = static_cast<uint32_t>(id);
+      if (!p.last) p.table[v] = table_base(p.state) + static_cast<uint32_t>(id);
     }
   }
   if (blockIdx.x == tiles - 1 && threadIdx.x == 0) *p.n_next = running;
@@ -221,6 +271,8 @@ struct LookupParams {
   int64_t ns_cap[kMaxHops];
   int64_t fanout[kMaxHops];
   const uint32_t* table;
+  const uint32_t* state;
+  int last_is_bid;  // the last hop's table entries are still bids (see HopParams::last)
 };
 
 // Slots that lost the ownership race read the winner's id (all hops at once).
@@ -229,20 +281,20 @@ __global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
   while (h + 1 < p.num_hops && static_cast<int64_t>(blockIdx.x) >= p.block_begin[h + 1]) ++h;
   const int64_t nn = actual_count(p.ns_cap[h], p.ns_dev[h]) * p.fanout[h];
   const int64_t blocks = p.block_begin[h + 1] - p.block_begin[h];
+  const uint32_t tb = table_base(p.state);
+  const bool via_owner = p.last_is_bid && h == p.num_hops - 1;
+  const int64_t ns = actual_count(p.ns_cap[h], p.ns_dev[h]);
   for (int64_t j = (static_cast<int64_t>(blockIdx.x) - p.block_begin[h]) * kMbBlock + threadIdx.x;
        j < nn; j += blocks * kMbBlock) {
-    if (p.relabeled[h][j] == kPending) p.relabeled[h][j] = p.table[p.neighbors[h][j]];
+    if (p.relabeled[h][j] != kPending) continue;
+    const int64_t e = p.table[p.neighbors[h][j]] - tb;
+    // via_owner: e is the winning bid ns + slot; the winner's slot holds the id
+    // (it is an owner, so its slot is final and never pending).
+    p.relabeled[h][j] = via_owner ? p.relabeled[h][e - ns] : e;
   }
 }
 
-// table[v] := empty for every node of the batch.
-__global__ __launch_bounds__(kMbBlock) void mb_reset_kernel(uint32_t* table, const int64_t* nodes,
-                                                            const int64_t* n_dev, int64_t n_cap) {
-  const int64_t n = actual_count(n_cap, n_dev);
-  for (int64_t r = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; r < n;
-       r += static_cast<int64_t>(gridDim.x) * kMbBlock)
-    table[nodes[r]] = kEmpty;
-}
+__global__ void mb_zero_state_kernel(uint32_t* state) { state[threadIdx.x] = 0; }
 
 __global__ __launch_bounds__(kMbBlock) void mb_fill_table_kernel(uint4* table, int64_t vecs) {
   const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
@@ -257,7 +309,14 @@ struct MbLayout {
   size_t flags_off, tile_off, total;
   int64_t caps[kMaxHops + 1];
   int64_t max_items;
+  uint32_t payload_bits;  // ids and bids of the plan are < 2^payload_bits
 };
+
+int tuning_payload_bits();  // 0 = as few as the plan needs
+
+static size_t table_state_offset(int64_t table_len) {
+  return (static_cast<size_t>(table_len) * sizeof(uint32_t) + 255) / 256 * 256;
+}
 
 static bool mb_layout(int64_t batch, const int* fanouts, int num_hops, MbLayout& L) {
   L.caps[0] = batch;
@@ -270,6 +329,10 @@ static bool mb_layout(int64_t batch, const int* fanouts, int num_hops, MbLayout&
     const int64_t items = h == 0 ? L.caps[h] * (1 + f) : L.caps[h] * f;
     if (items > L.max_items) L.max_items = items;
   }
+  L.payload_bits = 1;
+  while ((int64_t{1} << L.payload_bits) < L.caps[num_hops] + 1) ++L.payload_bits;
+  if (tuning_payload_bits() > static_cast<int>(L.payload_bits) && tuning_payload_bits() <= 31)
+    L.payload_bits = static_cast<uint32_t>(tuning_payload_bits());
   const int64_t tiles = ceil_div(L.max_items, kMbTile);
   size_t off = 0;
   L.flags_off = off; off = mb_align(off + sizeof(uint64_t) * tiles * kMbIters * kMbWaves);
@@ -282,16 +345,21 @@ static bool mb_layout(int64_t batch, const int* fanouts, int num_hops, MbLayout&
 
 extern "C" size_t apt_rank_table_bytes(int64_t num_total_nodes) {
   if (num_total_nodes < 0 || num_total_nodes >= (int64_t{1} << 32) - 1) return 0;
-  return (static_cast<size_t>(num_total_nodes) * sizeof(uint32_t) + 255) / 256 * 256;
+  return apt::table_state_offset(num_total_nodes) + 256;  // entries + epoch state
 }
 
 extern "C" int apt_rank_table_init(void* table, size_t table_bytes, void* stream) {
   using namespace apt;
-  APT_REQUIRE(table != nullptr && table_bytes % 16 == 0 &&
-                  (reinterpret_cast<uintptr_t>(table) & 15) == 0,
-              APT_EINVAL, "apt_rank_table_init: table must be 16-byte aligned and sized");
-  if (table_bytes == 0) return APT_OK;
-  const int64_t vecs = static_cast<int64_t>(table_bytes / 16);
+  APT_REQUIRE(table != nullptr && table_bytes >= 256 && table_bytes % 256 == 0 &&
+                  (reinterpret_cast<uintptr_t>(table) & 255) == 0,
+              APT_EINVAL, "apt_rank_table_init: table must be 256-byte aligned and sized by "
+                          "apt_rank_table_bytes");
+  // entries all-ones; the trailing state block all-zero (epoch 0 = "start over")
+  hipLaunchKernelGGL(mb_zero_state_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     reinterpret_cast<uint32_t*>(static_cast<char*>(table) + table_bytes - 256));
+  APT_LAUNCH_CHECK("mb_zero_state_kernel");
+  if (table_bytes == 256) return APT_OK;
+  const int64_t vecs = static_cast<int64_t>((table_bytes - 256) / 16);
   const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(vecs, kMbBlock), 16384));
   hipLaunchKernelGGL(mb_fill_table_kernel, dim3(blocks), dim3(kMbBlock), 0,
                      static_cast<hipStream_t>(stream), static_cast<uint4*>(table), vecs);
@@ -343,9 +411,22 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   char* ws = static_cast<char*>(workspace);
   int64_t* total = sizes + num_hops + 1;
 
+  uint32_t* state = reinterpret_cast<uint32_t*>(static_cast<char*>(rank_table) +
+                                                table_state_offset(rank_table_len));
+  // next epoch (or a refill once they are used up)
+  hipLaunchKernelGGL(mb_begin_kernel, dim3(1), dim3(64), 0, st, state, L.payload_bits);
+  APT_LAUNCH_CHECK("mb_begin_kernel");
+  {
+    const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
+    hipLaunchKernelGGL(mb_refill_kernel, dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(vecs, kMbBlock), 4096)))),
+                       dim3(kMbBlock), 0, st, static_cast<uint4*>(rank_table), vecs, state);
+    APT_LAUNCH_CHECK("mb_refill_kernel");
+  }
+
   HopParams hp{};
   hp.table = static_cast<uint32_t*>(rank_table);
   hp.table_len = rank_table_len;
+  hp.state = state;
   hp.nodes = nodes;
   hp.flags = reinterpret_cast<uint64_t*>(ws + L.flags_off);
   hp.tile_cnt = reinterpret_cast<uint32_t*>(ws + L.tile_off);
@@ -371,9 +452,13 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     const int64_t nn_cap = ns_cap * f;
     const int64_t* frontier = h == 0 ? seeds : nodes;
     const int64_t* ns_dev = h == 0 ? nullptr : sizes + h;
+    // The sampling kernel looks every id up in the rank table as soon as it has
+    // loaded it (fanouts up to one wavefront); otherwise a separate pass does.
+    const bool fuse = f <= kWave && tuning_fuse_mark() != 0;
+    SampleMark mark{static_cast<uint32_t*>(rank_table), rank_table_len, state, relabeled[h], h == 0 ? 1 : 0};
     int rc = sample_launch(graph, frontier, ns_cap, ns_dev, static_cast<int>(f), replace, rng_seed,
                            rng_seed_dev, h, neighbors[h], counts != nullptr ? counts[h] : nullptr,
-                           total, st, "apt_minibatch_sample");
+                           total, st, "apt_minibatch_sample", fuse ? &mark : nullptr);
     if (rc != APT_OK) return rc;
     hp.ns_cap = ns_cap;
     hp.ns_dev = ns_dev;
@@ -381,19 +466,24 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     hp.neighbors = neighbors[h];
     hp.relabeled = relabeled[h];
     hp.n_next = sizes + h + 1;
+    hp.last = (h == num_hops - 1 && h > 0) ? 1 : 0;
     const int64_t items_cap = h == 0 ? ns_cap + nn_cap : nn_cap;
     const dim3 tiles = grid_for(items_cap, kMbTile, int64_t{1} << 30);
     const dim3 flat = grid_for(nn_cap, kMbBlock, 1 << 16);
     if (h == 0) {
-      hipLaunchKernelGGL(mb_mark_neighbors_kernel<true>, flat, dim3(kMbBlock), 0, st, hp);
-      APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      if (!fuse) {
+        hipLaunchKernelGGL(mb_mark_neighbors_kernel<true>, flat, dim3(kMbBlock), 0, st, hp);
+        APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      }
       hipLaunchKernelGGL(mb_count_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
       APT_LAUNCH_CHECK("mb_count_kernel");
       hipLaunchKernelGGL(mb_place_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
       APT_LAUNCH_CHECK("mb_place_kernel");
     } else {
-      hipLaunchKernelGGL(mb_mark_neighbors_kernel<false>, flat, dim3(kMbBlock), 0, st, hp);
-      APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      if (!fuse) {
+        hipLaunchKernelGGL(mb_mark_neighbors_kernel<false>, flat, dim3(kMbBlock), 0, st, hp);
+        APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      }
       hipLaunchKernelGGL(mb_count_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
       APT_LAUNCH_CHECK("mb_count_kernel");
       hipLaunchKernelGGL(mb_place_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
@@ -403,6 +493,8 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   LookupParams lp{};
   lp.num_hops = num_hops;
   lp.table = static_cast<const uint32_t*>(rank_table);
+  lp.state = state;
+  lp.last_is_bid = num_hops > 1 ? 1 : 0;
   int64_t nblocks = 0;
   for (int h = 0; h < num_hops; ++h) {
     lp.block_begin[h] = nblocks;
@@ -416,8 +508,5 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   lp.block_begin[num_hops] = nblocks;
   hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kMbBlock), 0, st, lp);
   APT_LAUNCH_CHECK("mb_lookup_kernel");
-  hipLaunchKernelGGL(mb_reset_kernel, grid_for(L.caps[num_hops], kMbBlock, 1 << 15), dim3(kMbBlock), 0,
-                     st, static_cast<uint32_t*>(rank_table), nodes, sizes + num_hops, L.caps[num_hops]);
-  APT_LAUNCH_CHECK("mb_reset_kernel");
   return APT_OK;
 }

@@ -18,6 +18,15 @@
 
 namespace apt {
 
+// Arguments of the fused relabel marking (see SampleParams).
+struct SampleMark {
+  uint32_t* table;
+  int64_t table_len;
+  const uint32_t* state;  // [0] epoch, [1] payload bits: entries of this batch start at epoch << bits
+  int64_t* relabeled;
+  int first_hop;
+};
+
 struct SampleParams {
   apt_graph g;
   const int64_t* frontier;
@@ -31,7 +40,31 @@ struct SampleParams {
   int64_t* counts;
   int64_t* total;
   int rows_per_group;
+  // Optional fusion with the rank-table relabel of the multi-hop driver: every
+  // sampled id is looked up / bid for in `table` right after it is loaded.
+  uint32_t* table;       // NULL = plain sampling
+  int64_t table_len;
+  const uint32_t* table_state;
+  int64_t* relabeled;    // [n * fanout]
+  int first_hop;         // the table holds seed indices, not ids: nothing is final yet
 };
+
+constexpr int64_t kRelabelPending = -2;
+
+// Relabel step for one sampled slot (slot index j of this hop, ns frontier
+// rows): a node that is already in the batch has its id in the table; any other
+// node is bid for with ns + j, the smallest bid becoming its owner.
+__device__ __forceinline__ int64_t mark_slot(const SampleParams& p, uint32_t tb, int64_t v, int64_t ns,
+                                             int64_t j) {
+  if (v < 0) return v;
+  if (v >= p.table_len) return -1;
+  const uint32_t bid = tb + static_cast<uint32_t>(ns + j);
+  // Values only decrease, so a stale read can only cause a redundant atomic.
+  const uint32_t cur = p.table[v];
+  if (!p.first_hop && cur < tb + static_cast<uint32_t>(ns)) return cur - tb;
+  if (cur > bid) atomicMin(&p.table[v], bid);
+  return kRelabelPending;
+}
 
 constexpr int kSampleBlock = 256;
 constexpr int kMaxRowsPerGroup = 16;
@@ -167,6 +200,16 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
         if (gis[u] < n && l < fanout) p.out[gis[u] * fanout + l] = val[u];
+      if (p.table != nullptr) {
+        const uint32_t tb = p.table_state[0] << p.table_state[1];
+        int64_t rel[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          rel[u] = (gis[u] < n && l < fanout) ? mark_slot(p, tb, val[u], n, gis[u] * fanout + l) : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (gis[u] < n && l < fanout) p.relabeled[gis[u] * fanout + l] = rel[u];
+      }
     }
   } else {
     // fanout wider than a group: slots are resolved LPS at a time and earlier
@@ -260,7 +303,7 @@ namespace apt {
 int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
                   const int64_t* num_frontier_dev, int fanout, int replace, uint64_t rng_seed,
                   const uint64_t* rng_seed_dev, int hop, int64_t* out_neighbors, int64_t* out_counts,
-                  int64_t* out_total, hipStream_t st, const char* who) {
+                  int64_t* out_total, hipStream_t st, const char* who, const SampleMark* mark) {
   APT_REQUIRE(graph != nullptr, APT_EINVAL, "%s: graph is NULL", who);
   APT_REQUIRE(num_frontier >= 0, APT_EINVAL, "%s: num_frontier %lld < 0", who, (long long)num_frontier);
   APT_REQUIRE(fanout > 0, APT_EINVAL, "%s: fanout %d must be > 0", who, fanout);
@@ -294,6 +337,19 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
   p.out = out_neighbors;
   p.counts = out_counts;
   p.total = out_total;
+  p.table = nullptr;
+  p.table_len = 0;
+  p.table_state = nullptr;
+  p.relabeled = nullptr;
+  p.first_hop = 0;
+  if (mark != nullptr) {
+    APT_REQUIRE(fanout <= kWave, APT_EINVAL, "%s: fused relabel marking needs fanout <= %d", who, kWave);
+    p.table = mark->table;
+    p.table_len = mark->table_len;
+    p.table_state = mark->state;
+    p.relabeled = mark->relabeled;
+    p.first_hop = mark->first_hop;
+  }
 
   // Lanes per frontier row: the smallest power of two that holds the fanout
   // (8..64).  One whole wavefront per row leaves most lanes idle at the usual
@@ -304,6 +360,8 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
     while (lps < fanout && lps < kWave) lps <<= 1;
   }
   if (!replace && fanout > lps) lps = kWave;  // chunked Floyd needs whole waves
+  if (mark != nullptr)                          // marking lives in the one-chunk path
+    while (lps < fanout) lps <<= 1;
   const int groups = kSampleBlock / lps;
   // Enough workgroups to cover 256 CUs several times over before rows are
   // serialised inside a group.
@@ -333,5 +391,5 @@ extern "C" int apt_sample_neighbors(const apt_graph* graph, const int64_t* front
                                     int64_t* out_total, void* stream) {
   return apt::sample_launch(graph, frontier, num_frontier, num_frontier_dev, fanout, replace,
                             rng_seed, nullptr, hop, out_neighbors, out_counts, out_total,
-                            static_cast<hipStream_t>(stream), "apt_sample_neighbors");
+                            static_cast<hipStream_t>(stream), "apt_sample_neighbors", nullptr);
 }

@@ -47,7 +47,13 @@ int apt_abi_version(void);
  * src/cuda/npc_kernel.h:10-14).  value 0 restores the default.
  *   "sample_lanes_per_row"   8|16|32|64 lanes of a wavefront per frontier row
  *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing
- *   "gather_max_blocks"      cap on the gather grid (rows are strided over) */
+ *   "gather_max_blocks"      cap on the gather grid (rows are strided over)
+ *   "minibatch_payload_bits" width of the id field of rank-table entries (0 = as
+ *                            narrow as the plan allows); wider = fewer epochs
+ *                            between table refills (used to test the refill)
+ *   "minibatch_fuse_mark"    1 (default; note: 0 here also means "off", not
+ *                            "default") the sampling kernel of apt_minibatch_sample
+ *                            also does the rank-table lookup / bid of each id */
 int apt_set_tuning(const char* key, int value);
 
 /* A CSR (CSC in the reference's naming: row v lists the in-neighbours of v)
@@ -237,11 +243,14 @@ int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_dev,
  *                   --fan_out list reversed, python/npc/sampler.py:191)
  *   rng_seed_dev    optional device uint64[1] overriding rng_seed (lets a
  *                   captured HIP graph be replayed with a new seed)
- *   rank_table      device uint32[rank_table_len], rank_table_len >= every node
- *                   id of the graph; apt_rank_table_bytes / apt_rank_table_init
- *                   size and initialise it once, every call leaves it
- *                   initialised again.  A node id outside [0, rank_table_len)
- *                   is treated like padding (no edge, not in the node list).
+ *   rank_table      device scratch of apt_rank_table_bytes(rank_table_len) bytes,
+ *                   256-byte aligned, rank_table_len > every node id of the
+ *                   graph (4 bytes per node + a small state block); initialise
+ *                   it once with apt_rank_table_init, after that it belongs to
+ *                   the library: calls may follow each other on one stream
+ *                   without any clearing in between.  A node id outside
+ *                   [0, rank_table_len) is treated like padding (no edge, not
+ *                   in the node list).
  *   nodes           device int64[capacity(num_hops)]: the unique node list;
  *                   its first sizes[h] entries are the frontier of hop h and
  *                   the source nodes of hop h-1's block, its first
