@@ -54,7 +54,7 @@ def parse_args():
     ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused"],
                     help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
                          "unfused: per-hop sample + hash relabel calls")
-    ap.add_argument("--inflight", type=int, default=3,
+    ap.add_argument("--inflight", type=int, default=4,
                     help="batches in flight: N pipelines on N HIP streams, batches dealt round-robin")
     ap.add_argument("--calibration_copy_mib", type=int, default=0,
                     help="also launch the plain copy kernel once on this many MiB (for scaling "
