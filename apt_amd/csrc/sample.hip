@@ -2,8 +2,9 @@
 //
 // Replaces _CSRRowWiseSampleReplaceKernel / LocalSampleNeighbors
 // (reference src/cuda/npc_kernel.cu:248-316).  Differences by design:
-//   * a lane group (8..64 lanes of a wave64, default one whole wavefront) owns
-//     a frontier row; the block first stages every row's (neighbour pointer,
+//   * a lane group (8..64 lanes of a wave64, the smallest power of two that
+//     holds the fanout) owns a frontier row, with several rows per group in
+//     flight; the block first stages every row's (neighbour pointer,
 //     degree, node) in LDS with one lane per row, so the dependent
 //     frontier -> pos_map -> indptr loads of a whole tile are in flight
 //     together instead of one chain per wave;
