@@ -1,0 +1,128 @@
+"""The pipeline at the benchmark's sizes.
+
+medium (2.4 M nodes / 62 M edges): the graph is copied to the host and the
+whole batch is compared with the oracle, bit for bit.
+full (111 M nodes / 3.2 B edges, 128 x bf16): too big to hand to the CPU oracle
+in a test, so the batch is checked through properties that do not depend on
+size: counts = min(fanout, degree), sampled ids are true neighbours, the node
+list has no duplicates and starts with the seeds, nodes[relabeled] gives the
+sampled ids back, the gathered rows equal torch's own index_select, and the
+same rng key reproduces the batch.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _check_properties(pipe, graph_t, feats, seeds, hops, replace):
+    indptr, indices = graph_t
+    res = pipe.result()
+    nodes = res["input_nodes"]
+    B = seeds.numel()
+    assert torch.equal(nodes[:B], seeds)                                    # dst nodes are a prefix of src nodes
+    assert torch.unique(nodes).numel() == nodes.numel()                     # no duplicates
+    total = 0
+    for h, blk in enumerate(reversed(res["blocks"])):
+        f = blk["fanout"]
+        front = blk["seeds"]
+        deg = indptr[front + 1] - indptr[front]
+        want_cnt = torch.where(deg > 0, torch.full_like(deg, f), torch.zeros_like(deg)) if replace \
+            else torch.minimum(deg, torch.full_like(deg, f))
+        assert torch.equal(blk["counts"], want_cnt)
+        nbr = blk["neighbors"].view(-1, f)
+        rel = blk["relabeled"].view(-1, f)
+        valid = torch.arange(f, device=DEV)[None, :] < blk["counts"][:, None]
+        assert torch.equal(nbr >= 0, valid) and torch.equal(rel >= 0, valid)
+        assert torch.equal(blk["unique"][rel[valid]], nbr[valid])           # relabel round trip
+        assert int(rel.max()) < blk["unique"].numel()
+        total += int(blk["counts"].sum())
+        # rows that fit in the fanout come back whole, in CSR order
+        if not replace:
+            small = torch.nonzero((deg > 0) & (deg <= f)).flatten()[:2000]
+            for r in small[:200].tolist():
+                s, e = int(indptr[front[r]]), int(indptr[front[r] + 1])
+                assert torch.equal(nbr[r, :e - s], indices[s:e])
+        # a sample of the other rows: every id is a neighbour; without replacement no position twice
+        big = torch.nonzero(deg > f).flatten()
+        pick = big[torch.randperm(big.numel(), device=DEV)[:100]]
+        for r in pick.tolist():
+            s, e = int(indptr[front[r]]), int(indptr[front[r] + 1])
+            row = indices[s:e]
+            got = nbr[r]
+            assert bool(torch.isin(got, row).all())
+            if not replace:
+                # multiset containment: an id may repeat in a multigraph row, but not more often than it occurs
+                vals, cnts = torch.unique(got, return_counts=True)
+                for v, c in zip(vals.tolist(), cnts.tolist()):
+                    assert int((row == v).sum()) >= c
+    assert total == res["num_edges"]
+    if feats is not None:
+        assert torch.equal(res["features"].view(torch.int16) if feats.dtype == torch.bfloat16 else res["features"],
+                           (feats.index_select(0, nodes).view(torch.int16) if feats.dtype == torch.bfloat16
+                            else feats.index_select(0, nodes)))
+    return res
+
+
+def test_medium_scale_vs_oracle(orc, capi):
+    from apt_amd import synth
+    from apt_amd.pipeline import MiniBatchPipeline
+    N, E, D = 2_449_029, 62_000_000, 100
+    indptr, indices = synth.rmat_csr_gpu(N, E, 1, DEV)
+    feats = synth.random_features(N, D, torch.float32, 2, DEV)
+    graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
+    hops = [5, 10, 15]
+    pipe = MiniBatchPipeline(graph, store, 1024, hops, replace=False)
+    og = orc.Graph(indptr.cpu().numpy(), indices.cpu().numpy())
+    ofs = orc.FeatStore(feats.cpu().numpy())
+    orc.set_threads(16)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(3)
+    for batch in range(3):
+        seeds = torch.randperm(N, generator=gen, device=DEV)[:1024].contiguous()
+        pipe.run(seeds, 77 + batch)
+        res = _check_properties(pipe, (indptr, indices), feats, seeds, hops, False)
+        want_in, want_blocks = orc.sample_blocks(og, seeds.cpu().numpy(), hops, False, 77 + batch)
+        assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+        for got, want in zip(res["blocks"], want_blocks):
+            for k in ("neighbors", "relabeled", "counts"):
+                assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+        want_f, _ = orc.gather_rows(ofs, want_in)
+        assert np.array_equal(res["features"].cpu().numpy(), want_f)
+    orc.set_threads(1)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_full_scale_properties(capi, replace):
+    from apt_amd import synth
+    from apt_amd.pipeline import MiniBatchPipeline
+    N, E, D = 111_059_956, 3_200_000_000, 128
+    indptr, indices = synth.rmat_csr_gpu(N, E, 1, DEV)
+    assert indices.numel() > 3_000_000_000 and int(indptr[-1]) == indices.numel()
+    feats = synth.random_features(N, D, torch.bfloat16, 2, DEV)
+    graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
+    hops = [5, 10, 15]
+    pipe = MiniBatchPipeline(graph, store, 4096, hops, replace=replace)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(5)
+    seeds = torch.randperm(N, generator=gen, device=DEV)[:4096].contiguous()
+    pipe.run(seeds, 2025)
+    res = _check_properties(pipe, (indptr, indices), feats, seeds, hops, replace)
+    first = {k: res[k].clone() for k in ("input_nodes", "features")}
+    rel0 = [b["relabeled"].clone() for b in res["blocks"]]
+    # the same key reproduces the batch (also after other batches went through the rank table)
+    pipe.run(torch.randperm(N, generator=gen, device=DEV)[:4096].contiguous(), 1)
+    pipe.result()
+    pipe.run(seeds, 2025)
+    again = pipe.result()
+    assert torch.equal(again["input_nodes"], first["input_nodes"])
+    assert torch.equal(again["features"].view(torch.int16), first["features"].view(torch.int16))
+    for a, b in zip(again["blocks"], rel0):
+        assert torch.equal(a["relabeled"], b)
+    # a different key samples differently
+    pipe.run(seeds, 2026)
+    assert not torch.equal(pipe.result()["input_nodes"], first["input_nodes"])
+    del pipe, feats, indices, indptr
+    torch.cuda.empty_cache()
