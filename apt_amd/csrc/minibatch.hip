@@ -503,7 +503,7 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     lp.ns_dev[h] = h == 0 ? nullptr : sizes + h;
     lp.ns_cap[h] = L.caps[h];
     lp.fanout[h] = hop_fanouts[h];
-    nblocks += std::max<int64_t>(1, std::min<int64_t>(ceil_div(L.caps[h] * hop_fanouts[h], kMbBlock), 1 << 15));
+    nblocks += std::max<int64_t>(1, std::min<int64_t>(ceil_div(L.caps[h] * hop_fanouts[h], kMbBlock), 2048));
   }
   lp.block_begin[num_hops] = nblocks;
   hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kMbBlock), 0, st, lp);

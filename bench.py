@@ -3,10 +3,13 @@
 
 A step is one mini-batch: multi-hop uniform neighbour sampling without
 replacement + relabel on every hop + feature gather of the input nodes, with
-the graph, the feature table and the seeds resident in HBM.  Prints ONE JSON
-line: sampled edges/s for the whole step, the gather kernel's achieved HBM
-bandwidth against the 8 TB/s peak (roofline), and the CPU oracle timed on this
-machine's host cores on a bounded sample of the same workload (cpu_baseline).
+the graph, the feature table and the seeds resident in HBM.  K steps are timed
+back to back on one stream.  Prints ONE JSON line: sampled edges/s for the
+whole step, the gather kernel's achieved HBM bandwidth against the 8 TB/s peak
+(roofline, from HIP events around every gather launch of the timed region),
+and the CPU oracle timed on this machine's host cores on a bounded sample of
+the same workload (cpu_baseline).  stages.in_flight is the same K batches with
+several batches in flight on separate streams.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload full|medium|small]
 """
@@ -19,7 +22,7 @@ import time
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes the gather kernel moves per gathered row, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this script (profiles/gather_kernel_full_pmc.txt); None where it has not been measured.
-MEASURED_GATHER_TRAFFIC_PER_ROW = {"full": 520.0}
+MEASURED_GATHER_TRAFFIC_PER_ROW = {"full": 520.0}   # (190.5 MB + 184.7 MB) / 721651 rows
 
 WORKLOADS = {
     # BASELINE.json configs[3]: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
@@ -55,7 +58,8 @@ def parse_args():
                     help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
                          "unfused: per-hop sample + hash relabel calls")
     ap.add_argument("--inflight", type=int, default=4,
-                    help="batches in flight: N pipelines on N HIP streams, batches dealt round-robin")
+                    help="after the timed single-stream region, also run the K batches with N of them in "
+                         "flight (N pipelines on N HIP streams) and report it under stages.in_flight; 1 = skip")
     ap.add_argument("--calibration_copy_mib", type=int, default=0,
                     help="also launch the plain copy kernel once on this many MiB (for scaling "
                          "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
@@ -161,29 +165,37 @@ def main():
         seed_sets = [(seed_lo + torch.randperm(seed_n, generator=gen, device=dev)[:B]).contiguous()
                      for _ in range(K + W)]
 
-    # N batches in flight: each pipeline owns its buffers, rank table and stream
-    pipes, streams = [pipe], [torch.cuda.current_stream()]
-    for _ in range(1, max(1, args.inflight)):
-        pipes.append(make_pipe(args.driver == "graph"))
-        streams.append(torch.cuda.Stream())
-    torch.cuda.synchronize()
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    staged = args.driver != "graph"   # a graph replay cannot be bracketed stage by stage
 
-    def run_batches(first, count):
-        for i in range(count):
-            k = i % len(pipes)
-            with torch.cuda.stream(streams[k]):
-                pipes[k].run(seed_sets[first + i], args.seed + 100 + first + i)
+    def run_step(p, i, marks=None):
+        seeds, key = seed_sets[i], args.seed + 100 + i
+        if marks is None or not staged:
+            p.run(seeds, key)
+            return
+        marks[0].record()
+        p.sample(seeds, key)
+        marks[1].record()
+        p.gather()
+        marks[2].record()
 
     # ---- warm-up
-    run_batches(0, W)
+    for i in range(W):
+        run_step(pipe, i)
     torch.cuda.synchronize()
 
-    # ---- timed region: exactly K steps
+    # ---- timed region: exactly K steps on one stream; sampling+relabel and the gather launch of every
+    # step are bracketed by HIP events recorded on that stream
+    marks = [(ev(), ev(), ev()) for _ in range(K)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    run_batches(W, K)
+    for i in range(K):
+        run_step(pipe, W + i, marks[i])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    if staged:
+        t_sample = sum(m[0].elapsed_time(m[1]) for m in marks)
+        t_gather = sum(m[1].elapsed_time(m[2]) for m in marks)
 
     if args.calibration_copy_mib > 0:
         a = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
@@ -192,42 +204,64 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    # ---- the same K steps on one stream (latency of a batch when nothing overlaps)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        pipe.run(seed_sets[W + i], args.seed + 100 + W + i)
-    torch.cuda.synchronize()
-    single_stream_ms = (time.perf_counter() - t0) / K * 1e3
-
-    # ---- per-stage pass over the same K batches (HIP events on the launch stream)
-    ev = lambda: torch.cuda.Event(enable_timing=True)
-    t_sample = t_gather = 0.0
+    # ---- the same K batches once more, untimed, to read their sizes (one host sync per batch); with the
+    # graph driver this pass also provides the stage timings
     edges = rows = 0
     hop_sizes = []
+    if not staged:
+        t_sample = t_gather = 0.0
     for i in range(K):
-        e0, e1, e2 = ev(), ev(), ev()
-        e0.record()
+        m = (ev(), ev(), ev())
+        m[0].record()
         stage_pipe.sample(seed_sets[W + i], args.seed + 100 + W + i)
-        e1.record()
+        m[1].record()
         stage_pipe.gather()
-        e2.record()
+        m[2].record()
         torch.cuda.synchronize()
-        t_sample += e0.elapsed_time(e1)
-        t_gather += e1.elapsed_time(e2)
+        if not staged:
+            t_sample += m[0].elapsed_time(m[1])
+            t_gather += m[1].elapsed_time(m[2])
         sizes = stage_pipe.sizes.cpu().tolist()
         edges += sizes[-1]
         rows += sizes[len(hops)] if requests is None else int(stage_pipe.request_sizes[0].item())
         hop_sizes.append(sizes[:-1])
-    assert all(int(p.misses.item()) == 0 for p in pipes) and int(stage_pipe.misses.item()) == 0
     request_sizes = None if requests is None else stage_pipe.request_sizes.cpu().tolist()
     bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
 
+    # ---- the same K batches with N batches in flight: N pipelines (own buffers, rank table) on N
+    # streams, batches dealt round-robin; reported beside the single-stream figure
+    in_flight = None
+    if args.inflight > 1:
+        pipes, streams = [pipe], [torch.cuda.current_stream()]
+        for _ in range(1, args.inflight):
+            pipes.append(make_pipe(args.driver == "graph"))
+            streams.append(torch.cuda.Stream())
+        torch.cuda.synchronize()
+
+        def run_batches(first, count):
+            for i in range(count):
+                k = i % len(pipes)
+                with torch.cuda.stream(streams[k]):
+                    pipes[k].run(seed_sets[first + i], args.seed + 100 + first + i)
+
+        run_batches(0, W)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_batches(W, K)
+        torch.cuda.synchronize()
+        t_fl = time.perf_counter() - t0
+        assert all(int(p.misses.item()) == 0 for p in pipes)
+        in_flight = {"batches_in_flight": len(pipes), "ms_per_step": t_fl / K * 1e3,
+                     "edges_per_s": edges / t_fl}
+        del pipes[1:]
+    assert int(pipe.misses.item()) == 0 and int(stage_pipe.misses.item()) == 0
+
     # ---- optional aggregation stage on the outermost block of the last batch
     agg = None
     if args.aggregation:
+        stage_pipe.run(seed_sets[W + K - 1], args.seed + 100 + W + K - 1)
         res = stage_pipe.result()
         blk = res["blocks"][0]
         rel = blk["relabeled"]
@@ -349,7 +383,7 @@ def main():
                         f"fan_out {w['fan_out']} (hops from the seeds: {hops}), "
                         f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
                         f"gather of all input nodes" + part_note,
-            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver, "batches_in_flight": len(pipes),
+            "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver,
         },
         "roofline": {
             "bound": "hbm", "kernel": "gather_kernel",
@@ -365,7 +399,7 @@ def main():
         "cpu_baseline": cpu,
         "aggregation": agg,
         "stages": {
-            "single_stream_ms_per_step": single_stream_ms,
+            "in_flight": in_flight,
             "edges_per_step": edges / K,
             "input_nodes_per_step": rows / K,
             "sample_relabel_ms": t_sample / K,
