@@ -54,6 +54,7 @@ SYMBOLS = {
     "apt_rank_table_bytes": (_SZ, [_I64]),
     "apt_rank_table_init": (_I, [_P, _SZ, _P]),
     "apt_minibatch_workspace_bytes": (_SZ, [_I64, C.POINTER(C.c_int), _I]),
+    "apt_minibatch_workspace_init": (_I, [_P, _SZ, _P]),
     "apt_minibatch_capacity": (_I64, [_I64, C.POINTER(C.c_int), _I, _I]),
     "apt_minibatch_sample": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
@@ -378,6 +379,7 @@ class MinibatchPlan:
         self.table_len = graph.num_total_nodes
         need = int(lib().apt_minibatch_workspace_bytes(self.batch, self._cf, H))
         self.workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+        check(lib().apt_minibatch_workspace_init(_ptr(self.workspace), self.workspace.numel(), _stream()))
         self._nb = (C.c_void_p * H)(*[t.data_ptr() for t in self.neighbors])
         self._rl = (C.c_void_p * H)(*[t.data_ptr() for t in self.relabeled])
         self._ct = (C.c_void_p * H)(*[t.data_ptr() for t in self.counts]) if want_counts else None

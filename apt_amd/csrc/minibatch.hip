@@ -32,13 +32,12 @@
 // On the last hop the owners' ids are not even written to the table: the few
 // slots that lost a race fetch the id from the winner's output slot instead.
 #include "common.hpp"
+#include "rank_table.hpp"
 
 namespace apt {
 
 struct SampleMark {  // fused relabel marking inside the sampling kernel (sample.hip)
-  uint32_t* table;
-  int64_t table_len;
-  const uint32_t* state;
+  RankTable table;
   int64_t* relabeled;
   int first_hop;
 };
@@ -55,7 +54,6 @@ constexpr int kMbIters = 4;
 constexpr int kMbTile = kMbBlock * kMbIters;     // items per workgroup in count / place
 constexpr int kMbWaves = kMbBlock / kWave;
 constexpr uint32_t kEmpty = 0xFFFFFFFFu;
-constexpr int64_t kPending = -2;                  // relabeled[] slot still to be looked up
 constexpr int kMaxHops = APT_MAX_HOPS;
 
 struct HopParams {
@@ -73,6 +71,7 @@ struct HopParams {
   int64_t* n_next;           // receives the size of the list after this hop
   uint64_t* flags;           // owner bit per item, one word per wavefront-load
   uint32_t* tile_cnt;
+  uint8_t* displaced;        // per slot: a smaller bid took the node over (rank_table.hpp)
 };
 
 struct HopSizes {
@@ -88,11 +87,6 @@ __device__ __forceinline__ HopSizes hop_sizes(const HopParams& p) {
 
 __device__ __forceinline__ bool in_table(const HopParams& p, int64_t v) {
   return v >= 0 && v < p.table_len;
-}
-
-// Smallest table value of the current batch: (epoch << payload bits).
-__device__ __forceinline__ uint32_t table_base(const uint32_t* state) {
-  return state[0] << state[1];
 }
 
 // One thread: next epoch, or a refill request when the epochs are used up or
@@ -132,28 +126,16 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, in
   }
 }
 
-// Every sampled slot: already in the batch -> relabelled now; otherwise bid
-// for ownership with (ns + slot index).  FIRST: the table holds seed indices,
-// not ids, so nothing can be finalised yet.
+// Stand-alone marking pass (fanouts wider than a wavefront, or the fusion into
+// the sampling kernel switched off): the same per-slot step as in sample.hip.
 template <bool FIRST>
 __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p) {
   const HopSizes s = hop_sizes(p);
   const uint32_t tb = table_base(p.state);
+  const RankTable t{p.table, p.table_len, p.state, p.displaced};
   for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < s.nn;
-       j += static_cast<int64_t>(gridDim.x) * kMbBlock) {
-    const int64_t v = p.neighbors[j];
-    int64_t out = kPending;
-    if (!in_table(p, v)) {
-      out = v < 0 ? v : -1;  // padding, or an id the table cannot hold: no edge
-    } else {
-      const uint32_t bid = tb + static_cast<uint32_t>(s.ns + j);
-      // Values only decrease, so a stale read can only cause a redundant atomic.
-      const uint32_t cur = p.table[v];
-      if (!FIRST && cur < tb + static_cast<uint32_t>(s.ns)) out = cur - tb;
-      else if (cur > bid) atomicMin(&p.table[v], bid);
-    }
-    p.relabeled[j] = out;
-  }
+       j += static_cast<int64_t>(gridDim.x) * kMbBlock)
+    p.relabeled[j] = rank_table_bid(t, tb, FIRST, p.neighbors[j], s.ns, j);
 }
 
 // Item i of a hop: FIRST -> seeds followed by neighbours (index = bid);
@@ -169,9 +151,12 @@ __device__ __forceinline__ bool mb_is_owner(const HopParams& p, const HopSizes& 
     bid = static_cast<uint32_t>(i);
     if (!in_table(p, v)) return false;
   } else {
-    if (p.relabeled[i] != kPending) return false;  // padding or already in the batch
-    v = p.neighbors[i];
-    bid = static_cast<uint32_t>(s.ns + i);
+    // Later hops: the bidding itself settled ownership (rank_table.hpp); the
+    // flag is consumed so that the buffer is clean for the next hop.
+    if (p.relabeled[i] != kSlotOwner) return false;
+    if (p.displaced[i] == 0) return true;
+    p.displaced[i] = 0;
+    return false;
   }
   return p.table[v] == table_base(p.state) + bid;
 }
@@ -286,7 +271,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
   const int64_t ns = actual_count(p.ns_cap[h], p.ns_dev[h]);
   for (int64_t j = (static_cast<int64_t>(blockIdx.x) - p.block_begin[h]) * kMbBlock + threadIdx.x;
        j < nn; j += blocks * kMbBlock) {
-    if (p.relabeled[h][j] != kPending) continue;
+    if (p.relabeled[h][j] > kSlotOwner) continue;  // an id, or padding (-1)
     const int64_t e = p.table[p.neighbors[h][j]] - tb;
     // via_owner: e is the winning bid ns + slot; the winner's slot holds the id
     // (it is an owner, so its slot is final and never pending).
@@ -295,6 +280,13 @@ __global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
 }
 
 __global__ void mb_zero_state_kernel(uint32_t* state) { state[threadIdx.x] = 0; }
+
+__global__ __launch_bounds__(kMbBlock) void mb_zero_kernel(uint4* p, int64_t vecs) {
+  const uint4 z = make_uint4(0, 0, 0, 0);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
+       i += static_cast<int64_t>(gridDim.x) * kMbBlock)
+    p[i] = z;
+}
 
 __global__ __launch_bounds__(kMbBlock) void mb_fill_table_kernel(uint4* table, int64_t vecs) {
   const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
@@ -306,7 +298,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_fill_table_kernel(uint4* table, i
 static size_t mb_align(size_t x) { return (x + 255) / 256 * 256; }
 
 struct MbLayout {
-  size_t flags_off, tile_off, total;
+  size_t flags_off, tile_off, displaced_off, total;
   int64_t caps[kMaxHops + 1];
   int64_t max_items;
   uint32_t payload_bits;  // ids and bids of the plan are < 2^payload_bits
@@ -337,6 +329,7 @@ static bool mb_layout(int64_t batch, const int* fanouts, int num_hops, MbLayout&
   size_t off = 0;
   L.flags_off = off; off = mb_align(off + sizeof(uint64_t) * tiles * kMbIters * kMbWaves);
   L.tile_off = off;  off = mb_align(off + sizeof(uint32_t) * tiles);
+  L.displaced_off = off; off = mb_align(off + static_cast<size_t>(L.max_items));
   L.total = off;
   return true;
 }
@@ -372,6 +365,19 @@ extern "C" size_t apt_minibatch_workspace_bytes(int64_t batch, const int* hop_fa
   if (batch < 0 || hop_fanouts == nullptr || num_hops < 1 || num_hops > apt::kMaxHops) return 0;
   if (!apt::mb_layout(batch, hop_fanouts, num_hops, L)) return 0;
   return L.total;
+}
+
+extern "C" int apt_minibatch_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(workspace != nullptr && workspace_bytes % 16 == 0 &&
+                  (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
+              APT_EINVAL, "apt_minibatch_workspace_init: workspace must be 16-byte aligned and sized");
+  if (workspace_bytes == 0) return APT_OK;
+  const int64_t vecs = static_cast<int64_t>(workspace_bytes / 16);
+  hipLaunchKernelGGL(mb_zero_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(ceil_div(vecs, kMbBlock), 4096))),
+                     dim3(kMbBlock), 0, static_cast<hipStream_t>(stream), static_cast<uint4*>(workspace), vecs);
+  APT_LAUNCH_CHECK("mb_zero_kernel");
+  return APT_OK;
 }
 
 extern "C" int64_t apt_minibatch_capacity(int64_t batch, const int* hop_fanouts, int num_hops, int hop) {
@@ -430,6 +436,7 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   hp.nodes = nodes;
   hp.flags = reinterpret_cast<uint64_t*>(ws + L.flags_off);
   hp.tile_cnt = reinterpret_cast<uint32_t*>(ws + L.tile_off);
+  hp.displaced = reinterpret_cast<uint8_t*>(ws + L.displaced_off);
   hp.seeds = seeds;
   hp.ns_cap = batch;
   hp.ns_dev = nullptr;
@@ -455,7 +462,8 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     // The sampling kernel looks every id up in the rank table as soon as it has
     // loaded it (fanouts up to one wavefront); otherwise a separate pass does.
     const bool fuse = f <= kWave && tuning_fuse_mark() != 0;
-    SampleMark mark{static_cast<uint32_t*>(rank_table), rank_table_len, state, relabeled[h], h == 0 ? 1 : 0};
+    SampleMark mark{RankTable{static_cast<uint32_t*>(rank_table), rank_table_len, state, hp.displaced},
+                    relabeled[h], h == 0 ? 1 : 0};
     int rc = sample_launch(graph, frontier, ns_cap, ns_dev, static_cast<int>(f), replace, rng_seed,
                            rng_seed_dev, h, neighbors[h], counts != nullptr ? counts[h] : nullptr,
                            total, st, "apt_minibatch_sample", fuse ? &mark : nullptr);

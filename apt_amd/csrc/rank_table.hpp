@@ -1,0 +1,57 @@
+// The per-slot step of the rank-table relabel, shared by the sampling kernel
+// (marking fused into sampling) and the stand-alone marking pass.
+#pragma once
+
+#include "common.hpp"
+
+namespace apt {
+
+// States of a relabeled[] slot before its compact id is known.
+constexpr int64_t kSlotOwner = -2;  // bid placed and, so far, the smallest for its node
+constexpr int64_t kSlotLoser = -3;  // another slot holds a smaller bid for the same node
+
+struct RankTable {
+  uint32_t* entries;        // one per node: (epoch << payload bits) | id or bid
+  int64_t len;
+  const uint32_t* state;    // [0] epoch, [1] payload bits, [2] refill request
+  uint8_t* displaced;       // per slot of the current hop: set when a smaller bid took the node over
+};
+
+// Smallest entry value of the current batch.
+__device__ __forceinline__ uint32_t table_base(const uint32_t* state) { return state[0] << state[1]; }
+
+// Slot j (of ns * fanout) of a hop with ns frontier rows sampled node v.
+//   v already in the batch (id < ns in the table)  -> its id, no atomic;
+//   otherwise bid ns + j: the smallest bid owns the node.  A returning
+//   atomicMin tells the bidder whether it is the smallest so far, and which
+//   earlier bid it displaced; that slot is flagged, so after the kernel a slot
+//   owns its node iff it is kSlotOwner and not flagged: no second look at the
+//   table is needed.  (The value only ever decreases, and every decrease is an
+//   atomicMin that returns the bid it replaces, so exactly the final minimum is
+//   never flagged.)
+// first_hop: the table holds seed indices, not ids, so hits cannot be resolved
+// yet and ownership is decided by re-reading the table; no flags are kept.
+__device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, uint32_t tb, bool first_hop,
+                                                  int64_t v, int64_t ns, int64_t j) {
+  if (v < 0) return v;
+  if (v >= t.len) return -1;  // an id the table cannot hold: treated as padding
+  const uint32_t first_bid = tb + static_cast<uint32_t>(ns);
+  const uint32_t bid = first_bid + static_cast<uint32_t>(j);
+  // A stale read can only show a larger value than the table holds now, which
+  // at worst causes a redundant atomic.
+  const uint32_t cur = t.entries[v];
+  if (first_hop) {
+    if (cur > bid) atomicMin(&t.entries[v], bid);
+    return kSlotOwner;
+  }
+  if (cur < first_bid) return static_cast<int64_t>(cur - tb);
+  if (cur < bid) return kSlotLoser;
+  const uint32_t old = atomicMin(&t.entries[v], bid);
+  if (old < bid) return old < first_bid ? static_cast<int64_t>(old - tb) : kSlotLoser;
+  // old > bid: this slot is the smallest so far.  If old belongs to this batch it
+  // is a bid of this hop (ids are below first_bid): that slot has been displaced.
+  if ((old >> t.state[1]) == t.state[0]) t.displaced[old - first_bid] = 1;
+  return kSlotOwner;
+}
+
+}  // namespace apt

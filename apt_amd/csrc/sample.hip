@@ -16,14 +16,13 @@
 //   * unused output slots are written as -1 (the reference leaves garbage for
 //     degree-0 rows, :277).
 #include "common.hpp"
+#include "rank_table.hpp"
 
 namespace apt {
 
 // Arguments of the fused relabel marking (see SampleParams).
 struct SampleMark {
-  uint32_t* table;
-  int64_t table_len;
-  const uint32_t* state;  // [0] epoch, [1] payload bits: entries of this batch start at epoch << bits
+  RankTable table;
   int64_t* relabeled;
   int first_hop;
 };
@@ -42,30 +41,11 @@ struct SampleParams {
   int64_t* total;
   int rows_per_group;
   // Optional fusion with the rank-table relabel of the multi-hop driver: every
-  // sampled id is looked up / bid for in `table` right after it is loaded.
-  uint32_t* table;       // NULL = plain sampling
-  int64_t table_len;
-  const uint32_t* table_state;
+  // sampled id is looked up / bid for in the rank table right after it is loaded.
+  RankTable table;       // entries == NULL: plain sampling
   int64_t* relabeled;    // [n * fanout]
-  int first_hop;         // the table holds seed indices, not ids: nothing is final yet
+  int first_hop;
 };
-
-constexpr int64_t kRelabelPending = -2;
-
-// Relabel step for one sampled slot (slot index j of this hop, ns frontier
-// rows): a node that is already in the batch has its id in the table; any other
-// node is bid for with ns + j, the smallest bid becoming its owner.
-__device__ __forceinline__ int64_t mark_slot(const SampleParams& p, uint32_t tb, int64_t v, int64_t ns,
-                                             int64_t j) {
-  if (v < 0) return v;
-  if (v >= p.table_len) return -1;
-  const uint32_t bid = tb + static_cast<uint32_t>(ns + j);
-  // Values only decrease, so a stale read can only cause a redundant atomic.
-  const uint32_t cur = p.table[v];
-  if (!p.first_hop && cur < tb + static_cast<uint32_t>(ns)) return cur - tb;
-  if (cur > bid) atomicMin(&p.table[v], bid);
-  return kRelabelPending;
-}
 
 constexpr int kSampleBlock = 256;
 constexpr int kMaxRowsPerGroup = 16;
@@ -201,12 +181,14 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
         if (gis[u] < n && l < fanout) p.out[gis[u] * fanout + l] = val[u];
-      if (p.table != nullptr) {
-        const uint32_t tb = p.table_state[0] << p.table_state[1];
+      if (p.table.entries != nullptr) {
+        const uint32_t tb = table_base(p.table.state);
         int64_t rel[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          rel[u] = (gis[u] < n && l < fanout) ? mark_slot(p, tb, val[u], n, gis[u] * fanout + l) : -1;
+          rel[u] = (gis[u] < n && l < fanout)
+                       ? rank_table_bid(p.table, tb, p.first_hop != 0, val[u], n, gis[u] * fanout + l)
+                       : -1;
 #pragma unroll
         for (int u = 0; u < U; ++u)
           if (gis[u] < n && l < fanout) p.relabeled[gis[u] * fanout + l] = rel[u];
@@ -338,16 +320,12 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
   p.out = out_neighbors;
   p.counts = out_counts;
   p.total = out_total;
-  p.table = nullptr;
-  p.table_len = 0;
-  p.table_state = nullptr;
+  p.table = RankTable{nullptr, 0, nullptr, nullptr};
   p.relabeled = nullptr;
   p.first_hop = 0;
   if (mark != nullptr) {
     APT_REQUIRE(fanout <= kWave, APT_EINVAL, "%s: fused relabel marking needs fanout <= %d", who, kWave);
     p.table = mark->table;
-    p.table_len = mark->table_len;
-    p.table_state = mark->state;
     p.relabeled = mark->relabeled;
     p.first_hop = mark->first_hop;
   }

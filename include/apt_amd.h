@@ -263,11 +263,16 @@ int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_dev,
  *   sizes           device int64[num_hops + 2]: sizes[h] = frontier rows
  *                   entering hop h (sizes[0] = batch), sizes[num_hops] = input
  *                   nodes, sizes[num_hops + 1] = sampled edges of the batch
+ *   workspace       device scratch of apt_minibatch_workspace_bytes, zeroed once
+ *                   with apt_minibatch_workspace_init before its first use (and
+ *                   again after a call that failed half-way); calls leave it
+ *                   ready for the next one
  *   capacity(h)     apt_minibatch_capacity: batch * prod_{i<h}(1 + fanout_i)
  */
 size_t apt_rank_table_bytes(int64_t num_total_nodes);
 int apt_rank_table_init(void* table, size_t table_bytes, void* stream);
 size_t apt_minibatch_workspace_bytes(int64_t batch, const int* hop_fanouts, int num_hops);
+int apt_minibatch_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 int64_t apt_minibatch_capacity(int64_t batch, const int* hop_fanouts, int num_hops, int hop);
 int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
                          const int* hop_fanouts, int num_hops, int replace,
