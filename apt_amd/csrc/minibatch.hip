@@ -27,8 +27,9 @@
 // lower epoch, so the entries of earlier batches (larger epochs, or the
 // all-ones fill) compare greater than anything the current batch writes and an
 // atomicMin overrides them without being told.  The epoch lives in device
-// memory next to the table, so a captured HIP graph replays correctly; when
-// the epochs run out (every 2^(32-P) - 1 calls) the table is refilled.
+// memory next to the table (the first kernel of a batch advances it), so a
+// captured HIP graph replays correctly; when the epochs run out (every
+// 2^(32-P) - 1 calls) that kernel refills the table.
 // On the last hop the owners' ids are not even written to the table: the few
 // slots that lost a race fetch the id from the winner's output slot instead.
 #include "common.hpp"
@@ -65,7 +66,7 @@ struct HopParams {
   int64_t* relabeled;        // [ns_cap * fanout]
   uint32_t* table;
   int64_t table_len;
-  const uint32_t* state;     // [0] epoch, [1] payload bits, [2] refill request
+  const uint32_t* state;     // [0] epoch, [1] payload bits (see mb_begin_kernel)
   int last;                  // last hop: ids are not written back to the table
   int64_t* nodes;            // growing unique list
   int64_t* n_next;           // receives the size of the list after this hop
@@ -89,29 +90,35 @@ __device__ __forceinline__ bool in_table(const HopParams& p, int64_t v) {
   return v >= 0 && v < p.table_len;
 }
 
-// One thread: next epoch, or a refill request when the epochs are used up or
-// the table was last used with another payload width.
-__global__ void mb_begin_kernel(uint32_t* state, uint32_t payload_bits) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  const uint32_t top = (1u << (32 - payload_bits)) - 1;  // all-ones epoch = the fill value
-  if (state[1] != payload_bits || state[0] == 0 || state[0] > top - 1) {
-    state[0] = top - 1;
-    state[1] = payload_bits;
-    state[2] = 1;
-  } else {
-    state[0] -= 1;
-    state[2] = 0;
-  }
-}
+// Epoch bookkeeping (state block behind the table entries):
+//   [0] epoch of the latest batch  [1] payload bits  [3] finished-workgroup counter
+// First kernel of every batch, a few workgroups: move to the next lower epoch,
+// or, when the epochs are used up (or the table was last used with another
+// payload width, or is new), refill the table with all-ones and start the
+// numbering over.  Every workgroup reads the state before any of them can
+// change it, because only the workgroup that finishes last writes.
+constexpr int kBeginBlocks = 64;
 
-// Refill, only when mb_begin_kernel asked for it.
-__global__ __launch_bounds__(kMbBlock) void mb_refill_kernel(uint4* table, int64_t vecs,
-                                                             const uint32_t* state) {
-  if (state[2] == 0) return;
-  const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
-       i += static_cast<int64_t>(gridDim.x) * kMbBlock)
-    table[i] = ones;
+__global__ __launch_bounds__(kMbBlock) void mb_begin_kernel(uint4* table, int64_t vecs, uint32_t* state,
+                                                            uint32_t payload_bits) {
+  const bool refill = state[1] != payload_bits || state[0] == 0;
+  if (refill) {
+    const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
+         i += static_cast<int64_t>(gridDim.x) * kMbBlock)
+      table[i] = ones;
+    __threadfence();
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && atomicAdd(&state[3], 1u) == gridDim.x - 1) {
+    state[3] = 0;
+    if (refill) {
+      state[0] = (1u << (32 - payload_bits)) - 2;  // the all-ones epoch is the fill value
+      state[1] = payload_bits;
+    } else {
+      state[0] -= 1;
+    }
+  }
 }
 
 // First hop only: seeds may repeat, so they race like everything else; the
@@ -281,6 +288,10 @@ __global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
 
 __global__ void mb_zero_state_kernel(uint32_t* state) { state[threadIdx.x] = 0; }
 
+__global__ void mb_zero_sizes_kernel(int64_t* sizes, int n) {
+  if (static_cast<int>(threadIdx.x) < n) sizes[threadIdx.x] = 0;
+}
+
 __global__ __launch_bounds__(kMbBlock) void mb_zero_kernel(uint4* p, int64_t vecs) {
   const uint4 z = make_uint4(0, 0, 0, 0);
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; i < vecs;
@@ -419,14 +430,17 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
 
   uint32_t* state = reinterpret_cast<uint32_t*>(static_cast<char*>(rank_table) +
                                                 table_state_offset(rank_table_len));
-  // next epoch (or a refill once they are used up)
-  hipLaunchKernelGGL(mb_begin_kernel, dim3(1), dim3(64), 0, st, state, L.payload_bits);
-  APT_LAUNCH_CHECK("mb_begin_kernel");
+  if (batch == 0) {
+    hipLaunchKernelGGL(mb_zero_sizes_kernel, dim3(1), dim3(64), 0, st, sizes, num_hops + 2);
+    APT_LAUNCH_CHECK("mb_zero_sizes_kernel");
+    return APT_OK;
+  }
   {
+    // next epoch; refills only when the epochs are used up (or the table is new)
     const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
-    hipLaunchKernelGGL(mb_refill_kernel, dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(vecs, kMbBlock), 4096)))),
-                       dim3(kMbBlock), 0, st, static_cast<uint4*>(rank_table), vecs, state);
-    APT_LAUNCH_CHECK("mb_refill_kernel");
+    hipLaunchKernelGGL(mb_begin_kernel, dim3(kBeginBlocks), dim3(kMbBlock), 0, st,
+                       static_cast<uint4*>(rank_table), vecs, state, L.payload_bits);
+    APT_LAUNCH_CHECK("mb_begin_kernel");
   }
 
   HopParams hp{};
@@ -448,8 +462,6 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
                        dim3(kMbBlock), 0, st, hp, sizes, num_hops + 2);
     APT_LAUNCH_CHECK("mb_mark_seeds_kernel");
   }
-  if (batch == 0) return APT_OK;
-
   auto grid_for = [](int64_t n, int64_t per_block, int64_t cap) {
     return dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, per_block), cap))));
   };

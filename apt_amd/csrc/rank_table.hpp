@@ -13,7 +13,7 @@ constexpr int64_t kSlotLoser = -3;  // another slot holds a smaller bid for the 
 struct RankTable {
   uint32_t* entries;        // one per node: (epoch << payload bits) | id or bid
   int64_t len;
-  const uint32_t* state;    // [0] epoch, [1] payload bits, [2] refill request
+  const uint32_t* state;    // [0] epoch, [1] payload bits
   uint8_t* displaced;       // per slot of the current hop: set when a smaller bid took the node over
 };
 
