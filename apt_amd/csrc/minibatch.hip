@@ -17,8 +17,10 @@
 //   * a sampled neighbour that is already in the batch is relabelled by one
 //     load, with no atomic at all (hubs are almost always already there);
 //   * the others race with atomicMin on (n_h + slot index); the smallest index
-//     owns the node, owners are ranked with ballots + a two-level prefix, get
-//     id n_h + rank and are appended to the list.
+//     owns the node.  The atomic returns the bid it replaces, the bidder flags
+//     that slot as displaced, so ownership is known without reading the table
+//     again (rank_table.hpp); owners are ranked with ballots + a two-level
+//     prefix, get id n_h + rank and are appended to the list.
 // Random atomics are the scarcest resource on this GPU (~20 G/s against
 // ~45 G/s random loads), which is why the table is indexed directly (no CAS
 // to claim a slot, no probing) and why nodes already present never touch one.
