@@ -25,17 +25,17 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_GATHER_TRAFFIC_PER_ROW = {"full": 520.0}   # (190.5 MB + 184.7 MB) / 721651 rows
 
 WORKLOADS = {
-    # BASELINE.json configs[3]: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
+    # full-scale single GPU: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
     "full": dict(nodes=111_059_956, edges=3_200_000_000, dim=128, dtype="bf16", batch=4096,
                  fan_out=[15, 10, 5]),
-    # configs[1]: products-sized, 62M edges, 100 x fp32, batch 1024
+    # products-sized: 2.4M nodes, 62M edges, 100 x fp32, batch 1024
     "medium": dict(nodes=2_449_029, edges=62_000_000, dim=100, dtype="fp32", batch=1024,
                    fan_out=[15, 10, 5]),
-    # configs[2]: one GPU's share of the full graph: a contiguous 1/8 of the rows, local features plus a
+    # one GPU's share of the full graph: a contiguous 1/8 of the rows, local features plus a
     # cache of the 20% hottest remote rows, misses bucketed into 8 owner request lists
     "partition": dict(nodes=111_059_956, edges=3_200_000_000, dim=128, dtype="fp32", batch=1024,
                       fan_out=[15, 10, 5], parts=8, part=3, cache_ratio=0.2),
-    # configs[0]: CPU-runnable plumbing case
+    # the small plumbing case: 100k nodes, 2 hops
     "small": dict(nodes=100_000, edges=1_500_000, dim=128, dtype="fp32", batch=1024, fan_out=[10, 5]),
 }
 
@@ -173,11 +173,10 @@ def main():
         if marks is None or not staged:
             p.run(seeds, key)
             return
-        marks[0].record()
         p.sample(seeds, key)
-        marks[1].record()
+        marks[0].record()
         p.gather()
-        marks[2].record()
+        marks[1].record()
 
     # ---- warm-up
     for i in range(W):
@@ -186,16 +185,20 @@ def main():
 
     # ---- timed region: exactly K steps on one stream; sampling+relabel and the gather launch of every
     # step are bracketed by HIP events recorded on that stream
-    marks = [(ev(), ev(), ev()) for _ in range(K)]
+    # (two events per step: gather start and gather end; a step's sampling+relabel runs from the
+    # previous step's gather end to its own gather start)
+    marks = [(ev(), ev()) for _ in range(K)]
+    start = ev()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    start.record()
     for i in range(K):
         run_step(pipe, W + i, marks[i])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     if staged:
-        t_sample = sum(m[0].elapsed_time(m[1]) for m in marks)
-        t_gather = sum(m[1].elapsed_time(m[2]) for m in marks)
+        t_gather = sum(m[0].elapsed_time(m[1]) for m in marks)
+        t_sample = start.elapsed_time(marks[-1][1]) - t_gather
 
     if args.calibration_copy_mib > 0:
         a = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
