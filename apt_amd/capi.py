@@ -383,6 +383,8 @@ class MinibatchPlan:
         self._nb = (C.c_void_p * H)(*[t.data_ptr() for t in self.neighbors])
         self._rl = (C.c_void_p * H)(*[t.data_ptr() for t in self.relabeled])
         self._ct = (C.c_void_p * H)(*[t.data_ptr() for t in self.counts]) if want_counts else None
+        # the table and workspace were initialised on the current stream; the plan may be used on any
+        torch.cuda.current_stream().synchronize()
 
     def launch(self, seeds, rng_seed=None):
         """Asynchronous.  rng_seed=None reads the seed from self.rng_seed_dev."""

@@ -254,3 +254,43 @@ def test_rank_table_epochs_and_refill(orc, capi, fuse_mark):
     pipe2.run(dev(seeds), 5)
     want_in, _ = orc.sample_blocks(og, seeds, [3], True, 5)
     assert np.array_equal(pipe2.result()["input_nodes"].cpu().numpy(), want_in)
+
+
+def test_batches_in_flight_are_reproducible(orc, capi):
+    """Three pipelines on three streams: whatever else is running, a batch with
+    the same seeds and rng key gives the same node list and compact ids."""
+    from apt_amd import synth
+    from apt_amd.pipeline import MiniBatchPipeline
+    N = 500_000
+    indptr, indices = synth.rmat_csr_gpu(N, 12_000_000, 3, DEV)
+    g = capi.Graph(indptr, indices)
+    hops = [5, 10, 15]
+    pipes = [MiniBatchPipeline(g, None, 1024, hops, gather=False) for _ in range(3)]
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(9)
+    seeds = torch.randperm(N, generator=gen, device=DEV)[:1024].contiguous()
+    other = [torch.randperm(N, generator=gen, device=DEV)[:1024].contiguous() for _ in range(4)]
+    torch.cuda.synchronize()
+    ref = None
+    for it in range(12):
+        for k in range(3):
+            with torch.cuda.stream(streams[k]):
+                if k == it % 3:
+                    pipes[k].run(seeds, 4242)
+                else:
+                    pipes[k].run(other[(it + k) % 4], it)
+        torch.cuda.synchronize()
+        r = pipes[it % 3].result()
+        cur = (r["input_nodes"].clone(), [b["relabeled"].clone() for b in r["blocks"]])
+        if ref is None:
+            ref = cur
+            og = orc.Graph(indptr.cpu().numpy(), indices.cpu().numpy())
+            want_in, want_blocks = orc.sample_blocks(og, seeds.cpu().numpy(), hops, False, 4242)
+            assert np.array_equal(cur[0].cpu().numpy(), want_in)
+            for a, b in zip(cur[1], want_blocks):
+                assert np.array_equal(a.cpu().numpy(), b["relabeled"])
+        else:
+            assert torch.equal(cur[0], ref[0]), it
+            for a, b in zip(cur[1], ref[1]):
+                assert torch.equal(a, b), it
