@@ -277,3 +277,34 @@ def test_cluster_reqs(orc, capi):
     got = capi.cluster_reqs(dev(ids), dev(fm), dev(rwm), dev(min_vids), W, R)
     for g, w in zip(got, want):
         assert np.array_equal(host(g), w)
+
+
+# ------------------------------------------------------------------ uniformity on the GPU itself
+@pytest.mark.parametrize("deg,fanout,replace", [(16, 15, False), (40, 10, False), (1000, 15, False),
+                                                (37, 8, True), (6, 3, False)])
+def test_sampling_uniformity_chi_square(capi, deg, fanout, replace):
+    """20000 nodes with identical rows 0..deg-1: every node is an independent
+    draw (the counter is keyed by the node id), so the position histogram must
+    be flat; for deg=6, k=3 all 20 subsets must be equally likely."""
+    import itertools
+    from scipy import stats
+    n = 20000
+    indptr = np.arange(n + 1, dtype=np.int64) * deg
+    indices = np.tile(np.arange(deg, dtype=np.int64), n)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    nbr, cnt = capi.sample_neighbors(dg, dev(np.arange(n)), fanout, replace, 987654321, 2)
+    nbr = host(nbr).reshape(n, fanout)
+    assert np.all(host(cnt) == fanout) and nbr.min() >= 0 and nbr.max() < deg
+    hist = np.bincount(nbr.reshape(-1), minlength=deg)
+    assert stats.chisquare(hist).pvalue > 1e-4
+    if not replace:
+        assert all(len(set(r.tolist())) == fanout for r in nbr[:2000])        # distinct positions
+        if deg == 6:
+            subsets = {s: 0 for s in itertools.combinations(range(deg), fanout)}
+            for r in nbr:
+                subsets[tuple(sorted(r.tolist()))] += 1
+            obs = np.array(list(subsets.values()))
+            assert np.all(obs > 0) and stats.chisquare(obs).pvalue > 1e-4
+    else:
+        for s in range(fanout):                                               # every slot on its own
+            assert stats.chisquare(np.bincount(nbr[:, s], minlength=deg)).pvalue > 1e-5
