@@ -59,6 +59,9 @@ SYMBOLS = {
     "apt_minibatch_sample": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                   _SZ, _P]),
+    "apt_count_ids": (_I, [_P, _I64, _P, _P, _I64, _P]),
+    "apt_csr_row_degrees": (_I, [_P, _I64, _I64, _P, _I64, _P, _P]),
+    "apt_csr_copy_rows": (_I, [_P, _P, _I64, _P, _I64, _P, _I64, _P, _P]),
     "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
     "apt_spmm_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I64, _I, _I, _P, _P]),
     "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
@@ -469,3 +472,37 @@ def spmm_block(neighbors, num_dst, fanout, x, mean=False, num_dst_dev=None, out=
                                x.shape[0], x.shape[1], x.element_size(), int(bool(mean)), _ptr(out),
                                _stream()))
     return out
+
+
+def count_ids(ids, freq, n_dev=None):
+    """freq[ids] += 1 (in place), ids outside [0, len(freq)) ignored."""
+    ids = _dev_i64(ids, "ids")
+    freq = _dev_i64(freq, "freq")
+    check(lib().apt_count_ids(_ptr(ids), ids.numel(), _ptr(n_dev), _ptr(freq), freq.numel(), _stream()))
+    return freq
+
+
+def csr_row_degrees(graph, rows):
+    """Degree of every node of `rows` in the graph's main table (0 outside it)."""
+    rows = _dev_i64(rows, "rows")
+    deg = torch.empty(rows.numel(), dtype=torch.int64, device=rows.device)
+    if rows.numel():
+        check(lib().apt_csr_row_degrees(_ptr(graph.indptr), graph.row_begin, graph.num_rows, _ptr(rows),
+                                        rows.numel(), _ptr(deg), _stream()))
+    return deg
+
+
+def csr_select_rows(graph, rows):
+    """The adjacency rows of `rows` (node ids) as a CSR of their own ->
+    (indptr int64[n+1], indices int64[sum of degrees]).  Reads the graph's main
+    table only (not a cache registered on it)."""
+    rows = _dev_i64(rows, "rows")
+    n = rows.numel()
+    dev = rows.device
+    out_indptr = torch.zeros(n + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(csr_row_degrees(graph, rows), 0, out=out_indptr[1:])
+    total = int(out_indptr[-1].item())
+    out_indices = torch.empty(total, dtype=torch.int64, device=dev)
+    check(lib().apt_csr_copy_rows(_ptr(graph.indptr), _ptr(graph.indices), graph.row_begin, _ptr(rows), n,
+                                  _ptr(out_indptr), total, _ptr(out_indices), _stream()))
+    return out_indptr, out_indices

@@ -282,6 +282,28 @@ int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t b
                          int64_t* const* counts, int64_t* sizes, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/* Cache construction (the callers of the registries).
+ *   apt_count_ids        freq[ids[i]] += 1 for ids in [0, num_total_nodes): the
+ *                        access counting of a dry run (examples/dryrun.py:86-92,
+ *                        counter[nodes] += 1 per batch, done there on the host);
+ *                        n_dev as in apt_sample_neighbors
+ *   apt_csr_row_degrees  degrees[i] = degree of node rows[i] (0 when the node has
+ *                        no row in [row_begin, row_begin + num_rows))
+ *   apt_csr_copy_rows    the adjacency rows of the chosen nodes as a second CSR:
+ *                        out_indices[out_indptr[i] + k] = k-th neighbour of rows[i],
+ *                        with out_indptr the exclusive prefix sum of the degrees
+ *                        (n + 1 entries, out_indptr[n] = num_out_edges) — what
+ *                        python/npc/ops.py:370-384 builds with one slice per node
+ *                        before mix_cache_graphs.
+ * The cached feature table is apt_gather_rows on the chosen ids. */
+int apt_count_ids(const int64_t* ids, int64_t n, const int64_t* n_dev, int64_t* freq,
+                  int64_t num_total_nodes, void* stream);
+int apt_csr_row_degrees(const int64_t* indptr, int64_t row_begin, int64_t num_rows,
+                        const int64_t* rows, int64_t n, int64_t* degrees, void* stream);
+int apt_csr_copy_rows(const int64_t* indptr, const int64_t* indices, int64_t row_begin,
+                      const int64_t* rows, int64_t n, const int64_t* out_indptr,
+                      int64_t num_out_edges, int64_t* out_indices, void* stream);
+
 /* Aggregation over the COO edges of sampled blocks (optional stage).
  * Replaces CopyUSum / CopyESum / UMulESum (src/spmm.cc:9-42, src/cuda/spmm.cu:8-148)
  * and UAddV / UMulV (src/sddmm.cc:9-31, src/cuda/sddmm.cu:8-103).

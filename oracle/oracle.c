@@ -24,6 +24,7 @@
  *   orc_cluster_*       numpy searchsorted + stable argsort closed form; the
  *                       inputs of tests/test_shuffle_seeds.cc:19-26.
  *   orc_permute/scatter numpy take / put.
+ *   orc_count_ids, orc_csr_select_rows   numpy bincount / concatenated slices.
  *   orc_spmm_sum/sddmm  numpy closed forms (np.add.at over fancy-indexed rows,
  *                       in float64); a sum over a row of ones equals its
  *                       in-degree.
@@ -444,4 +445,33 @@ void orc_sddmm(int op, const int64_t* row, const int64_t* col, int64_t E, const 
       out[e * dim + d] = op == 0 ? a + b : a * b;
     }
   }
+}
+
+/* ------------------------------------------------------------------ */
+/* Cache construction: access counting (examples/dryrun.py:90-92) and   */
+/* the cached CSR of chosen rows (python/npc/ops.py:370-384).  Pinned   */
+/* by numpy closed forms (bincount; concatenation of row slices).       */
+/* ------------------------------------------------------------------ */
+void orc_count_ids(const int64_t* ids, int64_t n, int64_t* freq, int64_t num_total) {
+  for (int64_t i = 0; i < n; ++i)
+    if (ids[i] >= 0 && ids[i] < num_total) freq[ids[i]] += 1;
+}
+
+/* out_indptr must hold n + 1 entries; returns the number of edges.  With
+ * out_indices == NULL only the offsets are computed. */
+int64_t orc_csr_select_rows(const int64_t* indptr, const int64_t* indices, int64_t row_begin,
+                            int64_t num_rows, const int64_t* rows, int64_t n, int64_t* out_indptr,
+                            int64_t* out_indices) {
+  int64_t acc = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    out_indptr[i] = acc;
+    int64_t r = rows[i] - row_begin;
+    if (r < 0 || r >= num_rows) continue;
+    int64_t s = indptr[r], e = indptr[r + 1];
+    if (out_indices)
+      for (int64_t k = s; k < e; ++k) out_indices[acc + (k - s)] = indices[k];
+    acc += e - s;
+  }
+  out_indptr[n] = acc;
+  return acc;
 }

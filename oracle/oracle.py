@@ -16,7 +16,7 @@ __all__ = [
     "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
     "sample_neighbors", "sample_positions", "relabel", "gather_rows",
     "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
-    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm",
+    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows",
 ]
 
 
@@ -290,3 +290,24 @@ def sddmm(op, row, col, lhs, rhs, coo_offset=None, lhs_offset=None, rhs_offset=N
     lib().orc_sddmm(C.c_int(op), _p(row), _p(col), C.c_int64(E), _p(lhs), _p(rhs), C.c_int64(dim),
                     _p(coo), _p(lo), _p(ro), C.c_int(len(coo) - 1), _p(out))
     return out
+
+
+def count_ids(ids, freq):
+    """freq[ids] += 1 in place (ids outside the table ignored)."""
+    v = _i64(ids)
+    assert freq.dtype == np.int64 and freq.flags.c_contiguous
+    lib().orc_count_ids(_p(v), C.c_int64(len(v)), _p(freq), C.c_int64(len(freq)))
+    return freq
+
+
+def csr_select_rows(graph, rows):
+    """-> (indptr, indices) of the chosen nodes' adjacency rows."""
+    r = _i64(rows)
+    out_indptr = np.zeros(len(r) + 1, dtype=np.int64)
+    lib().orc_csr_select_rows.restype = C.c_int64
+    args = [_p(graph.indptr), _p(graph.indices), C.c_int64(graph.row_begin), C.c_int64(graph.num_rows),
+            _p(r), C.c_int64(len(r)), _p(out_indptr)]
+    total = lib().orc_csr_select_rows(*args, None)
+    out_indices = np.empty(total, dtype=np.int64)
+    lib().orc_csr_select_rows(*args, _p(out_indices))
+    return out_indptr, out_indices
