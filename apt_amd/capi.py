@@ -62,9 +62,13 @@ SYMBOLS = {
     "apt_count_ids": (_I, [_P, _I64, _P, _P, _I64, _P]),
     "apt_csr_row_degrees": (_I, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "apt_csr_copy_rows": (_I, [_P, _P, _I64, _P, _I64, _P, _I64, _P, _P]),
+    "apt_block_workspace_bytes": (_SZ, [_I64, _I, _I64, _I]),
+    "apt_block_formats": (_I, [_P, _I64, _P, _I, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
     "apt_spmm_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I64, _I, _I, _P, _P]),
     "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
+    "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
+    "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
@@ -506,3 +510,91 @@ def csr_select_rows(graph, rows):
     check(lib().apt_csr_copy_rows(_ptr(graph.indptr), _ptr(graph.indices), graph.row_begin, _ptr(rows), n,
                                   _ptr(out_indptr), total, _ptr(out_indices), _stream()))
     return out_indptr, out_indices
+
+
+class BlockFormats:
+    """COO / CSC / CSR of one hop's fixed-stride block (apt_block_formats).
+    Buffers are sized for the upper bounds and reused by every emit(); the edge
+    count stays on the device (num_edges).  narrow() waits and cuts to size."""
+
+    def __init__(self, num_dst, fanout, num_src, want_csr=True, device="cuda:0"):
+        self.num_dst, self.fanout, self.num_src, self.want_csr = int(num_dst), int(fanout), int(num_src), want_csr
+        i64 = dict(dtype=torch.int64, device=device)
+        slots = max(self.num_dst * self.fanout, 1)
+        self.coo_row, self.coo_col = torch.empty(slots, **i64), torch.empty(slots, **i64)
+        self.csc_indptr = torch.empty(self.num_dst + 1, **i64)
+        self.num_edges = torch.zeros(1, **i64)
+        self.csr_indptr = torch.empty(self.num_src + 1, **i64) if want_csr else None
+        self.csr_indices = torch.empty(slots, **i64) if want_csr else None
+        self.csr_eids = torch.empty(slots, **i64) if want_csr else None
+        need = int(lib().apt_block_workspace_bytes(self.num_dst, self.fanout, self.num_src, int(want_csr)))
+        if need == 0 and slots > 1:
+            raise AptError("block formats: sizes out of range")
+        self.workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=device)
+
+    def emit(self, relabeled, num_dst_dev=None):
+        """Asynchronous."""
+        relabeled = _dev_i64(relabeled, "relabeled")
+        if relabeled.numel() < self.num_dst * self.fanout:
+            raise AptError("block formats: relabeled is shorter than num_dst * fanout")
+        check(lib().apt_block_formats(_ptr(relabeled), self.num_dst, _ptr(num_dst_dev), self.fanout, self.num_src,
+                                      _ptr(self.coo_row), _ptr(self.coo_col), _ptr(self.csc_indptr),
+                                      _ptr(self.num_edges), _ptr(self.csr_indptr), _ptr(self.csr_indices),
+                                      _ptr(self.csr_eids), _ptr(self.workspace), self.workspace.numel(), _stream()))
+        return self
+
+    def narrow(self, num_dst=None, num_src=None):
+        """-> dict of the formats cut to the real sizes (waits for the stream)."""
+        e = int(self.num_edges.item())
+        nd = self.num_dst if num_dst is None else int(num_dst)
+        ns = self.num_src if num_src is None else int(num_src)
+        out = dict(num_edges=e, coo_row=self.coo_row[:e], coo_col=self.coo_col[:e], csc_indptr=self.csc_indptr[:nd + 1])
+        if self.want_csr:
+            out.update(csr_indptr=self.csr_indptr[:ns + 1], csr_indices=self.csr_indices[:e], csr_eids=self.csr_eids[:e])
+        return out
+
+
+def block_formats(relabeled, num_dst, fanout, num_src, want_csr=True, num_dst_dev=None):
+    """One-shot form of BlockFormats: allocates, emits, narrows."""
+    f = BlockFormats(num_dst, fanout, num_src, want_csr, device=relabeled.device)
+    nd = num_dst if num_dst_dev is None else int(num_dst_dev.item())
+    return f.emit(relabeled, num_dst_dev).narrow(num_dst=nd)
+
+
+def _f32(t, name):
+    if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float32):
+        raise TypeError(f"{name} must be a contiguous fp32 GPU tensor")
+    return t
+
+
+def gat_scores(x, attn):
+    """(x * attn).sum(-1): x [n, heads, dim] fp32 / bf16, attn [heads, dim] fp32 -> fp32 [n, heads]."""
+    if not (x.is_cuda and x.is_contiguous() and x.dim() == 3 and x.dtype in (torch.float32, torch.bfloat16)):
+        raise TypeError("x must be a contiguous [n, heads, dim] fp32 or bf16 GPU tensor")
+    attn = _f32(attn, "attn")
+    n, heads, dim = x.shape
+    if tuple(attn.shape) != (heads, dim):
+        raise AptError("gat_scores: attn must be [heads, dim]")
+    out = torch.empty((n, heads), dtype=torch.float32, device=x.device)
+    check(lib().apt_gat_scores(_ptr(x), n, heads, dim, x.element_size(), _ptr(attn), _ptr(out), _stream()))
+    return out
+
+
+def gat_block(neighbors, num_dst, fanout, ft, el, er, negative_slope=0.2, num_dst_dev=None, want_attn=False):
+    """Edge-softmax aggregation of a GAT layer over a fixed-stride block (see
+    apt_gat_block) -> fp32 [num_dst, heads, dim] (, attention [num_dst * fanout, heads])."""
+    neighbors = _dev_i64(neighbors, "neighbors")
+    if not (ft.is_cuda and ft.is_contiguous() and ft.dim() == 3 and ft.dtype in (torch.float32, torch.bfloat16)):
+        raise TypeError("ft must be a contiguous [num_src, heads, dim] fp32 or bf16 GPU tensor")
+    el, er = _f32(el, "el"), _f32(er, "er")
+    num_src, heads, dim = ft.shape
+    if neighbors.numel() < num_dst * fanout:
+        raise AptError("gat_block: neighbors shorter than num_dst * fanout")
+    if tuple(el.shape) != (num_src, heads) or tuple(er.shape) != (num_dst, heads):
+        raise AptError("gat_block: el must be [num_src, heads] and er [num_dst, heads]")
+    out = torch.empty((num_dst, heads, dim), dtype=torch.float32, device=ft.device)
+    attn = torch.empty((num_dst * fanout, heads), dtype=torch.float32, device=ft.device) if want_attn else None
+    check(lib().apt_gat_block(_ptr(neighbors), int(num_dst), _ptr(num_dst_dev), int(fanout), _ptr(ft), num_src,
+                              heads, dim, ft.element_size(), _ptr(el), _ptr(er), float(negative_slope), _ptr(out),
+                              _ptr(attn), _stream()))
+    return (out, attn) if want_attn else out

@@ -22,6 +22,8 @@ int tuning_gather_rows() { return g_gather_rows; }
 int tuning_gather_max_blocks() { return g_gather_max_blocks; }
 int tuning_fuse_mark() { return g_fuse_mark; }
 int tuning_payload_bits() { return g_payload_bits; }
+static int g_block_fused_scan = 1;
+int tuning_block_fused_scan() { return g_block_fused_scan; }
 
 }  // namespace apt
 
@@ -50,6 +52,10 @@ extern "C" int apt_set_tuning(const char* key, int value) {
   }
   if (std::strcmp(key, "minibatch_fuse_mark") == 0) {
     apt::g_fuse_mark = value != 0;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "block_fused_scan") == 0) {
+    apt::g_block_fused_scan = value != 0;
     return APT_OK;
   }
   if (std::strcmp(key, "gather_max_blocks") == 0) {

@@ -246,6 +246,133 @@ static void launch_ell(const int64_t* nbr, int64_t num_dst, const int64_t* num_d
 #undef APT_ELL
 }
 
+// GAT attention logits: out[r, h] = sum_d x[r, h, d] * attn[h, d]
+// (python/npc/model/gatconv.py:116-117: (feat * attn).sum(-1)).  A wavefront per
+// (row, head); lanes stride over d and reduce with shuffles in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(kAggBlock) void gat_scores_kernel(const T* __restrict__ x, int64_t num_rows,
+                                                               int heads, int64_t dim,
+                                                               const float* __restrict__ attn,
+                                                               float* __restrict__ out) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t items = num_rows * heads;
+  for (int64_t it = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave; it < items;
+       it += static_cast<int64_t>(gridDim.x) * kAggWaves) {
+    const int h = static_cast<int>(it % heads);
+    float acc = 0.f;
+    for (int64_t d = lane; d < dim; d += kWave) acc += to_float<T>(x[it * dim + d]) * attn[h * dim + d];
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) acc += __shfl_down(acc, off, kWave);
+    if (lane == 0) out[it] = acc;
+  }
+}
+
+// GATConv aggregation over a fixed-stride block (gatconv.py:118-126, DGL's
+// u_add_v -> LeakyReLU -> edge_softmax -> u_mul_e + sum): for destination i and
+// head h, e_k = leaky(el[src_k, h] + er[i, h]) over the row's slots, a = softmax(e),
+// out[i, h, :] = sum_k a_k * ft[src_k, h, :].  A lane group owns a destination
+// row (all heads); the softmax runs online over the slots (running maximum,
+// rescaled sum), so a row's features are read once and nothing is written but
+// the result: no per-edge score, exponent or weight arrays, no atomics.
+template <typename T, int VEC, int LPR>
+__global__ __launch_bounds__(kAggBlock) void gat_ell_kernel(const int64_t* __restrict__ nbr, int64_t num_dst,
+                                                            const int64_t* num_dst_dev, int fanout,
+                                                            const T* __restrict__ ft, int64_t num_src,
+                                                            int heads, int64_t dim,
+                                                            const float* __restrict__ el,
+                                                            const float* __restrict__ er, float slope,
+                                                            float* __restrict__ out,
+                                                            float* __restrict__ attn_out) {
+  constexpr int kGroups = kAggBlock / LPR;
+  constexpr int kUnroll = 5;
+  const int64_t n = actual_count(num_dst, num_dst_dev);
+  const int64_t row_len = static_cast<int64_t>(heads) * dim;
+  const int grp = threadIdx.x / LPR, l = threadIdx.x % LPR;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kGroups + grp; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kGroups) {
+    const int64_t* ids = nbr + i * fanout;
+    for (int64_t d = static_cast<int64_t>(l) * VEC; d < row_len; d += LPR * VEC) {
+      const int h = static_cast<int>(d / dim);   // VEC divides dim: a lane's features share a head
+      const float er_i = er[i * heads + h];
+      float acc[VEC];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
+      float top = -INFINITY, denom = 0.f;
+      for (int s0 = 0; s0 < fanout; s0 += kUnroll) {
+        float v[kUnroll][VEC];
+        float sc[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          ok[u] = false;
+          sc[u] = 0.f;
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) v[u][k] = 0.f;
+          if (s0 + u < fanout) {
+            const int64_t src = ids[s0 + u];
+            if (src >= 0 && src < num_src) {
+              ok[u] = true;
+              sc[u] = el[src * heads + h];
+              load_vec<T, VEC>(ft, src * row_len + d, v[u]);
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          if (!ok[u]) continue;
+          float e = sc[u] + er_i;
+          e = e > 0.f ? e : e * slope;
+          if (e > top) {
+            const float shrink = expf(top - e);   // 0 on the first edge (top = -inf)
+            denom *= shrink;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] *= shrink;
+            top = e;
+          }
+          const float w = expf(e - top);
+          denom += w;
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) acc[k] += w * v[u][k];
+        }
+      }
+      const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) out[i * row_len + d + k] = acc[k] * inv;
+      // the lane that holds a head's first features also writes its attention weights
+      if (attn_out != nullptr && d % dim == 0) {
+        for (int s = 0; s < fanout; ++s) {
+          const int64_t src = ids[s];
+          float a = 0.f;
+          if (src >= 0 && src < num_src) {
+            float e = el[src * heads + h] + er_i;
+            e = e > 0.f ? e : e * slope;
+            a = expf(e - top) * inv;
+          }
+          attn_out[(i * fanout + s) * heads + h] = a;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int VEC>
+static void launch_gat(const int64_t* nbr, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+                       const void* ft, int64_t num_src, int heads, int64_t dim, const float* el,
+                       const float* er, float slope, float* out, float* attn_out, hipStream_t st) {
+  const int64_t per_row = ceil_div(static_cast<int64_t>(heads) * dim, VEC);
+  const T* x = static_cast<const T*>(ft);
+#define APT_GAT(LPR)                                                                                  \
+  hipLaunchKernelGGL((gat_ell_kernel<T, VEC, LPR>),                                                   \
+                     dim3(static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst, kAggBlock / LPR), 1 << 20))), \
+                     dim3(kAggBlock), 0, st, nbr, num_dst, num_dst_dev, fanout, x, num_src, heads, dim, el, er, \
+                     slope, out, attn_out)
+  if (per_row <= 8) APT_GAT(8);
+  else if (per_row <= 16) APT_GAT(16);
+  else if (per_row <= 32) APT_GAT(32);
+  else APT_GAT(64);
+#undef APT_GAT
+}
+
 static int agg_check(const char* who, const int64_t* row, const int64_t* col, int64_t E, const void* in,
                      float* out, const int64_t* coo_off, int num_seg, int64_t dim, int elem_size) {
   APT_REQUIRE(E >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (E %lld, dim %lld)", who, (long long)E,
@@ -353,5 +480,56 @@ extern "C" int apt_spmm_block(const int64_t* neighbors, int64_t num_dst, const i
     else launch_ell<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
   }
   APT_LAUNCH_CHECK("spmm_ell_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_gat_scores(const void* x, int64_t num_rows, int heads, int64_t dim, int elem_size,
+                              const float* attn, float* out, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_rows >= 0 && heads > 0 && dim > 0, APT_EINVAL,
+              "apt_gat_scores: bad shape (rows %lld, heads %d, dim %lld)", (long long)num_rows, heads,
+              (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_gat_scores: elem_size %d (4 = fp32, 2 = bf16)",
+              elem_size);
+  if (num_rows == 0) return APT_OK;
+  APT_REQUIRE(x != nullptr && attn != nullptr && out != nullptr, APT_EINVAL, "apt_gat_scores: a tensor is NULL");
+  const unsigned blocks =
+      static_cast<unsigned>(std::min<int64_t>(ceil_div(num_rows * heads, kAggWaves), 1 << 20));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (elem_size == 4)
+    hipLaunchKernelGGL(gat_scores_kernel<float>, dim3(blocks), dim3(kAggBlock), 0, st,
+                       static_cast<const float*>(x), num_rows, heads, dim, attn, out);
+  else
+    hipLaunchKernelGGL(gat_scores_kernel<uint16_t>, dim3(blocks), dim3(kAggBlock), 0, st,
+                       static_cast<const uint16_t*>(x), num_rows, heads, dim, attn, out);
+  APT_LAUNCH_CHECK("gat_scores_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+                             const void* ft, int64_t num_src, int heads, int64_t dim, int elem_size,
+                             const float* el, const float* er, float negative_slope, float* out,
+                             float* attn_out, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_dst >= 0 && fanout > 0 && heads > 0 && dim > 0 && num_src >= 0, APT_EINVAL,
+              "apt_gat_block: bad shape (num_dst %lld, fanout %d, heads %d, dim %lld)", (long long)num_dst,
+              fanout, heads, (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_gat_block: elem_size %d (4 = fp32, 2 = bf16)",
+              elem_size);
+  if (num_dst == 0) return APT_OK;
+  APT_REQUIRE(neighbors != nullptr && out != nullptr && er != nullptr &&
+                  ((ft != nullptr && el != nullptr) || num_src == 0),
+              APT_EINVAL, "apt_gat_block: a tensor is NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(ft) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (elem_size == 4) {
+    if (vec4) launch_gat<float, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+    else launch_gat<float, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+  } else {
+    if (vec4) launch_gat<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+    else launch_gat<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+  }
+  APT_LAUNCH_CHECK("gat_ell_kernel");
   return APT_OK;
 }

@@ -22,7 +22,7 @@ from . import capi
 
 class MiniBatchPipeline:
     def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
-                 use_graph=False, requests=None):
+                 use_graph=False, requests=None, formats=False):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
         --fan_out list reversed).
 
@@ -32,7 +32,11 @@ class MiniBatchPipeline:
         src/load_subtensor.cc:41-56,83-86): bucket 0 = rows present on this GPU,
         which are gathered; the other buckets are the per-owner request lists
         that the reference would send (left in `request_ids`, grouped by
-        bucket, sizes in `request_sizes`)."""
+        bucket, sizes in `request_sizes`).
+
+        formats: True or "csc" also emits every hop's block as COO + CSC (+ CSR
+        with True), what DGL derives from (row, col) in the reference
+        (python/npc/sampler.py:59-69); result() then carries them per block."""
         self.graph, self.feat = graph, feat
         self.fanouts = [int(f) for f in hop_fanouts]
         self.replace = bool(replace)
@@ -73,6 +77,15 @@ class MiniBatchPipeline:
             self.request_perm = torch.empty(self.caps[-1], **i64)
             need = int(capi.lib().apt_bucket_workspace_bytes(self.caps[-1], R))
             self.request_ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        self.formats = None
+        if formats:
+            self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=formats != "csc", device=dev)
+                            for h, f in enumerate(self.fanouts)]
+            # a hop's formats are a string of small dependent launches: the hops run beside each other
+            # (and beside the gather) on streams of their own
+            self.format_streams = [torch.cuda.Stream(device=dev) for _ in self.fanouts]
+            self.format_fork = torch.cuda.Event()
+            self.format_done = [torch.cuda.Event() for _ in self.fanouts]
         self.seeds = None
         self.graph_exec = None
         if use_graph:
@@ -103,14 +116,17 @@ class MiniBatchPipeline:
         self.static_seeds = torch.zeros(self.caps[0], dtype=torch.int64, device=self.device)
         # run once eagerly so lazy initialisation happens outside the capture
         self.plan.launch(self.static_seeds, rng_seed=None)
+        self.emit_formats()
         if self.features is not None:
             self.gather()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             self.plan.launch(self.static_seeds, rng_seed=None)
+            self.emit_formats(join=False)
             if self.features is not None:
                 self.gather()
+            self.join_formats()
         self.graph_exec = g
 
     # ------------------------------------------------------------ public
@@ -123,6 +139,29 @@ class MiniBatchPipeline:
             self.plan.launch(seeds, rng_seed)
         else:
             self._sample_unfused(seeds, rng_seed)
+
+    def emit_formats(self, join=True):
+        """COO / CSC / CSR of every hop's block, asynchronous (no-op unless asked
+        for).  Each hop is emitted on its own stream once the current stream has
+        finished sampling; join=False leaves the current stream free to go on (the
+        gather) and the caller joins later with join_formats()."""
+        if self.formats is None:
+            return
+        self.format_fork.record()
+        for h, fmt in enumerate(self.formats):
+            with torch.cuda.stream(self.format_streams[h]):
+                self.format_streams[h].wait_event(self.format_fork)
+                fmt.emit(self.relabeled[h], self._size(h))
+                self.format_done[h].record()
+        if join:
+            self.join_formats()
+
+    def join_formats(self):
+        """The current stream waits for the formats (before the buffers are reused)."""
+        if self.formats is not None:
+            cur = torch.cuda.current_stream()
+            for e in self.format_done:
+                cur.wait_event(e)
 
     def gather(self):
         """Features of the input nodes (the last hop's unique ids), asynchronous."""
@@ -149,8 +188,10 @@ class MiniBatchPipeline:
             self.graph_exec.replay()
             return
         self.sample(seeds, rng_seed)
+        self.emit_formats(join=False)
         if self.features is not None:
             self.gather()
+        self.join_formats()
 
     def result(self):
         """Waits for the batch and narrows the buffers to their real sizes ->
@@ -168,6 +209,8 @@ class MiniBatchPipeline:
             blocks.insert(0, dict(seeds=src, neighbors=self.neighbors[h][:n * f],
                                   relabeled=self.relabeled[h][:n * f], counts=self.counts[h][:n],
                                   unique=uniq, fanout=f))
+            if self.formats is not None:
+                blocks[0]["formats"] = self.formats[h].narrow(num_dst=n, num_src=sizes[h + 1])
         feats = None if self.features is None else self.features[:sizes[H]]
         inp = self.nodes[:sizes[H]] if self.fused else self.frontier[H][:sizes[H]]
         out = dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],

@@ -63,6 +63,8 @@ def parse_args():
     ap.add_argument("--calibration_copy_mib", type=int, default=0,
                     help="also launch the plain copy kernel once on this many MiB (for scaling "
                          "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
+    ap.add_argument("--formats", action="store_true",
+                    help="also time the emission of every hop's block as COO + CSC (+ CSR)")
     ap.add_argument("--aggregation", action="store_true",
                     help="also time GraphSAGE-style SpMM (hidden 256, fp32 and bf16) and SDDMM on the "
                          "outermost sampled block of the last batch")
@@ -319,6 +321,31 @@ def main():
         agg["sddmm_u_add_v_fp32_GBps"] = (3 * E * hid * 4 + 16 * E) / t / 1e9
         del h, hd
 
+    # ---- optional: every hop's block as COO + CSC (+ CSR), device-side sizes, after sampling
+    fmt = None
+    if args.formats:
+        fmt = {}
+        for name, what in (("coo_csc", "csc"), ("coo_csc_csr", True)):
+            fp = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, formats=what, requests=requests)
+            t = 0.0
+            for i in range(W + K):
+                m = (ev(), ev())
+                fp.sample(seed_sets[i], args.seed + 100 + i)
+                m[0].record()
+                fp.emit_formats()
+                m[1].record()
+                torch.cuda.synchronize()
+                if i >= W:
+                    t += m[0].elapsed_time(m[1])
+            fmt[name + "_ms"] = t / K                       # the hops beside each other, nothing else running
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(K):
+                fp.run(seed_sets[W + i], args.seed + 100 + W + i)
+            torch.cuda.synchronize()
+            fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
+            del fp
+
     # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
     cpu = None
     budget = args.cpu_seconds
@@ -401,6 +428,7 @@ def main():
         },
         "cpu_baseline": cpu,
         "aggregation": agg,
+        "block_formats": fmt,
         "stages": {
             "in_flight": in_flight,
             "edges_per_step": edges / K,

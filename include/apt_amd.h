@@ -53,7 +53,11 @@ int apt_abi_version(void);
  *                            between table refills (used to test the refill)
  *   "minibatch_fuse_mark"    1 (default; note: 0 here also means "off", not
  *                            "default") the sampling kernel of apt_minibatch_sample
- *                            also does the rank-table lookup / bid of each id */
+ *                            also does the rank-table lookup / bid of each id
+ *   "block_fused_scan"       1 (default; 0 = off) apt_block_formats lets its place
+ *                            and scatter workgroups add up the tile counts
+ *                            themselves when there are few tiles; off = always
+ *                            the separate scan launches of large inputs */
 int apt_set_tuning(const char* key, int value);
 
 /* A CSR (CSC in the reference's naming: row v lists the in-neighbours of v)
@@ -304,6 +308,31 @@ int apt_csr_copy_rows(const int64_t* indptr, const int64_t* indices, int64_t row
                       const int64_t* rows, int64_t n, const int64_t* out_indptr,
                       int64_t num_out_edges, int64_t* out_indices, void* stream);
 
+/* Sparse formats of a sampled block.  The reference hands (row, col) of a hop to
+ * DGL, which materialises COO, CSR and CSC (python/npc/sampler.py:59-69,76-91;
+ * create_block_from_csc :44-56 takes a CSC as it is).  Input is the hop's
+ * fixed-stride block: relabeled[d * fanout + k] = k-th source of destination d,
+ * negative where d has fewer neighbours.
+ *   coo_row, coo_col   int64[num_dst * fanout]: edges in destination-major order,
+ *                      row = source, col = destination; *num_edges_dev of them
+ *   csc_indptr         int64[num_dst + 1] over destinations (its indices are
+ *                      coo_row, its edge ids 0..E-1)
+ *   csr_indptr         int64[num_src + 1] over sources, or NULL for no CSR;
+ *   csr_indices, csr_eids  int64[num_dst * fanout]: destination and COO position of
+ *                      every edge grouped by source, edges of one source by
+ *                      increasing edge id (deterministic)
+ * num_dst / num_src are upper bounds when the real counts live on the device
+ * (num_dst_dev as n_dev in apt_sample_neighbors; sources need no count): the
+ * offsets of rows past the real counts equal the edge total, i.e. empty rows.
+ * workspace: apt_block_workspace_bytes(num_dst, fanout, num_src, csr != NULL)
+ * bytes of device scratch; 0 = sizes out of range. */
+size_t apt_block_workspace_bytes(int64_t num_dst, int fanout, int64_t num_src, int want_csr);
+int apt_block_formats(const int64_t* relabeled, int64_t num_dst, const int64_t* num_dst_dev,
+                      int fanout, int64_t num_src, int64_t* coo_row, int64_t* coo_col,
+                      int64_t* csc_indptr, int64_t* num_edges_dev, int64_t* csr_indptr,
+                      int64_t* csr_indices, int64_t* csr_eids, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* Aggregation over the COO edges of sampled blocks (optional stage).
  * Replaces CopyUSum / CopyESum / UMulESum (src/spmm.cc:9-42, src/cuda/spmm.cu:8-148)
  * and UAddV / UMulV (src/sddmm.cc:9-31, src/cuda/sddmm.cu:8-103).
@@ -344,6 +373,28 @@ int apt_sddmm(int op, const int64_t* coo_row, const int64_t* coo_col, int64_t nu
               const void* lhs, int64_t num_lhs_rows, const void* rhs, int64_t num_rhs_rows,
               int64_t dim, int elem_size, const int64_t* coo_offset, const int64_t* lhs_offset,
               const int64_t* rhs_offset, int num_segments, float* out, void* stream);
+
+/* GATConv aggregation (optional stage).  The reference's GAT layer computes its
+ * attention with DGL on the sampled block (python/npc/model/gatconv.py:116-126):
+ * el = (ft * attn_l).sum(-1), er likewise on the destination rows,
+ * e = LeakyReLU(el[src] + er[dst]), a = edge_softmax over the in-edges of a
+ * destination, out[dst] = sum a * ft[src].
+ *   apt_gat_scores  out[r, h] = sum_d x[r, h, d] * attn[h, d]; x is
+ *                   [num_rows, heads, dim] fp32 or bf16, attn and out fp32
+ *   apt_gat_block   the rest, fused, over the sampler's fixed-stride block
+ *                   (neighbors / num_dst / num_dst_dev / fanout as in
+ *                   apt_spmm_block): ft [num_src, heads, dim] fp32 or bf16,
+ *                   el [num_src, heads], er [num_dst, heads] fp32,
+ *                   out [num_dst, heads, dim] fp32 (zero rows for destinations
+ *                   without neighbours); attn_out, optional (NULL = not wanted):
+ *                   [num_dst * fanout, heads] fp32 attention weights, 0 in empty
+ *                   slots.  fp32 accumulation, fixed summation order. */
+int apt_gat_scores(const void* x, int64_t num_rows, int heads, int64_t dim, int elem_size,
+                   const float* attn, float* out, void* stream);
+int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+                  const void* ft, int64_t num_src, int heads, int64_t dim, int elem_size,
+                  const float* el, const float* er, float negative_slope, float* out,
+                  float* attn_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,9 @@
  *   orc_cluster_*       numpy searchsorted + stable argsort closed form; the
  *                       inputs of tests/test_shuffle_seeds.cc:19-26.
  *   orc_permute/scatter numpy take / put.
+ *   orc_gat_scores/_block  scipy.special.softmax on a dense adjacency, the mean
+ *                       SpMM when all logits are equal, shift invariance.
+ *   orc_block_formats   numpy nonzero / stable argsort / bincount + cumsum.
  *   orc_count_ids, orc_csr_select_rows   numpy bincount / concatenated slices.
  *   orc_spmm_sum/sddmm  numpy closed forms (np.add.at over fancy-indexed rows,
  *                       in float64); a sum over a row of ones equals its
@@ -32,6 +35,7 @@
  * Build: make -C oracle   (gcc -O3 -fopenmp -shared -fPIC)
  */
 #include <stdint.h>
+#include <math.h>
 #include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
@@ -474,4 +478,93 @@ int64_t orc_csr_select_rows(const int64_t* indptr, const int64_t* indices, int64
   }
   out_indptr[n] = acc;
   return acc;
+}
+
+/* ------------------------------------------------------------------ */
+/* Sparse formats of a block (python/npc/sampler.py:59-69,76-91: DGL   */
+/* builds coo/csr/csc from row = relabeled, col = dst).  Pinned by      */
+/* numpy closed forms (nonzero, stable argsort, bincount + cumsum).     */
+/* ------------------------------------------------------------------ */
+/* Arrays hold num_dst * fanout entries (offsets num_dst + 1 / num_src + 1);
+ * returns the number of edges.  csr_* may be NULL. */
+int64_t orc_block_formats(const int64_t* relabeled, int64_t num_dst, int fanout, int64_t num_src,
+                          int64_t* coo_row, int64_t* coo_col, int64_t* csc_indptr, int64_t* csr_indptr,
+                          int64_t* csr_indices, int64_t* csr_eids) {
+  int64_t e = 0;
+  for (int64_t d = 0; d < num_dst; ++d) {
+    csc_indptr[d] = e;
+    for (int k = 0; k < fanout; ++k) {
+      const int64_t v = relabeled[d * fanout + k];
+      if (v < 0) continue;
+      coo_row[e] = v;
+      coo_col[e] = d;
+      ++e;
+    }
+  }
+  csc_indptr[num_dst] = e;
+  if (!csr_indptr) return e;
+  for (int64_t s = 0; s <= num_src; ++s) csr_indptr[s] = 0;
+  for (int64_t i = 0; i < e; ++i) csr_indptr[coo_row[i] + 1] += 1;
+  for (int64_t s = 0; s < num_src; ++s) csr_indptr[s + 1] += csr_indptr[s];
+  int64_t* next = (int64_t*)malloc(sizeof(int64_t) * (size_t)(num_src > 0 ? num_src : 1));
+  for (int64_t s = 0; s < num_src; ++s) next[s] = csr_indptr[s];
+  for (int64_t i = 0; i < e; ++i) {   /* edge order = increasing edge id inside a source */
+    const int64_t at = next[coo_row[i]]++;
+    csr_indices[at] = coo_col[i];
+    csr_eids[at] = i;
+  }
+  free(next);
+  return e;
+}
+
+/* ------------------------------------------------------------------ */
+/* GAT aggregation (python/npc/model/gatconv.py:116-126; the arithmetic */
+/* is DGL's: u_add_v, LeakyReLU, edge_softmax, u_mul_e + sum).  Double   */
+/* accumulation.  Pinned by scipy.special.softmax on a dense adjacency,  */
+/* by the mean SpMM (all logits equal) and by shift invariance.          */
+/* ------------------------------------------------------------------ */
+void orc_gat_scores(const float* x, int64_t n, int heads, int64_t dim, const float* attn, float* out) {
+  for (int64_t r = 0; r < n; ++r)
+    for (int h = 0; h < heads; ++h) {
+      double acc = 0.0;
+      for (int64_t d = 0; d < dim; ++d) acc += (double)x[(r * heads + h) * dim + d] * (double)attn[h * dim + d];
+      out[r * heads + h] = (float)acc;
+    }
+}
+
+/* attn_out may be NULL */
+void orc_gat_block(const int64_t* nbr, int64_t num_dst, int fanout, const float* ft, int64_t num_src, int heads,
+                   int64_t dim, const float* el, const float* er, double slope, float* out, float* attn_out) {
+  double* e = (double*)malloc(sizeof(double) * (size_t)(fanout > 0 ? fanout : 1));
+  double* acc = (double*)malloc(sizeof(double) * (size_t)dim);
+  for (int64_t i = 0; i < num_dst; ++i)
+    for (int h = 0; h < heads; ++h) {
+      double top = -INFINITY, denom = 0.0;
+      for (int k = 0; k < fanout; ++k) {
+        const int64_t s = nbr[i * fanout + k];
+        if (s < 0 || s >= num_src) continue;
+        double v = (double)el[s * heads + h] + (double)er[i * heads + h];
+        if (v < 0) v *= slope;
+        e[k] = v;
+        if (v > top) top = v;
+      }
+      for (int k = 0; k < fanout; ++k) {
+        const int64_t s = nbr[i * fanout + k];
+        if (s < 0 || s >= num_src) continue;
+        denom += exp(e[k] - top);
+      }
+      for (int64_t d = 0; d < dim; ++d) acc[d] = 0.0;
+      for (int k = 0; k < fanout; ++k) {
+        const int64_t s = nbr[i * fanout + k];
+        double a = 0.0;
+        if (s >= 0 && s < num_src) {
+          a = exp(e[k] - top) / denom;
+          for (int64_t d = 0; d < dim; ++d) acc[d] += a * (double)ft[(s * heads + h) * dim + d];
+        }
+        if (attn_out) attn_out[(i * fanout + k) * heads + h] = (float)a;
+      }
+      for (int64_t d = 0; d < dim; ++d) out[(i * heads + h) * dim + d] = (float)acc[d];
+    }
+  free(e);
+  free(acc);
 }

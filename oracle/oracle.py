@@ -16,7 +16,7 @@ __all__ = [
     "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
     "sample_neighbors", "sample_positions", "relabel", "gather_rows",
     "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
-    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows",
+    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows", "block_formats", "gat_scores", "gat_block",
 ]
 
 
@@ -311,3 +311,44 @@ def csr_select_rows(graph, rows):
     out_indices = np.empty(total, dtype=np.int64)
     lib().orc_csr_select_rows(*args, _p(out_indices))
     return out_indptr, out_indices
+
+
+def block_formats(relabeled, num_dst, fanout, num_src, want_csr=True):
+    """COO / CSC / CSR of a fixed-stride block -> dict of int64 arrays."""
+    r = _i64(relabeled)
+    assert len(r) == num_dst * fanout
+    slots = max(len(r), 1)
+    coo_row, coo_col = np.empty(slots, np.int64), np.empty(slots, np.int64)
+    csc = np.empty(num_dst + 1, np.int64)
+    csr = np.empty(num_src + 1, np.int64) if want_csr else None
+    ci, ce = (np.empty(slots, np.int64), np.empty(slots, np.int64)) if want_csr else (None, None)
+    lib().orc_block_formats.restype = C.c_int64
+    e = lib().orc_block_formats(_p(r), C.c_int64(num_dst), C.c_int(fanout), C.c_int64(num_src), _p(coo_row),
+                                _p(coo_col), _p(csc), _p(csr) if want_csr else None,
+                                _p(ci) if want_csr else None, _p(ce) if want_csr else None)
+    out = dict(num_edges=int(e), coo_row=coo_row[:e], coo_col=coo_col[:e], csc_indptr=csc)
+    if want_csr:
+        out.update(csr_indptr=csr, csr_indices=ci[:e], csr_eids=ce[:e])
+    return out
+
+
+def gat_scores(x, attn):
+    """(x * attn).sum(-1): x [n, heads, dim], attn [heads, dim] -> float32 [n, heads]."""
+    x, attn = _f32(x), _f32(attn)
+    n, heads, dim = x.shape
+    out = np.empty((n, heads), dtype=np.float32)
+    lib().orc_gat_scores(_p(x), C.c_int64(n), C.c_int(heads), C.c_int64(dim), _p(attn), _p(out))
+    return out
+
+
+def gat_block(neighbors, num_dst, fanout, ft, el, er, negative_slope=0.2, want_attn=False):
+    """GATConv aggregation over a fixed-stride block -> float32 [num_dst, heads, dim]
+    (, attention [num_dst * fanout, heads])."""
+    nbr, ft, el, er = _i64(neighbors), _f32(ft), _f32(el), _f32(er)
+    num_src, heads, dim = ft.shape
+    assert len(nbr) >= num_dst * fanout and el.shape == (num_src, heads) and er.shape == (num_dst, heads)
+    out = np.empty((num_dst, heads, dim), dtype=np.float32)
+    attn = np.empty((num_dst * fanout, heads), dtype=np.float32) if want_attn else None
+    lib().orc_gat_block(_p(nbr), C.c_int64(num_dst), C.c_int(fanout), _p(ft), C.c_int64(num_src), C.c_int(heads),
+                        C.c_int64(dim), _p(el), _p(er), C.c_double(negative_slope), _p(out), _p(attn))
+    return (out, attn) if want_attn else out

@@ -125,3 +125,48 @@ def test_spmm_block_layout(orc, capi, dim, dtype):
     assert np.all(got.cpu().numpy()[cnt == 0] == 0)
     a = capi.spmm_block(dev(nbr.reshape(-1)), n_dst, f, x)
     assert torch.equal(a, got)                                       # fixed summation order
+
+
+def _ell(rng, n_dst, fanout, n_src, hole=0.25):
+    nbr = rng.integers(0, n_src, size=(n_dst, fanout)).astype(np.int64)
+    nbr[rng.random(nbr.shape) < hole] = -1
+    nbr[0, :] = -1
+    nbr[1, 1:] = -1
+    return nbr.reshape(-1)
+
+
+@pytest.mark.parametrize("heads,dim", [(4, 64), (1, 256), (3, 5), (8, 16), (2, 100)])
+def test_gat_fp32(orc, capi, heads, dim):
+    rng = np.random.default_rng(heads * 1000 + dim)
+    n_dst, fanout, n_src = 3000, 15, 20000
+    nbr = _ell(rng, n_dst, fanout, n_src)
+    ft = rng.standard_normal((n_src, heads, dim)).astype(np.float32)
+    al, ar = (rng.standard_normal((2, heads, dim)) * 0.3).astype(np.float32)
+    el, er = capi.gat_scores(dev(ft), dev(al)), capi.gat_scores(dev(ft[:n_dst]), dev(ar))
+    assert _close(el.cpu().numpy(), orc.gat_scores(ft, al), 1e-5)
+    assert _close(er.cpu().numpy(), orc.gat_scores(ft[:n_dst], ar), 1e-5)
+    h_el, h_er = el.cpu().numpy(), er.cpu().numpy()          # same logits into both, so only the block is compared
+    want, want_a = orc.gat_block(nbr, n_dst, fanout, ft, h_el, h_er, 0.2, want_attn=True)
+    got, got_a = capi.gat_block(dev(nbr), n_dst, fanout, dev(ft), el, er, 0.2, want_attn=True)
+    assert _close(got.cpu().numpy(), want, 1e-5)
+    assert np.max(np.abs(got_a.cpu().numpy() - want_a)) <= 1e-5
+    assert torch.equal(got, capi.gat_block(dev(nbr), n_dst, fanout, dev(ft), el, er, 0.2))   # reproducible
+    # device-side row count: rows past it are left alone
+    cnt = torch.tensor([1000], dtype=torch.int64, device=DEV)
+    part = capi.gat_block(dev(nbr), n_dst, fanout, dev(ft), el, er, 0.2, num_dst_dev=cnt)
+    assert torch.equal(part[:1000], got[:1000])
+
+
+def test_gat_bf16_config5_shape(orc, capi):
+    """4 heads x 64, bf16 features, fp32 accumulation: 1e-2 of the oracle on the same (rounded) inputs."""
+    rng = np.random.default_rng(11)
+    n_dst, fanout, n_src, heads, dim = 4000, 15, 30000, 4, 64
+    nbr = _ell(rng, n_dst, fanout, n_src)
+    ft16 = torch.from_numpy(rng.standard_normal((n_src, heads, dim)).astype(np.float32)).to(torch.bfloat16)
+    ft = ft16.to(torch.float32).numpy()
+    al, ar = (rng.standard_normal((2, heads, dim)) * 0.02).astype(np.float32)     # N(0, 0.02) weights
+    el, er = capi.gat_scores(ft16.to(DEV), dev(al)), capi.gat_scores(ft16[:n_dst].contiguous().to(DEV), dev(ar))
+    assert _close(el.cpu().numpy(), orc.gat_scores(ft, al), 1e-2)
+    want = orc.gat_block(nbr, n_dst, fanout, ft, el.cpu().numpy(), er.cpu().numpy(), 0.2)
+    got = capi.gat_block(dev(nbr), n_dst, fanout, ft16.to(DEV), el, er, 0.2)
+    assert _close(got.cpu().numpy(), want, 1e-2)

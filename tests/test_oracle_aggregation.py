@@ -48,3 +48,67 @@ def test_sddmm_closed_form(orc):
     rhs = rng.standard_normal((n_dst, 16)).astype(np.float32)
     assert np.array_equal(orc.sddmm(0, row, col, lhs, rhs), lhs[row] + rhs[col])
     assert np.array_equal(orc.sddmm(1, row, col, lhs, rhs), lhs[row] * rhs[col])
+
+
+def _ell_block(rng, n_dst, fanout, n_src, distinct=False, hole=0.25):
+    """Fixed-stride block; distinct=True: no source twice in a row."""
+    if distinct:
+        nbr = np.stack([rng.permutation(n_src)[:fanout] for _ in range(n_dst)]).astype(np.int64)
+    else:
+        nbr = rng.integers(0, n_src, size=(n_dst, fanout)).astype(np.int64)
+    nbr[rng.random(nbr.shape) < hole] = -1
+    nbr[0, :] = -1                                         # a destination without neighbours
+    nbr[1, 1:] = -1                                        # ... and with at most one
+    return nbr.reshape(-1)
+
+
+def test_gat_scores_and_block_pins(orc):
+    from scipy.special import softmax
+    rng = np.random.default_rng(7)
+    n_dst, fanout, n_src, heads, dim = 40, 6, 90, 3, 5
+    ft = rng.standard_normal((n_src, heads, dim)).astype(np.float32)
+    al, ar = rng.standard_normal((2, heads, dim)).astype(np.float32)
+    el, er = orc.gat_scores(ft, al), orc.gat_scores(ft[:n_dst], ar)
+    assert np.allclose(el, np.einsum("nhd,hd->nh", ft.astype(np.float64), al), rtol=1e-6, atol=1e-6)
+    # (1) dense statement with a library softmax: duplicate-free rows, so A[d, s] is one edge
+    nbr = _ell_block(rng, n_dst, fanout, n_src, distinct=True)
+    out, attn = orc.gat_block(nbr, n_dst, fanout, ft, el, er, 0.2, want_attn=True)
+    mask = np.zeros((n_dst, n_src), dtype=bool)
+    rows = np.repeat(np.arange(n_dst), fanout)
+    mask[rows[nbr >= 0], nbr[nbr >= 0]] = True
+    for h in range(heads):
+        z = el[None, :, h].astype(np.float64) + er[:, None, h]
+        z = np.where(z > 0, z, 0.2 * z)
+        z[~mask] = -np.inf
+        some = mask.any(1)
+        a = np.zeros_like(z)
+        a[some] = softmax(z[some], axis=1)
+        assert np.allclose(out[:, h, :], a @ ft[:, h, :].astype(np.float64), rtol=1e-6, atol=1e-6)
+        got_a = attn.reshape(n_dst, fanout, heads)[:, :, h]
+        assert np.allclose(got_a[nbr.reshape(n_dst, fanout) >= 0], a[rows[nbr >= 0], nbr[nbr >= 0]], rtol=1e-6, atol=1e-7)
+    assert np.all(out[0] == 0) and np.all(attn.reshape(n_dst, fanout, heads)[0] == 0)
+    # (2) equal logits -> plain mean over the row's edges (duplicates allowed), which the SpMM oracle computes
+    nbr = _ell_block(rng, n_dst, fanout, n_src)
+    zeros_s, zeros_d = np.zeros((n_src, heads), np.float32), np.zeros((n_dst, heads), np.float32)
+    out = orc.gat_block(nbr, n_dst, fanout, ft, zeros_s, zeros_d)
+    keep = nbr >= 0
+    mean = orc.spmm_sum(0, nbr[keep], rows[keep], ft.reshape(n_src, -1), n_dst)
+    cnt = np.maximum(np.bincount(rows[keep], minlength=n_dst), 1)[:, None]
+    assert np.allclose(out.reshape(n_dst, -1), mean / cnt, rtol=1e-6, atol=1e-6)
+    # (3) attention sums to one per destination and head; a lone neighbour passes through
+    out, attn = orc.gat_block(nbr, n_dst, fanout, ft, el, er, 0.2, want_attn=True)
+    sums = attn.reshape(n_dst, fanout, heads).sum(1)
+    has = np.bincount(rows[keep], minlength=n_dst) > 0
+    assert np.allclose(sums[has], 1, atol=1e-6) and np.all(sums[~has] == 0)
+    if nbr[fanout] >= 0:
+        assert np.allclose(out[1], ft[nbr[fanout]], rtol=1e-6)
+    # (4) softmax is shift invariant on the positive side: logits all > 0 stay linear under + c on er
+    big_l, big_r = np.abs(el) + 1, np.abs(er) + 1
+    a = orc.gat_block(nbr, n_dst, fanout, ft, big_l, big_r)
+    b = orc.gat_block(nbr, n_dst, fanout, ft, big_l, big_r + 3.5)
+    assert np.allclose(a, b, rtol=1e-5, atol=1e-6)
+    # (5) the slope matters only below zero
+    neg_l, neg_r = -np.abs(el) - 1, -np.abs(er) - 1
+    a = orc.gat_block(nbr, n_dst, fanout, ft, neg_l, neg_r, 0.2)
+    b = orc.gat_block(nbr, n_dst, fanout, ft, (0.2 * neg_l).astype(np.float32), (0.2 * neg_r).astype(np.float32), 1.0)
+    assert np.allclose(a, b, rtol=1e-5, atol=1e-6)
