@@ -54,6 +54,7 @@ template <> struct Pack<float, 4> { typedef float type __attribute__((ext_vector
 template <> struct Pack<float, 1> { typedef float type; };
 template <> struct Pack<uint16_t, 4> { typedef uint16_t type __attribute__((ext_vector_type(4))); };
 template <> struct Pack<uint16_t, 1> { typedef uint16_t type; };
+template <> struct Pack<uint16_t, 8> { typedef uint16_t type __attribute__((ext_vector_type(8))); };
 
 template <typename T, int VEC>
 __device__ __forceinline__ void load_vec(const T* base, int64_t elem, float (&v)[VEC]) {
@@ -267,6 +268,33 @@ __global__ __launch_bounds__(kAggBlock) void gat_scores_kernel(const T* __restri
   }
 }
 
+// The same for dim = VEC * LPH with LPH a power of two: LPH lanes per (row, head),
+// VEC features per lane in one 16-byte load, xor-shuffle reduction inside the
+// lane group.
+template <typename T, int VEC, int LPH>
+__global__ __launch_bounds__(kAggBlock) void gat_scores_vec_kernel(const T* __restrict__ x, int64_t items,
+                                                                   int heads, const float* __restrict__ attn,
+                                                                   float* __restrict__ out) {
+  constexpr int kGroups = kAggBlock / LPH;
+  constexpr int64_t dim = VEC * LPH;
+  const int grp = threadIdx.x / LPH, l = threadIdx.x % LPH;
+  for (int64_t it = static_cast<int64_t>(blockIdx.x) * kGroups + grp; it < items;
+       it += static_cast<int64_t>(gridDim.x) * kGroups) {
+    const int h = static_cast<int>(it % heads);
+    float v[VEC];
+    load_vec<T, VEC>(x, it * dim + l * VEC, v);
+    float acc = 0.f;
+#pragma unroll
+    for (int q = 0; q < VEC; q += 4) {
+      const float4 a = *reinterpret_cast<const float4*>(attn + h * dim + l * VEC + q);
+      acc += v[q] * a.x + v[q + 1] * a.y + v[q + 2] * a.z + v[q + 3] * a.w;
+    }
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+    if (l == 0) out[it] = acc;
+  }
+}
+
 // GATConv aggregation over a fixed-stride block (gatconv.py:118-126, DGL's
 // u_add_v -> LeakyReLU -> edge_softmax -> u_mul_e + sum): for destination i and
 // head h, e_k = leaky(el[src_k, h] + er[i, h]) over the row's slots, a = softmax(e),
@@ -476,7 +504,8 @@ extern "C" int apt_spmm_block(const int64_t* neighbors, int64_t num_dst, const i
     if (vec4) launch_ell<float, 4>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
     else launch_ell<float, 1>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
   } else {
-    if (vec4) launch_ell<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+    if (vec4 && dim % 8 == 0) launch_ell<uint16_t, 8>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
+    else if (vec4) launch_ell<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
     else launch_ell<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, input, num_src, dim, out, mean, st);
   }
   APT_LAUNCH_CHECK("spmm_ell_kernel");
@@ -493,9 +522,35 @@ extern "C" int apt_gat_scores(const void* x, int64_t num_rows, int heads, int64_
               elem_size);
   if (num_rows == 0) return APT_OK;
   APT_REQUIRE(x != nullptr && attn != nullptr && out != nullptr, APT_EINVAL, "apt_gat_scores: a tensor is NULL");
-  const unsigned blocks =
-      static_cast<unsigned>(std::min<int64_t>(ceil_div(num_rows * heads, kAggWaves), 1 << 20));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t items = num_rows * heads;
+  const int vec = elem_size == 2 && dim % 8 == 0 ? 8 : 4;   // 16 bytes per lane
+  const int64_t lph = dim / vec;
+  if (dim % 4 == 0 && lph <= kWave && (lph & (lph - 1)) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(attn) & 15) == 0) {
+#define APT_SCORES(T, V, LPH)                                                                           \
+  hipLaunchKernelGGL((gat_scores_vec_kernel<T, V, LPH>),                                                \
+                     dim3(static_cast<unsigned>(std::min<int64_t>(ceil_div(items, kAggBlock / LPH), 1 << 20))), \
+                     dim3(kAggBlock), 0, st, static_cast<const T*>(x), items, heads, attn, out)
+#define APT_SCORES_T(T, V)                               \
+  switch (lph) {                                         \
+    case 1: APT_SCORES(T, V, 1); break;                  \
+    case 2: APT_SCORES(T, V, 2); break;                  \
+    case 4: APT_SCORES(T, V, 4); break;                  \
+    case 8: APT_SCORES(T, V, 8); break;                  \
+    case 16: APT_SCORES(T, V, 16); break;                \
+    case 32: APT_SCORES(T, V, 32); break;                \
+    default: APT_SCORES(T, V, 64); break;                \
+  }
+    if (elem_size == 4) { APT_SCORES_T(float, 4) }
+    else if (vec == 8) { APT_SCORES_T(uint16_t, 8) }
+    else { APT_SCORES_T(uint16_t, 4) }
+#undef APT_SCORES_T
+#undef APT_SCORES
+    APT_LAUNCH_CHECK("gat_scores_vec_kernel");
+    return APT_OK;
+  }
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(items, kAggWaves), 1 << 20));
   if (elem_size == 4)
     hipLaunchKernelGGL(gat_scores_kernel<float>, dim3(blocks), dim3(kAggBlock), 0, st,
                        static_cast<const float*>(x), num_rows, heads, dim, attn, out);
@@ -527,7 +582,8 @@ extern "C" int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const in
     if (vec4) launch_gat<float, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
     else launch_gat<float, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
   } else {
-    if (vec4) launch_gat<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+    if (vec4 && dim % 8 == 0) launch_gat<uint16_t, 8>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
+    else if (vec4) launch_gat<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
     else launch_gat<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
   }
   APT_LAUNCH_CHECK("gat_ell_kernel");

@@ -305,6 +305,29 @@ def main():
             nbytes = E * hid * es + n_dst * hid * 4 + 8 * n_dst * f
             agg[f"spmm_block_mean_{name}_us"] = t * 1e6
             agg[f"spmm_block_mean_{name}_GBps"] = nbytes / t / 1e9
+        # GAT layer of the same block: 4 heads x 64, logits then fused LeakyReLU + edge softmax + weighted sum
+        heads, hdim = 4, 64
+        for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+            ft = synth.random_features(n_src, heads * hdim, dt, args.seed + 9, dev).view(n_src, heads, hdim)
+            al = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
+            ar = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
+            el, er = capi.gat_scores(ft, al), capi.gat_scores(ft[:n_dst], ar)
+            for tag, fn, nbytes in (
+                    ("gat_scores", lambda: capi.gat_scores(ft, al), n_src * heads * (hdim * es + 4)),
+                    ("gat_block", lambda: capi.gat_block(rel, n_dst, f, ft, el, er, 0.2),
+                     E * heads * (hdim * es + 4) + n_dst * heads * (hdim * 4 + 4) + 8 * n_dst * f)):
+                for _ in range(3):
+                    fn()
+                e0, e1 = ev(), ev()
+                e0.record()
+                for _ in range(10):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                t = e0.elapsed_time(e1) / 10 * 1e-3
+                agg[f"{tag}_{name}_us"] = t * 1e6
+                agg[f"{tag}_{name}_GBps"] = nbytes / t / 1e9
+            del ft, el, er
         hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
         h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)
         fn = lambda: capi.sddmm(0, row_e, col_e, h, hd)

@@ -135,7 +135,7 @@ def _ell(rng, n_dst, fanout, n_src, hole=0.25):
     return nbr.reshape(-1)
 
 
-@pytest.mark.parametrize("heads,dim", [(4, 64), (1, 256), (3, 5), (8, 16), (2, 100)])
+@pytest.mark.parametrize("heads,dim", [(4, 64), (1, 256), (3, 5), (8, 16), (2, 100), (5, 4), (3, 512), (2, 32)])
 def test_gat_fp32(orc, capi, heads, dim):
     rng = np.random.default_rng(heads * 1000 + dim)
     n_dst, fanout, n_src = 3000, 15, 20000
