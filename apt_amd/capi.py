@@ -62,6 +62,8 @@ SYMBOLS = {
     "apt_count_ids": (_I, [_P, _I64, _P, _P, _I64, _P]),
     "apt_csr_row_degrees": (_I, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "apt_csr_copy_rows": (_I, [_P, _P, _I64, _P, _I64, _P, _I64, _P, _P]),
+    "apt_map_to_vir": (_I, [_P, _I64, _P, _I64, _I, _P, _I, _I64, _I, _I, _I, _P, _P]),
+    "apt_vir_send_offset": (_I, [_I, _I64, _P, _I64, _P, _I64, _I, _P, _P]),
     "apt_block_workspace_bytes": (_SZ, [_I64, _I, _I64, _I]),
     "apt_block_formats": (_I, [_P, _I64, _P, _I, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
@@ -598,3 +600,28 @@ def gat_block(neighbors, num_dst, fanout, ft, el, er, negative_slope=0.2, num_ds
                               heads, dim, ft.element_size(), _ptr(el), _ptr(er), float(negative_slope), _ptr(out),
                               _ptr(attn), _stream()))
     return (out, attn) if want_attn else out
+
+
+def map_to_vir(src, fanout, min_vids, world_size, rank=0, node_beg=0, node_end=None, id_offset=0, dst=None,
+               num_dst=None):
+    """Virtual-node ids of SP mode (see apt_map_to_vir).  dst given: [dst part, src part]
+    as srcdst_to_vir; else num_dst must be given, as src_to_vir."""
+    src = _dev_i64(src, "src")
+    dst = _dev_i64(dst, "dst")
+    min_vids = _dev_i64(min_vids, "min_vids")
+    if min_vids.numel() < world_size + 1:
+        raise AptError("map_to_vir: min_vids needs world_size + 1 entries")
+    nd = dst.numel() if dst is not None else int(num_dst)
+    out = torch.empty((nd if dst is not None else 0) + src.numel(), dtype=torch.int64, device=src.device)
+    check(lib().apt_map_to_vir(_ptr(dst), nd, _ptr(src), src.numel(), int(fanout), _ptr(min_vids), int(world_size),
+                               int(id_offset), int(rank), int(node_beg),
+                               int(world_size if node_end is None else node_end), _ptr(out), _stream()))
+    return out
+
+
+def vir_send_offset(world_size, base, sorted_nodes, unique_nodes, with_dst=False):
+    sorted_nodes, unique_nodes = _dev_i64(sorted_nodes, "sorted_nodes"), _dev_i64(unique_nodes, "unique_nodes")
+    out = torch.empty(world_size * (3 if with_dst else 2) + 1, dtype=torch.int64, device=sorted_nodes.device)
+    check(lib().apt_vir_send_offset(int(world_size), int(base), _ptr(sorted_nodes), sorted_nodes.numel(),
+                                    _ptr(unique_nodes), unique_nodes.numel(), int(with_dst), _ptr(out), _stream()))
+    return out

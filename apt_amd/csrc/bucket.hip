@@ -214,6 +214,67 @@ static int run_bucketing(BucketParams& p, void* workspace, size_t workspace_byte
   return APT_OK;
 }
 
+// ------------------------------------------------------------ virtual nodes
+// SP mode groups the edges of a destination by the owner of their source:
+// "virtual node" (owner, destination) stands for the part of a destination's
+// neighbourhood that lives on one owner (reference src/cuda/npc_kernel.cu:15-113).
+//   with dst:  vir[i]           = owner(dst[i]) * num_dst + i                          i < num_dst
+//              vir[num_dst + j] = owner(src[j]) * num_dst + world * num_dst + j / fanout
+//   without:   vir[j]           = owner(src[j]) * num_dst + j / fanout
+// owner() is the bucketing rule of apt_cluster_permute.
+struct VirParams {
+  const int64_t* dst;        // NULL: sources only
+  int64_t num_dst;
+  const int64_t* src;
+  int64_t num_src;
+  int fanout;
+  const int64_t* min_vids;
+  int world;
+  int64_t id_offset;
+  int rank, node_beg, node_end;
+  int64_t* vir;
+};
+
+__global__ __launch_bounds__(kBktBlock) void map_to_vir_kernel(VirParams p) {
+  __shared__ int64_t s_min[APT_MAX_BUCKETS + 1];
+  if (threadIdx.x <= p.world) s_min[threadIdx.x] = p.min_vids[threadIdx.x];
+  __syncthreads();
+  const int64_t lead = p.dst != nullptr ? p.num_dst : 0;
+  const int64_t n = lead + p.num_src;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBktBlock + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kBktBlock) {
+    int64_t v, offset;
+    if (i < lead) {
+      v = p.dst[i];
+      offset = i;
+    } else {
+      const int64_t j = i - lead;
+      v = p.src[j];
+      offset = (p.dst != nullptr ? static_cast<int64_t>(p.world) * p.num_dst : 0) + j / p.fanout;
+    }
+    int64_t d = p.id_offset;
+    while (d + 1 < p.world && s_min[d + 1] <= v) ++d;
+    if (d < p.node_beg || d >= p.node_end) d = p.rank;
+    p.vir[i] = d * p.num_dst + offset;
+  }
+}
+
+// out[k] = first position in sorted[0..n) whose value is >= (first + k) * base
+// (thrust::lower_bound in GetVirSendOffset, reference :115-183).
+__global__ void vir_lower_bound_kernel(const int64_t* __restrict__ sorted, int64_t n, int64_t base,
+                                       int first, int count, int64_t* __restrict__ out) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= count) return;
+  const int64_t want = static_cast<int64_t>(first + k) * base;
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    const int64_t mid = lo + (hi - lo) / 2;
+    if (sorted[mid] < want) lo = mid + 1;
+    else hi = mid;
+  }
+  out[k] = lo;
+}
+
 }  // namespace apt
 
 extern "C" size_t apt_bucket_workspace_bytes(int64_t n, int num_buckets) {
@@ -305,4 +366,50 @@ extern "C" int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_
   p.permutation = permutation;
   return run_bucketing(p, workspace, workspace_bytes, static_cast<hipStream_t>(stream),
                        "apt_cluster_reqs");
+}
+
+extern "C" int apt_map_to_vir(const int64_t* dst, int64_t num_dst, const int64_t* src, int64_t num_src,
+                              int fanout, const int64_t* min_vids, int world_size, int64_t id_offset,
+                              int rank, int node_beg, int node_end, int64_t* vir_nodes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_dst >= 0 && num_src >= 0 && fanout > 0, APT_EINVAL,
+              "apt_map_to_vir: bad shape (num_dst %lld, num_src %lld, fanout %d)", (long long)num_dst,
+              (long long)num_src, fanout);
+  APT_REQUIRE(world_size >= 1 && world_size <= APT_MAX_BUCKETS, APT_ELIMIT,
+              "apt_map_to_vir: world_size %d outside [1, %d]", world_size, APT_MAX_BUCKETS);
+  APT_REQUIRE(id_offset >= 0 && id_offset < world_size && rank >= 0 && rank < world_size, APT_EINVAL,
+              "apt_map_to_vir: id_offset / rank outside [0, %d)", world_size);
+  const int64_t n = (dst != nullptr ? num_dst : 0) + num_src;
+  if (n == 0) return APT_OK;
+  APT_REQUIRE(min_vids != nullptr && vir_nodes != nullptr && (src != nullptr || num_src == 0), APT_EINVAL,
+              "apt_map_to_vir: a pointer is NULL");
+  VirParams p{dst, num_dst, src, num_src, fanout, min_vids, world_size, id_offset, rank, node_beg, node_end,
+              vir_nodes};
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(n, kBktBlock), 1 << 16));
+  hipLaunchKernelGGL(map_to_vir_kernel, dim3(blocks), dim3(kBktBlock), 0, static_cast<hipStream_t>(stream), p);
+  APT_LAUNCH_CHECK("map_to_vir_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_vir_send_offset(int world_size, int64_t base, const int64_t* sorted_nodes,
+                                   int64_t num_sorted, const int64_t* unique_nodes, int64_t num_unique,
+                                   int with_dst, int64_t* send_offset, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(world_size >= 1 && world_size <= APT_MAX_BUCKETS, APT_ELIMIT,
+              "apt_vir_send_offset: world_size %d outside [1, %d]", world_size, APT_MAX_BUCKETS);
+  APT_REQUIRE(num_sorted >= 0 && num_unique >= 0 && base >= 0, APT_EINVAL, "apt_vir_send_offset: negative size");
+  APT_REQUIRE(send_offset != nullptr && (sorted_nodes != nullptr || num_sorted == 0) &&
+                  (unique_nodes != nullptr || num_unique == 0),
+              APT_EINVAL, "apt_vir_send_offset: a pointer is NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // boundaries of the sorted virtual nodes, then of the unique ones
+  const int a_count = (with_dst ? 2 : 1) * world_size + 1;
+  const int b_first = with_dst ? world_size + 1 : 1;
+  hipLaunchKernelGGL(vir_lower_bound_kernel, dim3(1), dim3(256), 0, st, sorted_nodes, num_sorted, base, 0,
+                     a_count, send_offset);
+  APT_LAUNCH_CHECK("vir_lower_bound_kernel");
+  hipLaunchKernelGGL(vir_lower_bound_kernel, dim3(1), dim3(256), 0, st, unique_nodes, num_unique, base, b_first,
+                     world_size, send_offset + a_count);
+  APT_LAUNCH_CHECK("vir_lower_bound_kernel");
+  return APT_OK;
 }

@@ -295,6 +295,32 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> ClusterAndPermuteLocal(Tensor seeds) 
   return {size, offset, sorted, perm};
 }
 
+// reference src/sampling.cc:19-50: virtual nodes of SP mode (local arithmetic, no exchange)
+static Tensor MapToVir(const char* who, IdType fanout, const Tensor* dst, IdType num_dst, Tensor src) {
+  auto& s = S();
+  TORCH_CHECK(s.shuffle_min_vids.defined(), "npc: ", who, ": register_min_vids has not been called");
+  TORCH_CHECK(s.shuffle_min_vids.numel() >= s.world_size + 1, "npc: min_vids shorter than world_size + 1");
+  TORCH_CHECK(fanout > 0, "npc: ", who, ": fanout must be > 0");
+  auto sv = ids_on_device(src, "src");
+  Tensor dv;
+  if (dst != nullptr) {
+    dv = ids_on_device(*dst, "dst");
+    num_dst = dv.numel();
+  }
+  const int node_beg = static_cast<int>(s.rank - (s.rank % s.node_size));
+  auto out = torch::empty({(dst != nullptr ? num_dst : 0) + sv.numel()}, i64_opts());
+  check(apt_map_to_vir(dst != nullptr ? i64(dv) : nullptr, num_dst, i64(sv), sv.numel(), static_cast<int>(fanout),
+                       s.shuffle_min_vids.data_ptr<int64_t>(), static_cast<int>(s.world_size),
+                       s.shuffle_id_offset, static_cast<int>(s.rank), node_beg,
+                       node_beg + static_cast<int>(s.node_size), out.data_ptr<int64_t>(), stream()));
+  return out;
+}
+Tensor SrcDsttoVir(IdType fanout, Tensor dst, Tensor src) { return MapToVir("srcdst_to_vir", fanout, &dst, 0, src); }
+Tensor SrcToVir(IdType fanout, IdType num_dst, Tensor src) {
+  TORCH_CHECK(num_dst >= 0, "npc: src_to_vir: num_dst must be >= 0");
+  return MapToVir("src_to_vir", fanout, nullptr, num_dst, src);
+}
+
 // reference src/sampling.cc:159-193; with one GPU both all-to-alls are identity copies
 std::tuple<Tensor, Tensor, Tensor, Tensor> ShuffleSeeds(Tensor seeds) {
   TORCH_CHECK(S().world_size == 1,
@@ -439,8 +465,6 @@ Tensor NCCLGetUniqueId() { NPC_NEEDS_PEERS("nccl_get_unique_id"); }
 void Initialize(IdType, IdType, IdType, Tensor, IdType) { NPC_NEEDS_PEERS("init"); }
 void AlltoAll(Tensor, Tensor, Tensor, Tensor, IdType, IdType) { NPC_NEEDS_PEERS("alltoall"); }
 Tensor CrossMachineLoadSubtensor(Tensor) { NPC_NEEDS_PEERS("crossmachine_load_subtensor"); }
-Tensor SrcDsttoVir(IdType, Tensor, Tensor) { NPC_NEEDS_PEERS("srcdst_to_vir"); }
-Tensor SrcToVir(IdType, IdType, Tensor) { NPC_NEEDS_PEERS("src_to_vir"); }
 std::vector<Tensor> NPSampleAndShuffle(Tensor, IdType) { NPC_NEEDS_PEERS("np_sample_and_shuffle"); }
 std::vector<Tensor> SPSampleAndShuffle(IdType, Tensor, Tensor, Tensor, IdType) {
   NPC_NEEDS_PEERS("sp_sample_and_shuffle");

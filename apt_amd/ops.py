@@ -150,5 +150,36 @@ def sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset
     return _npc.sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset)
 
 
+class Aggregate(torch.autograd.Function):
+    """reference python/npc/model/sageconv.py:100-114: forward sums source rows
+    into destinations over the concatenated COO blocks; backward is the same
+    operator with the edge direction and the two offset tables swapped."""
+
+    @staticmethod
+    def forward(ctx, graph, X, X_offset, out_offset):
+        ctx.graph = graph
+        all_coo_row, all_coo_col, coo_offset = graph
+        out = _npc.spmm_copy_u_sum(all_coo_row, all_coo_col, X, coo_offset, X_offset, out_offset)
+        ctx.save_for_backward(X_offset, out_offset)
+        return out
+
+    @staticmethod
+    def backward(ctx, dZ):
+        all_coo_row, all_coo_col, coo_offset = ctx.graph
+        X_offset, out_offset = ctx.saved_tensors
+        dX = _npc.spmm_copy_u_sum(all_coo_col, all_coo_row, dZ.contiguous(), coo_offset, out_offset, X_offset)
+        return None, dX, None, None
+
+
+def srcdst_to_vir(fanout: int, dst: torch.Tensor, src: torch.Tensor) -> torch.Tensor:
+    """reference python/npc/sampler.py:20-21"""
+    return _npc.srcdst_to_vir(fanout, dst, src)
+
+
+def src_to_vir(fanout: int, num_dst: int, src: torch.Tensor) -> torch.Tensor:
+    """reference python/npc/sampler.py:16-17"""
+    return _npc.src_to_vir(fanout, num_dst, src)
+
+
 def np_sample_and_shuffle(seeds, fanout):
     return _npc.np_sample_and_shuffle(seeds, fanout)

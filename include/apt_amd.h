@@ -308,6 +308,29 @@ int apt_csr_copy_rows(const int64_t* indptr, const int64_t* indices, int64_t row
                       const int64_t* rows, int64_t n, const int64_t* out_indptr,
                       int64_t num_out_edges, int64_t* out_indices, void* stream);
 
+/* Virtual nodes of SP mode: the part of a destination's neighbourhood that one
+ * owner holds.  Replaces MapSrcDsttoVir / MapSrctoVir (src/cuda/npc_kernel.cu:15-113,
+ * called by SrcDsttoVir / SrcToVir, src/sampling.cc:19-50) and GetVirSendOffset /
+ * GetVirSendOffsetWithDst (:115-183).  owner() is the rule of apt_cluster_permute
+ * (min_vids, id_offset, rank, node_beg, node_end as there).
+ *   apt_map_to_vir, dst != NULL: vir_nodes[num_dst + num_src],
+ *       vir[i] = owner(dst[i]) * num_dst + i,
+ *       vir[num_dst + j] = owner(src[j]) * num_dst + world_size * num_dst + j / fanout
+ *   dst == NULL: vir_nodes[num_src], vir[j] = owner(src[j]) * num_dst + j / fanout
+ *   apt_vir_send_offset: lower bounds of multiples of base (= num_dst) in the
+ *       sorted virtual nodes and in their unique values:
+ *       with_dst == 0: send_offset[2 * world_size + 1]; [k] = lower_bound(sorted, k * base),
+ *           k = 0..world_size; [world_size + k] = lower_bound(unique, k * base), k = 1..world_size
+ *       with_dst != 0: send_offset[3 * world_size + 1]; [k] = lower_bound(sorted, k * base),
+ *           k = 0..2 * world_size; [2 * world_size + k] = lower_bound(unique,
+ *           (world_size + k) * base), k = 1..world_size */
+int apt_map_to_vir(const int64_t* dst, int64_t num_dst, const int64_t* src, int64_t num_src,
+                   int fanout, const int64_t* min_vids, int world_size, int64_t id_offset, int rank,
+                   int node_beg, int node_end, int64_t* vir_nodes, void* stream);
+int apt_vir_send_offset(int world_size, int64_t base, const int64_t* sorted_nodes, int64_t num_sorted,
+                        const int64_t* unique_nodes, int64_t num_unique, int with_dst,
+                        int64_t* send_offset, void* stream);
+
 /* Sparse formats of a sampled block.  The reference hands (row, col) of a hop to
  * DGL, which materialises COO, CSR and CSC (python/npc/sampler.py:59-69,76-91;
  * create_block_from_csc :44-56 takes a CSC as it is).  Input is the hop's

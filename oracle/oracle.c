@@ -26,6 +26,7 @@
  *   orc_permute/scatter numpy take / put.
  *   orc_gat_scores/_block  scipy.special.softmax on a dense adjacency, the mean
  *                       SpMM when all logits are equal, shift invariance.
+ *   orc_map_to_vir, orc_vir_send_offset   numpy searchsorted closed forms.
  *   orc_block_formats   numpy nonzero / stable argsort / bincount + cumsum.
  *   orc_count_ids, orc_csr_select_rows   numpy bincount / concatenated slices.
  *   orc_spmm_sum/sddmm  numpy closed forms (np.add.at over fancy-indexed rows,
@@ -567,4 +568,47 @@ void orc_gat_block(const int64_t* nbr, int64_t num_dst, int fanout, const float*
     }
   free(e);
   free(acc);
+}
+
+/* ------------------------------------------------------------------ */
+/* Virtual nodes of SP mode (src/cuda/npc_kernel.cu:15-183).  Pinned by */
+/* numpy searchsorted closed forms.                                     */
+/* ------------------------------------------------------------------ */
+static int64_t orc_owner(int64_t v, const int64_t* min_vids, int world, int64_t id_offset, int rank,
+                         int node_beg, int node_end) {
+  int64_t d = id_offset;
+  while (d + 1 < world && min_vids[d + 1] <= v) ++d;   /* :41-43 */
+  if (d < node_beg || d >= node_end) d = rank;          /* :45-47 */
+  return d;
+}
+
+void orc_map_to_vir(const int64_t* dst, int64_t num_dst, const int64_t* src, int64_t num_src, int fanout,
+                    const int64_t* min_vids, int world, int64_t id_offset, int rank, int node_beg,
+                    int node_end, int64_t* vir) {
+  int64_t lead = 0;
+  if (dst) {
+    lead = num_dst;
+    for (int64_t i = 0; i < num_dst; ++i)
+      vir[i] = orc_owner(dst[i], min_vids, world, id_offset, rank, node_beg, node_end) * num_dst + i;
+  }
+  for (int64_t j = 0; j < num_src; ++j)
+    vir[lead + j] = orc_owner(src[j], min_vids, world, id_offset, rank, node_beg, node_end) * num_dst +
+                    (dst ? (int64_t)world * num_dst : 0) + j / fanout;
+}
+
+static int64_t orc_lower_bound(const int64_t* a, int64_t n, int64_t want) {
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    int64_t mid = lo + (hi - lo) / 2;
+    if (a[mid] < want) lo = mid + 1; else hi = mid;
+  }
+  return lo;
+}
+
+void orc_vir_send_offset(int world, int64_t base, const int64_t* sorted, int64_t ns, const int64_t* uniq,
+                         int64_t nu, int with_dst, int64_t* out) {
+  const int a_count = (with_dst ? 2 : 1) * world + 1;
+  const int b_first = with_dst ? world + 1 : 1;
+  for (int k = 0; k < a_count; ++k) out[k] = orc_lower_bound(sorted, ns, (int64_t)k * base);
+  for (int k = 0; k < world; ++k) out[a_count + k] = orc_lower_bound(uniq, nu, (int64_t)(b_first + k) * base);
 }

@@ -16,7 +16,7 @@ __all__ = [
     "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
     "sample_neighbors", "sample_positions", "relabel", "gather_rows",
     "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
-    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows", "block_formats", "gat_scores", "gat_block",
+    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows", "block_formats", "gat_scores", "gat_block", "map_to_vir", "vir_send_offset",
 ]
 
 
@@ -352,3 +352,23 @@ def gat_block(neighbors, num_dst, fanout, ft, el, er, negative_slope=0.2, want_a
     lib().orc_gat_block(_p(nbr), C.c_int64(num_dst), C.c_int(fanout), _p(ft), C.c_int64(num_src), C.c_int(heads),
                         C.c_int64(dim), _p(el), _p(er), C.c_double(negative_slope), _p(out), _p(attn))
     return (out, attn) if want_attn else out
+
+
+def map_to_vir(src, fanout, min_vids, world_size, rank=0, node_beg=0, node_end=None, id_offset=0, dst=None,
+               num_dst=None):
+    src, mv = _i64(src), _i64(min_vids)
+    d = None if dst is None else _i64(dst)
+    nd = len(d) if d is not None else int(num_dst)
+    out = np.empty((nd if d is not None else 0) + len(src), dtype=np.int64)
+    lib().orc_map_to_vir(_p(d), C.c_int64(nd), _p(src), C.c_int64(len(src)), C.c_int(fanout), _p(mv),
+                         C.c_int(world_size), C.c_int64(id_offset), C.c_int(rank), C.c_int(node_beg),
+                         C.c_int(world_size if node_end is None else node_end), _p(out))
+    return out
+
+
+def vir_send_offset(world_size, base, sorted_nodes, unique_nodes, with_dst=False):
+    s, u = _i64(sorted_nodes), _i64(unique_nodes)
+    out = np.empty(world_size * (3 if with_dst else 2) + 1, dtype=np.int64)
+    lib().orc_vir_send_offset(C.c_int(world_size), C.c_int64(base), _p(s), C.c_int64(len(s)), _p(u),
+                              C.c_int64(len(u)), C.c_int(int(with_dst)), _p(out))
+    return out
