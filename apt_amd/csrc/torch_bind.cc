@@ -41,6 +41,10 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   uint64_t rng_seed = 7777777;  // reference src/cuda/npc_kernel.cu:292
   int64_t sample_calls = 0;
   bool strict = true;
+  // fused multi-hop driver: rank table of the registered graph, workspace of the last plan
+  Tensor rank_table, mb_workspace;
+  int64_t mb_batch = -1;
+  std::vector<int64_t> mb_fanouts;
 };
 
 State& S() {
@@ -154,6 +158,7 @@ void MixCacheGraphs(IdType num_cached_nodes, Tensor cached_node_idx, Tensor cach
   s.graph.row_begin = 0;
   s.graph.num_rows = total;
   s.graph.num_total_nodes = total;
+  s.rank_table = Tensor();
   s.adj_pos_map = Tensor();
   if (num_cached_nodes > 0) {
     auto idx = ids_on_device(cached_node_idx, "cached_node_idx");
@@ -187,6 +192,7 @@ void RegisterGraphPartition(Tensor indptr, Tensor indices, IdType row_begin, IdT
   s.graph.row_begin = row_begin;
   s.graph.num_rows = s.indptr.numel() - 1;
   s.graph.num_total_nodes = num_total_nodes;
+  s.rank_table = Tensor();
   s.has_graph = true;
 }
 
@@ -215,6 +221,114 @@ std::tuple<Tensor, Tensor> SampleNeighbors(Tensor seeds, IdType fanout, bool rep
                              static_cast<uint64_t>(rng_seed), static_cast<int>(hop),
                              out.data_ptr<int64_t>(), cnt.data_ptr<int64_t>(), nullptr, stream()));
   return {out, cnt};
+}
+
+// The whole multi-hop loop of MixedPSNeighborSampler.sample, DP branch (reference
+// python/npc/sampler.py:187-203,358-364: sample -> relabel -> frontier = unique, per
+// hop) as one operator: every kernel of the batch is enqueued by one C call, the
+// sizes stay on the device, and the host waits once, to cut the outputs to size.
+// hop_fanouts: from the seeds outward.  Returns
+//   [sizes (CPU int64[H + 2]: frontier rows entering each hop, input nodes, edges),
+//    input_nodes, then per hop h: neighbors_h, relabeled_h, counts_h]
+// with neighbors / relabeled in the fixed-stride layout [rows_h * fanout_h], -1 = no edge.
+// The rank table and workspace live in the registry and are reused: calls must be
+// ordered on one stream.
+std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts, bool replace, IdType rng_seed) {
+  auto& s = S();
+  TORCH_CHECK(s.has_graph, "npc: no graph registered (mix_cache_graphs)");
+  const int H = static_cast<int>(hop_fanouts.size());
+  TORCH_CHECK(H >= 1 && H <= APT_MAX_HOPS, "npc: sample_blocks: 1..", APT_MAX_HOPS, " hops");
+  auto sd = ids_on_device(seeds, "seeds");
+  const int64_t B = sd.numel();
+  TORCH_CHECK(B > 0, "npc: sample_blocks: no seeds");
+  std::vector<int> fan(H);
+  for (int h = 0; h < H; ++h) {
+    TORCH_CHECK(hop_fanouts[h] > 0 && hop_fanouts[h] <= (1 << 20), "npc: sample_blocks: bad fanout");
+    fan[h] = static_cast<int>(hop_fanouts[h]);
+  }
+  auto u8 = torch::TensorOptions().dtype(torch::kUInt8).device(device());
+  if (!s.rank_table.defined()) {
+    const size_t bytes = apt_rank_table_bytes(s.graph.num_total_nodes);
+    TORCH_CHECK(bytes > 0, "npc: sample_blocks: graph too large for the rank table");
+    s.rank_table = torch::empty({static_cast<int64_t>(bytes)}, u8);
+    check(apt_rank_table_init(s.rank_table.data_ptr(), bytes, stream()));
+  }
+  if (s.mb_batch != B || s.mb_fanouts != hop_fanouts || !s.mb_workspace.defined()) {
+    const size_t need = apt_minibatch_workspace_bytes(B, fan.data(), H);
+    TORCH_CHECK(need > 0, "npc: sample_blocks: unsupported batch / fanouts");
+    s.mb_workspace = torch::empty({static_cast<int64_t>(need)}, u8);
+    check(apt_minibatch_workspace_init(s.mb_workspace.data_ptr(), need, stream()));
+    s.mb_batch = B;
+    s.mb_fanouts = hop_fanouts;
+  }
+  std::vector<int64_t> cap(H + 1);
+  for (int h = 0; h <= H; ++h) {
+    cap[h] = apt_minibatch_capacity(B, fan.data(), H, h);
+    TORCH_CHECK(cap[h] > 0, "npc: sample_blocks: unsupported batch / fanouts");
+  }
+  auto nodes = torch::empty({cap[H]}, i64_opts());
+  auto sizes = torch::empty({H + 2}, i64_opts());
+  std::vector<Tensor> nb(H), rl(H), ct(H);
+  std::vector<int64_t*> nbp(H), rlp(H), ctp(H);
+  for (int h = 0; h < H; ++h) {
+    nb[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+    rl[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+    ct[h] = torch::empty({cap[h]}, i64_opts());
+    nbp[h] = nb[h].data_ptr<int64_t>();
+    rlp[h] = rl[h].data_ptr<int64_t>();
+    ctp[h] = ct[h].data_ptr<int64_t>();
+  }
+  const int rc = apt_minibatch_sample(&s.graph, i64(sd), B, fan.data(), H, replace ? 1 : 0,
+                                      static_cast<uint64_t>(rng_seed), nullptr, s.rank_table.data_ptr(),
+                                      s.graph.num_total_nodes, nodes.data_ptr<int64_t>(), nbp.data(), rlp.data(),
+                                      ctp.data(), sizes.data_ptr<int64_t>(), s.mb_workspace.data_ptr(),
+                                      static_cast<size_t>(s.mb_workspace.numel()), stream());
+  if (rc != APT_OK) s.mb_workspace = Tensor();  // re-initialised by the next call
+  check(rc);
+  auto host = sizes.cpu();  // the one wait of the batch
+  const int64_t* hs = host.data_ptr<int64_t>();
+  std::vector<Tensor> out{host, nodes.narrow(0, 0, hs[H])};
+  for (int h = 0; h < H; ++h) {
+    out.push_back(nb[h].narrow(0, 0, hs[h] * fan[h]));
+    out.push_back(rl[h].narrow(0, 0, hs[h] * fan[h]));
+    out.push_back(ct[h].narrow(0, 0, hs[h]));
+  }
+  return out;
+}
+
+// COO / CSC / CSR of a fixed-stride block (what DGL derives from (row, col) in the
+// reference, python/npc/sampler.py:59-69).  Returns [coo_row, coo_col, csc_indptr]
+// (+ [csr_indptr, csr_indices, csr_eids] with want_csr), cut to the edge count.
+std::vector<Tensor> BlockFormats(Tensor relabeled, IdType num_dst, IdType fanout, IdType num_src, bool want_csr) {
+  auto rl = ids_on_device(relabeled, "relabeled");
+  TORCH_CHECK(num_dst >= 0 && fanout > 0 && num_src >= 0, "npc: block_formats: bad shape");
+  TORCH_CHECK(rl.numel() >= num_dst * fanout, "npc: block_formats: relabeled shorter than num_dst * fanout");
+  const int64_t slots = num_dst * fanout;
+  const size_t need = apt_block_workspace_bytes(num_dst, static_cast<int>(fanout), num_src, want_csr);
+  TORCH_CHECK(need > 0 || slots == 0, "npc: block_formats: sizes out of range");
+  auto ws = torch::empty({static_cast<int64_t>(std::max<size_t>(need, 256))},
+                         torch::TensorOptions().dtype(torch::kUInt8).device(device()));
+  auto row = torch::empty({slots}, i64_opts()), col = torch::empty({slots}, i64_opts());
+  auto csc = torch::empty({num_dst + 1}, i64_opts()), edges = torch::zeros({1}, i64_opts());
+  Tensor csr, ci, ce;
+  if (want_csr) {
+    csr = torch::empty({num_src + 1}, i64_opts());
+    ci = torch::empty({slots}, i64_opts());
+    ce = torch::empty({slots}, i64_opts());
+  }
+  check(apt_block_formats(i64(rl), num_dst, nullptr, static_cast<int>(fanout), num_src, row.data_ptr<int64_t>(),
+                          col.data_ptr<int64_t>(), csc.data_ptr<int64_t>(), edges.data_ptr<int64_t>(),
+                          want_csr ? csr.data_ptr<int64_t>() : nullptr, want_csr ? ci.data_ptr<int64_t>() : nullptr,
+                          want_csr ? ce.data_ptr<int64_t>() : nullptr, ws.data_ptr(),
+                          static_cast<size_t>(ws.numel()), stream()));
+  const int64_t e = edges.item<int64_t>();
+  std::vector<Tensor> out{row.narrow(0, 0, e), col.narrow(0, 0, e), csc};
+  if (want_csr) {
+    out.push_back(csr);
+    out.push_back(ci.narrow(0, 0, e));
+    out.push_back(ce.narrow(0, 0, e));
+  }
+  return out;
 }
 
 // reference src/sampling.cc:13-17
@@ -508,6 +622,8 @@ TORCH_LIBRARY(npc, m) {
       .def("sddmm_u_mul_v", &UMulV)
       // additions (no counterpart in the reference)
       .def("sample_neighbors", &SampleNeighbors)
+      .def("sample_blocks", &SampleBlocks)
+      .def("block_formats", &BlockFormats)
       .def("cluster_and_permute", &ClusterAndPermuteLocal)
       .def("register_graph_partition", &RegisterGraphPartition)
       .def("set_topology", &SetTopology)

@@ -75,6 +75,25 @@ def sample_neighbors(seeds: torch.Tensor, fanout: int, replace: bool, rng_seed: 
     return _npc.sample_neighbors(seeds, fanout, replace, rng_seed, hop)
 
 
+def sample_blocks(seeds: torch.Tensor, hop_fanouts, replace: bool, rng_seed: int):
+    """Every hop of a batch in one operator call (sample -> relabel -> next
+    frontier; reference python/npc/sampler.py:187-203,358-364), one host wait.
+    hop_fanouts: from the seeds outward.
+    -> (sizes list[H + 2], input_nodes, [(neighbors, relabeled, counts) per hop])"""
+    out = _npc.sample_blocks(seeds, [int(f) for f in hop_fanouts], bool(replace), int(rng_seed))
+    hops = [tuple(out[2 + 3 * h:5 + 3 * h]) for h in range(len(hop_fanouts))]
+    return out[0].tolist(), out[1], hops
+
+
+def block_formats(relabeled: torch.Tensor, num_dst: int, fanout: int, num_src: int, want_csr: bool = True):
+    """COO / CSC (/ CSR) of a fixed-stride block -> dict of tensors."""
+    out = _npc.block_formats(relabeled, num_dst, fanout, num_src, want_csr)
+    d = dict(coo_row=out[0], coo_col=out[1], csc_indptr=out[2], num_edges=out[0].numel())
+    if want_csr:
+        d.update(csr_indptr=out[3], csr_indices=out[4], csr_eids=out[5])
+    return d
+
+
 def tensor_relabel_csc(seeds, neighbors) -> Tuple[torch.Tensor, torch.Tensor]:
     """reference python/npc/sampler.py:72-73"""
     return _npc.relabel_csc(seeds, neighbors)

@@ -1,7 +1,8 @@
 """Multi-hop mini-batch driver, the DP branch of MixedPSNeighborSampler
 (reference python/npc/sampler.py:159-203,358-364) and create_dgl_block
 (:76-91), without DGL: a block is a plain record of COO tensors."""
-from dataclasses import dataclass
+from dataclasses import dataclass, field
+from typing import Optional
 
 import torch
 
@@ -12,12 +13,34 @@ from . import ops
 class Block:
     """Bipartite block of one hop.  Edge e goes from source row[e] (index into
     src_ids) to destination col[e] (index into the hop's seeds); the first
-    num_dst source ids are the destination ids (reference sampler.py:76-91)."""
+    num_dst source ids are the destination ids (reference sampler.py:76-91).
+    relabeled / fanout: the same edges in the sampler's fixed-stride layout
+    (relabeled[d * fanout + k], -1 = no edge), which the block aggregations read
+    directly; csc() / csr() give DGL's other two formats on demand."""
     row: torch.Tensor
     col: torch.Tensor
     num_src: int
     num_dst: int
     src_ids: torch.Tensor
+    relabeled: Optional[torch.Tensor] = None
+    fanout: int = 0
+    formats: Optional[dict] = field(default=None, repr=False)
+
+    def _formats(self, want_csr):
+        if self.formats is None or (want_csr and "csr_indptr" not in self.formats):
+            self.formats = ops.block_formats(self.relabeled, self.num_dst, self.fanout, self.num_src, want_csr)
+        return self.formats
+
+    def csc(self):
+        """-> (indptr over destinations, source per edge, edge ids): the arguments
+        of the reference's create_block_from_csc (sampler.py:44-56)."""
+        f = self._formats(False)
+        return f["csc_indptr"], f["coo_row"], torch.arange(f["num_edges"], device=self.row.device)
+
+    def csr(self):
+        """-> (indptr over sources, destination per edge, edge ids)."""
+        f = self._formats(True)
+        return f["csr_indptr"], f["csr_indices"], f["csr_eids"]
 
     def number_of_src_nodes(self):
         return self.num_src
@@ -30,11 +53,12 @@ def create_block(seeds, neighbors, fanout):
     """reference sampler.py:76-91 (create_dgl_block); -1 padded slots (rows
     with fewer than fanout neighbours) produce no edge."""
     unique, relabeled = ops.relabel_csc(seeds, neighbors)
-    col = torch.arange(seeds.numel(), device=relabeled.device).repeat_interleave(fanout)
-    keep = relabeled >= 0
-    if not bool(keep.all()):
-        relabeled, col = relabeled[keep], col[keep]
-    return Block(relabeled, col, unique.numel(), seeds.numel(), unique)
+    return _block(seeds.numel(), unique, relabeled, fanout)
+
+
+def _block(num_dst, unique, relabeled, fanout):
+    f = ops.block_formats(relabeled, num_dst, fanout, unique.numel(), False)
+    return Block(f["coo_row"], f["coo_col"], unique.numel(), num_dst, unique, relabeled, fanout, f)
 
 
 class MixedPSNeighborSampler:
@@ -43,7 +67,7 @@ class MixedPSNeighborSampler:
     sampled with the last entry."""
 
     def __init__(self, rank, world_size, fanouts, system="DP", model=None, num_total_nodes=None,
-                 shuffle_with_dst=False, debug_info=None, replace=True, rng_seed=None):
+                 shuffle_with_dst=False, debug_info=None, replace=True, rng_seed=None, fused=True):
         if system != "DP":
             raise NotImplementedError(f"system {system!r} needs other GPUs; only 'DP' is available")
         self.rank, self.world_size = rank, world_size
@@ -52,11 +76,24 @@ class MixedPSNeighborSampler:
         self.system = system
         self.replace = replace
         self.rng_seed = rng_seed
+        self.fused = fused
         self.batches = 0
 
     def sample(self, graph, seeds):
+        """-> (input_nodes, output_nodes, blocks), blocks outermost first.  fused:
+        one operator call for all hops; otherwise one sampling and one relabel
+        call per hop as in the reference.  With an rng_seed both give the same
+        batch."""
         output_nodes = seeds
         blocks = []
+        if self.fused and (self.rng_seed is not None or not self.replace):
+            seed = (self.rng_seed if self.rng_seed is not None else 0) + self.batches
+            fan = list(reversed(self.fanouts))
+            sizes, nodes, hops = ops.sample_blocks(seeds, fan, self.replace, seed)
+            for h, (_, relabeled, _) in enumerate(hops):
+                blocks.insert(0, _block(sizes[h], nodes[:sizes[h + 1]], relabeled, fan[h]))
+            self.batches += 1
+            return (nodes, output_nodes, blocks)
         for layer_id, fanout in enumerate(reversed(self.fanouts)):
             if self.replace and self.rng_seed is None:
                 seeds, neighbors = ops.local_sample_one_layer(seeds, fanout)

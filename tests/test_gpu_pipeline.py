@@ -294,3 +294,48 @@ def test_batches_in_flight_are_reproducible(orc, capi):
             assert torch.equal(cur[0], ref[0]), it
             for a, b in zip(cur[1], ref[1]):
                 assert torch.equal(a, b), it
+
+
+def test_operator_layer_fused_sampler(orc, capi):
+    """sample_blocks (all hops in one operator call) through MixedPSNeighborSampler:
+    the same batch as the per-hop operators and as the oracle; Block.csc()/csr()."""
+    import apt_amd as npc
+    indptr, indices, feats = _setup(orc, capi, n=9000, dim=16, seed=8)
+    n = len(indptr) - 1
+    npc.set_topology(0, 1)
+    e = torch.empty(0, dtype=torch.int64)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
+    og = orc.Graph(indptr, indices)
+    rng = np.random.default_rng(4)
+    for replace in (False, True):
+        fused = npc.MixedPSNeighborSampler(0, 1, [12, 6, 3], "DP", replace=replace, rng_seed=500)
+        perhop = npc.MixedPSNeighborSampler(0, 1, [12, 6, 3], "DP", replace=replace, rng_seed=500, fused=False)
+        for batch in range(3):                                 # the registry's rank table and workspace are reused
+            seeds = rng.permutation(n)[:200]
+            a_in, a_out, a_blocks = fused.sample(None, dev(seeds))
+            b_in, _, b_blocks = perhop.sample(None, dev(seeds))
+            want_in, want_blocks = orc.sample_blocks(og, seeds, [3, 6, 12], replace, 500 + batch)
+            assert np.array_equal(a_in.cpu().numpy(), want_in) and torch.equal(a_in, b_in)
+            assert torch.equal(a_out, dev(seeds)) and len(a_blocks) == 3
+            for a, b, w in zip(a_blocks, b_blocks, want_blocks):
+                assert (a.num_src, a.num_dst) == (b.num_src, b.num_dst) == (len(w["unique"]), len(w["seeds"]))
+                assert torch.equal(a.row, b.row) and torch.equal(a.col, b.col) and torch.equal(a.src_ids, b.src_ids)
+                ref = orc.block_formats(w["relabeled"], a.num_dst, w["fanout"], a.num_src)
+                assert np.array_equal(a.row.cpu().numpy(), ref["coo_row"])
+                ip, ix, eid = a.csc()
+                assert np.array_equal(ip.cpu().numpy(), ref["csc_indptr"]) and np.array_equal(ix.cpu().numpy(), ref["coo_row"])
+                assert np.array_equal(eid.cpu().numpy(), np.arange(ref["num_edges"]))
+                ip, ix, eid = a.csr()
+                assert np.array_equal(ip.cpu().numpy(), ref["csr_indptr"])
+                assert np.array_equal(ix.cpu().numpy(), ref["csr_indices"]) and np.array_equal(eid.cpu().numpy(), ref["csr_eids"])
+    # a different batch size / fanout list re-plans; a new graph gets a new rank table
+    sizes, nodes, hops = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9)
+    want_in, want_blocks = orc.sample_blocks(og, np.arange(50), [4], False, 9)
+    assert sizes[:2] == [50, len(want_in)] and np.array_equal(nodes.cpu().numpy(), want_in)
+    assert np.array_equal(hops[0][0].cpu().numpy(), want_blocks[0]["neighbors"])
+    assert np.array_equal(hops[0][2].cpu().numpy(), want_blocks[0]["counts"])
+    indptr2, indices2, _ = _setup(orc, capi, n=300, dim=4, seed=9)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr2), torch.from_numpy(indices2))
+    sizes, nodes, hops = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9)
+    want_in, _ = orc.sample_blocks(orc.Graph(indptr2, indices2), np.arange(50), [4], False, 9)
+    assert np.array_equal(nodes.cpu().numpy(), want_in)
