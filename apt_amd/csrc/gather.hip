@@ -119,6 +119,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
 
 int tuning_gather_rows();        // 0 = default
 int tuning_gather_max_blocks();  // 0 = default
+int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
 
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
@@ -160,7 +161,9 @@ static int vector_bytes(const GatherParams& p, int elem_size) {
                    static_cast<uintptr_t>(p.col_offset_bytes) |
                    static_cast<uintptr_t>(p.out_row_bytes);
   if (p.cache_table != nullptr) bits |= reinterpret_cast<uintptr_t>(p.cache_table);
-  for (int v = 16; v > elem_size; v >>= 1)
+  int widest = tuning_gather_vector_bytes();
+  if (widest != 2 && widest != 4 && widest != 8) widest = 16;
+  for (int v = widest; v > elem_size; v >>= 1)
     if ((bits & (v - 1)) == 0) return v;
   return elem_size;
 }

@@ -22,6 +22,10 @@ int tuning_gather_rows() { return g_gather_rows; }
 int tuning_gather_max_blocks() { return g_gather_max_blocks; }
 int tuning_fuse_mark() { return g_fuse_mark; }
 int tuning_payload_bits() { return g_payload_bits; }
+static int g_sample_min_workgroups = 0;
+int tuning_sample_min_workgroups() { return g_sample_min_workgroups; }
+static int g_gather_vector_bytes = 0;
+int tuning_gather_vector_bytes() { return g_gather_vector_bytes; }
 static int g_block_fused_scan = 1;
 int tuning_block_fused_scan() { return g_block_fused_scan; }
 
@@ -52,6 +56,17 @@ extern "C" int apt_set_tuning(const char* key, int value) {
   }
   if (std::strcmp(key, "minibatch_fuse_mark") == 0) {
     apt::g_fuse_mark = value != 0;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "sample_min_workgroups") == 0) {
+    if (value < 0) return apt::fail(APT_EINVAL, "apt_set_tuning: sample_min_workgroups must be >= 0");
+    apt::g_sample_min_workgroups = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "gather_vector_bytes") == 0) {
+    if (value != 0 && value != 2 && value != 4 && value != 8 && value != 16)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: gather_vector_bytes must be 0, 2, 4, 8 or 16");
+    apt::g_gather_vector_bytes = value;
     return APT_OK;
   }
   if (std::strcmp(key, "block_fused_scan") == 0) {

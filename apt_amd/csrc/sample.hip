@@ -49,6 +49,7 @@ struct SampleParams {
 
 constexpr int kSampleBlock = 256;
 constexpr int kMaxRowsPerGroup = 16;
+constexpr int kSampleMinWorkgroups = 8192;
 constexpr int kMaxFanout = 1024;
 
 // Resolve node v to its neighbour list (reference :263-276).  Ids or map
@@ -264,19 +265,23 @@ template <int LPS>
 static int launch_sample(const SampleParams& p, bool replace, int64_t blocks, size_t dyn_lds,
                          hipStream_t st) {
   const dim3 grid(static_cast<unsigned>(blocks)), block(kSampleBlock);
-  const bool wide = p.rows_per_group >= 4;
+  // rows of a group in flight at once: as many as it has, up to 4
+  const int u = p.rows_per_group >= 4 ? 4 : (p.rows_per_group >= 2 ? 2 : 1);
   if (replace) {
-    if (wide) hipLaunchKernelGGL((sample_kernel<LPS, true, 4>), grid, block, dyn_lds, st, p);
+    if (u == 4) hipLaunchKernelGGL((sample_kernel<LPS, true, 4>), grid, block, dyn_lds, st, p);
+    else if (u == 2) hipLaunchKernelGGL((sample_kernel<LPS, true, 2>), grid, block, dyn_lds, st, p);
     else hipLaunchKernelGGL((sample_kernel<LPS, true, 1>), grid, block, dyn_lds, st, p);
   } else {
-    if (wide) hipLaunchKernelGGL((sample_kernel<LPS, false, 4>), grid, block, dyn_lds, st, p);
+    if (u == 4) hipLaunchKernelGGL((sample_kernel<LPS, false, 4>), grid, block, dyn_lds, st, p);
+    else if (u == 2) hipLaunchKernelGGL((sample_kernel<LPS, false, 2>), grid, block, dyn_lds, st, p);
     else hipLaunchKernelGGL((sample_kernel<LPS, false, 1>), grid, block, dyn_lds, st, p);
   }
   APT_LAUNCH_CHECK("sample_kernel");
   return APT_OK;
 }
 
-int tuning_sample_lanes();  // 0 = automatic
+int tuning_sample_lanes();
+int tuning_sample_min_workgroups();  // 0 = default
 
 }  // namespace apt
 
@@ -342,9 +347,14 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
   if (mark != nullptr)                          // marking lives in the one-chunk path
     while (lps < fanout) lps <<= 1;
   const int groups = kSampleBlock / lps;
-  // Enough workgroups to cover 256 CUs several times over before rows are
-  // serialised inside a group.
-  int64_t rpg = num_frontier / (static_cast<int64_t>(groups) * 2048);
+  // Rows are serialised inside a group only beyond kSampleMinWorkgroups
+  // workgroups.  In the mini-batch driver num_frontier is an upper bound about
+  // 3-4x the real count and the workgroups past the real count exit at once,
+  // so this leaves roughly 2-4 k working workgroups (9-18 per CU), measured
+  // best for the random-access bound hop.
+  int64_t min_wg = tuning_sample_min_workgroups();
+  if (min_wg <= 0) min_wg = kSampleMinWorkgroups;
+  int64_t rpg = num_frontier / (static_cast<int64_t>(groups) * min_wg);
   if (rpg < 1) rpg = 1;
   if (rpg > kMaxRowsPerGroup) rpg = kMaxRowsPerGroup;
   p.rows_per_group = static_cast<int>(rpg);

@@ -46,8 +46,12 @@ int apt_abi_version(void);
  * counterpart in the reference whose launch shapes are compile-time constants,
  * src/cuda/npc_kernel.h:10-14).  value 0 restores the default.
  *   "sample_lanes_per_row"   8|16|32|64 lanes of a wavefront per frontier row
+ *   "sample_min_workgroups"  workgroups a sampling launch must have before a lane
+ *                            group is given more than one row
  *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing
  *   "gather_max_blocks"      cap on the gather grid (rows are strided over)
+ *   "gather_vector_bytes"    2|4|8|16: widest load/store a lane of the gather uses
+ *                            (16 = global_load_dwordx4 where alignment allows)
  *   "minibatch_payload_bits" width of the id field of rank-table entries (0 = as
  *                            narrow as the plan allows); wider = fewer epochs
  *                            between table refills (used to test the refill)
