@@ -9,6 +9,8 @@
 // reads the id and the position once, and moves the row as 16-byte vectors
 // (8/4/2-byte vectors when the row geometry is not 16-byte aligned), with
 // several rows per group in flight.  Pure copy: results are bit-exact.
+#include <hip/hip_ext.h>
+
 #include "common.hpp"
 
 namespace apt {
@@ -117,6 +119,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
               static_cast<unsigned long long>(misses));
 }
 
+static thread_local hipEvent_t t_gather_start = nullptr, t_gather_stop = nullptr;
+
 int tuning_gather_rows();        // 0 = default
 int tuning_gather_max_blocks();  // 0 = default
 int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
@@ -134,12 +138,22 @@ static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int64_t blocks = ceil_div(p.n, static_cast<int64_t>(groups) * R);
   if (blocks > max_blocks) blocks = max_blocks;
   const dim3 grid(static_cast<unsigned>(blocks)), block(kGatherBlock);
+  // One-shot measurement hook: the launch itself records the two events
+  // (kernel begin / kernel end), see apt_time_next_gather.
+  hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;
+  t_gather_start = t_gather_stop = nullptr;
+#define APT_GATHER_LAUNCH(RR)                                                                        \
+  if (ev0 != nullptr || ev1 != nullptr)                                                              \
+    hipExtLaunchKernelGGL((gather_kernel<V, LPR, RR>), grid, block, 0, st, ev0, ev1, 0, p);          \
+  else                                                                                               \
+    hipLaunchKernelGGL((gather_kernel<V, LPR, RR>), grid, block, 0, st, p)
   switch (R) {
-    case 1: hipLaunchKernelGGL((gather_kernel<V, LPR, 1>), grid, block, 0, st, p); break;
-    case 2: hipLaunchKernelGGL((gather_kernel<V, LPR, 2>), grid, block, 0, st, p); break;
-    case 8: hipLaunchKernelGGL((gather_kernel<V, LPR, 8>), grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL((gather_kernel<V, LPR, 4>), grid, block, 0, st, p); break;
+    case 1: APT_GATHER_LAUNCH(1); break;
+    case 2: APT_GATHER_LAUNCH(2); break;
+    case 8: APT_GATHER_LAUNCH(8); break;
+    default: APT_GATHER_LAUNCH(4); break;
   }
+#undef APT_GATHER_LAUNCH
   APT_LAUNCH_CHECK("gather_kernel");
   return APT_OK;
 }
@@ -225,6 +239,12 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.scatter = 0;
   p.num_out_rows = 0;
   return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int apt_time_next_gather(void* start_event, void* stop_event) {
+  apt::t_gather_start = static_cast<hipEvent_t>(start_event);
+  apt::t_gather_stop = static_cast<hipEvent_t>(stop_event);
+  return APT_OK;
 }
 
 static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_t dim,

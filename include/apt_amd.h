@@ -183,6 +183,14 @@ int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
                     int64_t num_index, const int64_t* num_index_dev, void* out,
                     int64_t* miss_count, void* stream);
 
+/* Measurement hook (no counterpart in the reference): the next gather / permute /
+ * scatter launch made by the calling thread records start_event when its kernel
+ * begins and stop_event when it ends (the events ride on the dispatch itself), so
+ * hipEventElapsedTime gives the kernel's duration without the dispatch gaps that a
+ * hipEventRecord bracket includes.  Both are hipEvent_t created by the caller;
+ * one-shot; NULL, NULL cancels. */
+int apt_time_next_gather(void* start_event, void* stop_event);
+
 /* Row permutation of a dense [rows, dim] table, the on-GPU halves of
  * FeatShuffle (src/feat_shuffle.cc:9-30) and the row gather by inverse_idx in
  * front of it (python/npc/model/sage_model.py:67):
