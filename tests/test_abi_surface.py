@@ -48,6 +48,24 @@ def test_argument_checks_need_no_gpu():
     assert L.apt_minibatch_capacity(4096, fan, 3, 3) == 4096 * 6 * 11 * 16
     assert L.apt_minibatch_capacity(1 << 28, fan, 3, 3) == -1          # ids would not fit 32 bits
     assert L.apt_rank_table_bytes(111_059_956) >= 4 * 111_059_956
+    # entry points added around the core path
+    assert L.apt_block_workspace_bytes(1000, 15, 5000, 1) > L.apt_block_workspace_bytes(1000, 15, 5000, 0) > 0
+    assert L.apt_block_workspace_bytes(1 << 40, 15, 5000, 1) == 0
+    assert L.apt_block_formats(None, 10, None, 5, 100, None, None, None, None, None, None, None, None, 0, None) != 0
+    assert b"csc_indptr" in L.apt_last_error()
+    assert L.apt_count_ids(None, -1, None, None, 10, None) != 0
+    assert L.apt_csr_copy_rows(None, None, 0, None, 5, None, 7, None, None) != 0
+    assert L.apt_gat_block(None, 10, None, 0, None, 5, 4, 64, 2, None, None, 0.2, None, None, None) != 0
+    assert b"fanout" in L.apt_last_error()
+    assert L.apt_gat_scores(None, 10, 4, 64, 3, None, None, None) != 0 and b"elem_size" in L.apt_last_error()
+    assert L.apt_map_to_vir(None, 5, None, 10, 0, None, 8, 0, 0, 0, 8, None, None) != 0
+    assert L.apt_vir_send_offset(0, 5, None, 0, None, 0, 0, None, None) != 0
+    assert L.apt_spmm_block(None, 5, None, 0, None, 5, 8, 4, 0, None, None) != 0
+    for key in (b"sample_min_workgroups", b"gather_vector_bytes", b"block_fused_scan"):
+        assert L.apt_set_tuning(key, 0) == 0
+    assert L.apt_set_tuning(b"block_fused_scan", 1) == 0
+    assert L.apt_set_tuning(b"gather_vector_bytes", 3) != 0
+    assert L.apt_time_next_gather(None, None) == 0
 
 
 REFERENCE_OPS = {   # reference src/pybind.cc:19-47 with the schemas torch infers from the C++ types
@@ -66,7 +84,14 @@ REFERENCE_OPS = {   # reference src/pybind.cc:19-47 with the schemas torch infer
     "feat_shuffle": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, int _4, int _5) -> Tensor",
     "shuffle_seeds": "(Tensor _0) -> (Tensor, Tensor, Tensor, Tensor)",
     "relabel_csc": "(Tensor _0, Tensor _1) -> Tensor[]",
-    "alltoall": None, "srcdst_to_vir": None, "src_to_vir": None, "sp_sample_and_shuffle": None,
+    "srcdst_to_vir": "(int _0, Tensor _1, Tensor _2) -> Tensor",
+    "src_to_vir": "(int _0, int _1, Tensor _2) -> Tensor",
+    "spmm_copy_u_sum": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, Tensor _5) -> Tensor",
+    "spmm_copy_e_sum": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4) -> Tensor",
+    "spmm_u_mul_e_sum": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, Tensor _5, Tensor _6) -> Tensor",
+    "sddmm_u_add_v": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, Tensor _5, Tensor _6) -> Tensor",
+    "sddmm_u_mul_v": "(Tensor _0, Tensor _1, Tensor _2, Tensor _3, Tensor _4, Tensor _5, Tensor _6) -> Tensor",
+    "alltoall": None, "sp_sample_and_shuffle": None,
     "sp_sample_shuffle_src": None, "mp_sample_shuffle": None, "sp_feat_shuffle": None,
     "mp_feat_shuffle_fwd": None, "mp_feat_shuffle_bwd": None,
 }
