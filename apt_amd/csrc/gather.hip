@@ -121,6 +121,17 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
 
 static thread_local hipEvent_t t_gather_start = nullptr, t_gather_stop = nullptr;
 
+// Takes the one-shot events off the thread at entry; rearm() hands them to the
+// launch that follows.
+struct TimingArm {
+  hipEvent_t start, stop;
+  TimingArm() : start(t_gather_start), stop(t_gather_stop) { t_gather_start = t_gather_stop = nullptr; }
+  void rearm() const {
+    t_gather_start = start;
+    t_gather_stop = stop;
+  }
+};
+
 int tuning_gather_rows();        // 0 = default
 int tuning_gather_max_blocks();  // 0 = default
 int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
@@ -197,6 +208,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
                                int64_t num_index, const int64_t* num_index_dev, void* out,
                                int64_t* miss_count, void* stream) {
   using namespace apt;
+  const TimingArm arm;  // a call that returns before its launch must not leave the events armed
   APT_REQUIRE(store != nullptr, APT_EINVAL, "apt_gather_rows: store is NULL");
   APT_REQUIRE(num_index >= 0, APT_EINVAL, "apt_gather_rows: num_index %lld < 0",
               (long long)num_index);
@@ -238,6 +250,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.miss_count = miss_count;
   p.scatter = 0;
   p.num_out_rows = 0;
+  arm.rearm();
   return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
 }
 
@@ -251,6 +264,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
                           int elem_size, void* out, int scatter, int64_t num_rows_other,
                           void* stream, const char* who) {
   using namespace apt;
+  const TimingArm arm;
   APT_REQUIRE(n >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (n %lld, dim %lld)", who,
               (long long)n, (long long)dim);
   APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "%s: elem_size %d (2 or 4 supported)",
@@ -275,6 +289,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
   p.miss_count = nullptr;
   p.scatter = scatter;
   p.num_out_rows = scatter ? num_rows_other : 0;
+  arm.rearm();
   return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
 }
 

@@ -219,7 +219,8 @@ def main():
     elapsed = time.perf_counter() - t0
     if staged:
         timed = [k for k in kevs if k is not None]
-        t_gather = sum(kernel_ms(k) for k in timed) / len(timed) * K
+        gather_ms = sorted(kernel_ms(k) for k in timed)
+        t_gather = sum(gather_ms) / len(timed) * K
         t_sample = start.elapsed_time(stop) - t_gather
         for a, b in timed:
             hip.hipEventDestroy(a)
@@ -418,26 +419,43 @@ def main():
             ofs = orc.FeatStore(h_feats, to_np(cache), h_pos)
             h_mv, h_rw = min_vids.cpu().numpy(), requests["remote_worker_map"].cpu().numpy()
         h_seeds = [s.cpu().numpy() for s in seed_sets[W:]]
-        cpu_edges = cpu_batches = 0
-        tc = 0.0
-        while tc < budget:
-            # the timed batches, cycled with fresh rng keys once they are used up
-            s = h_seeds[cpu_batches % K]
-            key = args.seed + 100 + W + cpu_batches
-            t1 = time.perf_counter()
-            inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
-            if requests is None:
-                orc.gather_rows(ofs, inp)
-            else:
-                bs, _, so, _ = orc.cluster_reqs(inp, h_pos, h_rw, h_mv, P, P)
-                orc.gather_rows(ofs, so[:bs[0]])
-            tc += time.perf_counter() - t1
-            cpu_edges += sum(int(b["counts"].sum()) for b in blocks)
-            cpu_batches += 1
+        def cpu_leg(seconds, first):
+            """Batches of the timed seed sets (cycled with fresh rng keys) until `seconds` are used."""
+            edges_done = batches = 0
+            tc = 0.0
+            while tc < seconds:
+                s = h_seeds[(first + batches) % K]
+                key = args.seed + 100 + W + first + batches
+                t1 = time.perf_counter()
+                inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
+                if requests is None:
+                    orc.gather_rows(ofs, inp)
+                else:
+                    bs, _, so, _ = orc.cluster_reqs(inp, h_pos, h_rw, h_mv, P, P)
+                    orc.gather_rows(ofs, so[:bs[0]])
+                tc += time.perf_counter() - t1
+                edges_done += sum(int(b["counts"].sum()) for b in blocks)
+                batches += 1
+            return edges_done, batches, tc
+
+        # most of the budget on all threads (the reported value), the rest on one thread for reference
+        cpu_edges, cpu_batches, tc = cpu_leg(budget * 0.75, 0)
+        one = None
+        if threads > 1:
+            orc.set_threads(1)
+            e1, b1, t1s = cpu_leg(budget * 0.25, cpu_batches)
+            one = dict(value=e1 / t1s, batches=b1, seconds=t1s)
+            orc.set_threads(threads)
+        model = ""
+        try:
+            model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
+        except (OSError, StopIteration):
+            pass
         cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
                    sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
                           f"with fresh rng keys) in {tc:.1f} s: sampling and gather on {threads} "
-                          f"OpenMP threads, relabel on 1 thread")
+                          f"OpenMP threads, relabel on 1 thread",
+                   one_thread=one, host_cpu=model, host_logical_cpus=os.cpu_count())
         del h_indices, h_feats, og, ofs
 
     out = {
@@ -471,6 +489,8 @@ def main():
             "algorithmic_bytes_per_launch": bytes_per_row * rows / K,
             "bytes_per_row": bytes_per_row, "rows_per_launch": rows / K,
             "avg_launch_us": t_gather / K * 1e3,
+            "launch_us_min_median_max": ([gather_ms[0] * 1e3, gather_ms[len(gather_ms) // 2] * 1e3,
+                                          gather_ms[-1] * 1e3] if staged else None),
             "timing": (f"HIP events carried by {len(timed)} of the {K} gather dispatches of the timed region "
                        f"(kernel begin / end)" if staged else "HIP events recorded around each gather launch of an untimed pass"),
 
