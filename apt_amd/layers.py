@@ -1,0 +1,92 @@
+"""GNN layers over sampled blocks without DGL.
+
+The reference's DP models take their layers from DGL (examples/model.py:38-41);
+its own layers (python/npc/model/sageconv.py:118-188 MPSAGEConv, Aggregate
+:100-114) do A(XW) with the library's SpMM operator and get the backward pass
+from the same operator with the edges reversed.  The layers here keep that
+arithmetic on a Block of this package: the forward sum reads the sampler's
+fixed-stride layout directly (no atomics), the backward sum runs over the
+block's CSR order (edges grouped by source), so both directions are
+reproducible.
+"""
+import torch
+from torch import nn
+
+from . import capi
+
+
+class BlockAggregate(torch.autograd.Function):
+    """out[d] = sum (or mean) over the block's edges (s -> d) of X[s]."""
+
+    @staticmethod
+    def forward(ctx, block, X, mean):
+        ctx.block, ctx.mean = block, mean
+        return capi.spmm_block(block.relabeled, block.num_dst, block.fanout, X.contiguous(), mean=mean)
+
+    @staticmethod
+    def backward(ctx, dZ):
+        block = ctx.block
+        dZ = dZ.contiguous()
+        if ctx.mean:
+            indptr = block.csc()[0]
+            cnt = (indptr[1:] - indptr[:-1]).clamp(min=1).to(dZ.dtype)
+            dZ = dZ / cnt[:, None]
+        _, dst, eids = block.csr()                     # edges grouped by source, by increasing edge id
+        src = block.row[eids]
+        dX = capi.spmm_sum(0, dst, src, dZ, block.num_src)
+        return None, dX, None
+
+
+class SAGEConv(nn.Module):
+    """GraphSAGE layer, mean aggregator, with the reference's arithmetic
+    (python/npc/model/sageconv.py:118-188): fc_self(h_dst) + fc_neigh(mean of
+    the neighbours), the linear map applied before the aggregation when it
+    shrinks the features."""
+
+    def __init__(self, in_feats, out_feats, bias=True, activation=None):
+        super().__init__()
+        self.in_feats, self.out_feats, self.activation = in_feats, out_feats, activation
+        self.fc_neigh = nn.Linear(in_feats, out_feats, bias=False)
+        self.fc_self = nn.Linear(in_feats, out_feats, bias=bias)
+        gain = nn.init.calculate_gain("relu")
+        nn.init.xavier_uniform_(self.fc_self.weight, gain=gain)
+        nn.init.xavier_uniform_(self.fc_neigh.weight, gain=gain)
+
+    def forward(self, block, feat):
+        """feat: [block.num_src, in_feats]; the first num_dst rows are the destinations."""
+        h_self = feat[:block.num_dst]
+        if self.in_feats > self.out_feats:
+            h_neigh = BlockAggregate.apply(block, self.fc_neigh(feat), True)
+        else:
+            h_neigh = self.fc_neigh(BlockAggregate.apply(block, feat, True))
+        rst = self.fc_self(h_self) + h_neigh
+        return self.activation(rst) if self.activation is not None else rst
+
+
+class GATConv(nn.Module):
+    """GAT layer forward (python/npc/model/gatconv.py:207-236: fc, attention
+    logits, LeakyReLU, edge softmax, weighted sum, bias) in two kernels.
+    Inference only: the fused aggregation has no backward pass."""
+
+    def __init__(self, in_feats, out_feats, num_heads, negative_slope=0.2, bias=True, activation=None):
+        super().__init__()
+        self.num_heads, self.out_feats, self.negative_slope, self.activation = (num_heads, out_feats,
+                                                                                negative_slope, activation)
+        self.fc = nn.Linear(in_feats, out_feats * num_heads, bias=False)
+        self.attn_l = nn.Parameter(torch.empty(num_heads, out_feats))
+        self.attn_r = nn.Parameter(torch.empty(num_heads, out_feats))
+        self.bias = nn.Parameter(torch.zeros(num_heads * out_feats)) if bias else None
+        gain = nn.init.calculate_gain("relu")
+        nn.init.xavier_normal_(self.fc.weight, gain=gain)
+        nn.init.xavier_normal_(self.attn_l, gain=gain)
+        nn.init.xavier_normal_(self.attn_r, gain=gain)
+
+    @torch.no_grad()
+    def forward(self, block, feat):
+        ft = self.fc(feat).view(block.num_src, self.num_heads, self.out_feats).contiguous()
+        el = capi.gat_scores(ft, self.attn_l.detach().float().contiguous())
+        er = capi.gat_scores(ft[:block.num_dst].contiguous(), self.attn_r.detach().float().contiguous())
+        rst = capi.gat_block(block.relabeled, block.num_dst, block.fanout, ft, el, er, self.negative_slope)
+        if self.bias is not None:
+            rst = rst + self.bias.view(1, self.num_heads, self.out_feats)
+        return self.activation(rst) if self.activation is not None else rst
