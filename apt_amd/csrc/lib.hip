@@ -22,6 +22,8 @@ int tuning_gather_rows() { return g_gather_rows; }
 int tuning_gather_max_blocks() { return g_gather_max_blocks; }
 int tuning_fuse_mark() { return g_fuse_mark; }
 int tuning_payload_bits() { return g_payload_bits; }
+static int g_sample_max_blocks = 0;
+int tuning_sample_max_blocks() { return g_sample_max_blocks; }
 static int g_sample_min_workgroups = 0;
 int tuning_sample_min_workgroups() { return g_sample_min_workgroups; }
 static int g_gather_vector_bytes = 0;
@@ -56,6 +58,11 @@ extern "C" int apt_set_tuning(const char* key, int value) {
   }
   if (std::strcmp(key, "minibatch_fuse_mark") == 0) {
     apt::g_fuse_mark = value != 0;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "sample_max_blocks") == 0) {
+    if (value < 0) return apt::fail(APT_EINVAL, "apt_set_tuning: sample_max_blocks must be >= 0");
+    apt::g_sample_max_blocks = value;
     return APT_OK;
   }
   if (std::strcmp(key, "sample_min_workgroups") == 0) {

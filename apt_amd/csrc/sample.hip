@@ -47,9 +47,10 @@ struct SampleParams {
   int first_hop;
 };
 
-constexpr int kSampleBlock = 256;
+constexpr int kSampleBlock = 512;
 constexpr int kMaxRowsPerGroup = 16;
 constexpr int kSampleMinWorkgroups = 8192;
+constexpr int kSamplePersistentBlocks = 8192;
 constexpr int kMaxFanout = 1024;
 
 // Resolve node v to its neighbour list (reference :263-276).  Ids or map
@@ -125,33 +126,42 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
 
   const int64_t n = actual_count(p.n, p.n_dev);
   const int tile = G * p.rows_per_group;
-  const int64_t tile_base = static_cast<int64_t>(blockIdx.x) * tile;
-  if (tile_base >= n) return;  // block-uniform
+  if (static_cast<int64_t>(blockIdx.x) * tile >= n) return;  // block-uniform
   const uint64_t seed = p.seed_dev != nullptr ? *p.seed_dev : p.seed;
 
   const int tid = threadIdx.x;
-  if (tid == 0) s_total = 0;
-  // Stage 1: one lane per row of the tile, so the dependent
-  // frontier -> (pos_map ->) indptr loads of the whole tile overlap.
-  for (int t = tid; t < tile; t += kSampleBlock) {
-    const int64_t gi = tile_base + t;
-    const int64_t* nbrs = nullptr;
-    int64_t deg = 0, v = -1;
-    if (gi < n) {
-      v = p.frontier[gi];
-      resolve_row(p.g, v, nbrs, deg);
-    }
-    s_nbrs[t] = nbrs;
-    s_deg[t] = deg;
-    s_node[t] = v;
-  }
-  __syncthreads();
-
-  // Stage 2: one lane group per row.
   const int grp = tid / LPS;
   const int l = tid % LPS;
   const int fanout = p.fanout;
   int64_t my_total = 0;
+  if (tid == 0) s_total = 0;
+  // Stage 1 of a tile puts its rows into LDS, one lane per row, so the dependent
+  // frontier -> (pos_map ->) indptr loads of the whole tile overlap.  With one
+  // row per group there is nothing to overlap: every group resolves its own row
+  // (its lanes read the same addresses) and no group waits for another.
+  const bool direct = p.rows_per_group == 1 && p.fanout <= LPS;
+  __syncthreads();
+  // The grid may be smaller than the number of tiles (it is capped when the row
+  // count is only known on the device): a workgroup strides over the tiles.
+  for (int64_t tile_base = static_cast<int64_t>(blockIdx.x) * tile; tile_base < n;
+       tile_base += static_cast<int64_t>(gridDim.x) * tile) {
+  if (!direct) {
+    for (int t = tid; t < tile; t += kSampleBlock) {
+      const int64_t gi = tile_base + t;
+      const int64_t* nbrs = nullptr;
+      int64_t deg = 0, v = -1;
+      if (gi < n) {
+        v = p.frontier[gi];
+        resolve_row(p.g, v, nbrs, deg);
+      }
+      s_nbrs[t] = nbrs;
+      s_deg[t] = deg;
+      s_node[t] = v;
+    }
+    __syncthreads();
+  }
+
+  // Stage 2: one lane group per row.
   if (fanout <= LPS) {
     // U rows per group in flight: positions first, then the loads, then the
     // stores.
@@ -166,9 +176,16 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
         pos[u] = -1;
         src[u] = nullptr;
         if (gis[u] < n) {
-          const int64_t deg = s_deg[t];
-          src[u] = s_nbrs[t];
-          pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, s_node[t], seed, p.hop);
+          int64_t deg, node;
+          if (direct) {
+            node = p.frontier[gis[u]];
+            resolve_row(p.g, node, src[u], deg);
+          } else {
+            deg = s_deg[t];
+            node = s_node[t];
+            src[u] = s_nbrs[t];
+          }
+          pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, node, seed, p.hop);
           if (l == 0) {
             const int64_t cnt = REPLACE ? (deg > 0 ? fanout : 0) : (deg < fanout ? deg : fanout);
             if (p.counts != nullptr) p.counts[gis[u]] = cnt;
@@ -252,6 +269,8 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
       }
     }
   }
+  if (!direct) __syncthreads();  // the next tile overwrites the staged rows
+  }  // tiles
   if (p.total != nullptr) {
     if (l == 0 && my_total != 0)
       atomicAdd(&s_total, static_cast<unsigned long long>(my_total));
@@ -282,6 +301,7 @@ static int launch_sample(const SampleParams& p, bool replace, int64_t blocks, si
 
 int tuning_sample_lanes();
 int tuning_sample_min_workgroups();  // 0 = default
+int tuning_sample_max_blocks();      // 0 = default
 
 }  // namespace apt
 
@@ -359,7 +379,12 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
   if (rpg > kMaxRowsPerGroup) rpg = kMaxRowsPerGroup;
   p.rows_per_group = static_cast<int>(rpg);
   const int64_t tile = static_cast<int64_t>(groups) * rpg;
-  const int64_t blocks = ceil_div(num_frontier, tile);
+  int64_t blocks = ceil_div(num_frontier, tile);
+  // With a device-side count num_frontier is an upper bound: a capped grid that
+  // strides over the tiles avoids dispatching workgroups that find nothing to do.
+  int64_t max_blocks = tuning_sample_max_blocks();
+  if (max_blocks <= 0) max_blocks = num_frontier_dev != nullptr ? kSamplePersistentBlocks : (1 << 20);
+  if (blocks > max_blocks) blocks = max_blocks;
   APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT, "%s: %lld rows need too many workgroups", who,
               (long long)num_frontier);
   const size_t dyn = (!replace && fanout > lps) ? sizeof(int64_t) * groups * (size_t)fanout : 0;

@@ -56,6 +56,28 @@ def test_sampling_random_graph_all_lane_groups(orc, capi, lanes, replace):
         capi.set_tuning("sample_lanes_per_row", 0)
 
 
+@pytest.mark.parametrize("min_wg,max_blocks", [(0, 7), (1, 5), (3, 0), (1, 0)])
+def test_sampling_launch_shapes(orc, capi, min_wg, max_blocks):
+    """A small grid striding over many tiles, several rows per lane group (rows
+    staged in LDS) and one row per group (resolved directly) give the same rows;
+    fanouts below and above the 64 lanes of a wavefront."""
+    indptr, indices = small_graph(20000, 30, seed=21)
+    og, dg = _graphs(orc, capi, indptr, indices)
+    frontier = np.random.default_rng(5).integers(0, 20000, size=30011)
+    cnt = torch.tensor([25003], dtype=torch.int64, device=DEV)
+    capi.set_tuning("sample_min_workgroups", min_wg)
+    capi.set_tuning("sample_max_blocks", max_blocks)
+    try:
+        for fanout, replace in [(15, False), (7, True), (100, False), (70, True)]:
+            want_n, want_c = orc.sample_neighbors(og, frontier[:25003], fanout, replace, 9, 1)
+            got_n, got_c = capi.sample_neighbors(dg, dev(frontier), fanout, replace, 9, 1, num_frontier_dev=cnt)
+            assert np.array_equal(host(got_c)[:25003], want_c)
+            assert np.array_equal(host(got_n)[:25003 * fanout], want_n)
+    finally:
+        capi.set_tuning("sample_min_workgroups", 0)
+        capi.set_tuning("sample_max_blocks", 0)
+
+
 def test_sampling_position_map_and_partition(orc, capi):
     indptr, indices = small_graph(5000, 12, seed=12)
     n = 5000
