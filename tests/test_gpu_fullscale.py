@@ -66,6 +66,27 @@ def _check_properties(pipe, graph_t, feats, seeds, hops, replace):
     return res
 
 
+def _check_formats(blk):
+    """COO / CSC / CSR of a block against the fixed-stride layout they come from."""
+    f, fmt = blk["fanout"], blk["formats"]
+    rel = blk["relabeled"].view(-1, f)
+    num_dst, num_src, E = rel.shape[0], blk["unique"].numel(), fmt["num_edges"]
+    valid = rel >= 0
+    assert E == int(valid.sum())
+    assert torch.equal(fmt["coo_row"], rel[valid])                                   # destination-major order
+    assert torch.equal(fmt["coo_col"], torch.arange(num_dst, device=DEV)[:, None].expand(-1, f)[valid])
+    want = torch.zeros(num_dst + 1, dtype=torch.int64, device=DEV)
+    want[1:] = torch.cumsum(valid.sum(1), 0)
+    assert torch.equal(fmt["csc_indptr"], want)
+    eids, ip = fmt["csr_eids"], fmt["csr_indptr"]
+    assert ip.numel() == num_src + 1 and int(ip[0]) == 0 and int(ip[-1]) == E
+    assert torch.equal(torch.sort(eids).values, torch.arange(E, device=DEV))         # a permutation of the edges
+    src = fmt["coo_row"][eids]
+    assert torch.equal(src, torch.repeat_interleave(torch.arange(num_src, device=DEV), ip[1:] - ip[:-1]))
+    assert torch.equal(fmt["csr_indices"], fmt["coo_col"][eids])
+    assert bool(((eids[1:] > eids[:-1]) | (src[1:] != src[:-1])).all())              # stable inside a source
+
+
 def test_medium_scale_vs_oracle(orc, capi):
     from apt_amd import synth
     from apt_amd.pipeline import MiniBatchPipeline
@@ -104,12 +125,14 @@ def test_full_scale_properties(capi, replace):
     feats = synth.random_features(N, D, torch.bfloat16, 2, DEV)
     graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
     hops = [5, 10, 15]
-    pipe = MiniBatchPipeline(graph, store, 4096, hops, replace=replace)
+    pipe = MiniBatchPipeline(graph, store, 4096, hops, replace=replace, formats=True)
     gen = torch.Generator(device=DEV)
     gen.manual_seed(5)
     seeds = torch.randperm(N, generator=gen, device=DEV)[:4096].contiguous()
     pipe.run(seeds, 2025)
     res = _check_properties(pipe, (indptr, indices), feats, seeds, hops, replace)
+    for blk in res["blocks"]:
+        _check_formats(blk)
     first = {k: res[k].clone() for k in ("input_nodes", "features")}
     rel0 = [b["relabeled"].clone() for b in res["blocks"]]
     # the same key reproduces the batch (also after other batches went through the rank table)
@@ -124,5 +147,25 @@ def test_full_scale_properties(capi, replace):
     # a different key samples differently
     pipe.run(seeds, 2026)
     assert not torch.equal(pipe.result()["input_nodes"], first["input_nodes"])
+    if not replace:
+        # the million highest-degree rows in a second CSR built on the GPU: same offsets as the degrees say,
+        # and sampling through it (cached rows from the copy, the rest from the main table) changes nothing
+        deg = indptr[1:] - indptr[:-1]
+        hot = torch.topk(deg, 1_000_000).indices.contiguous()
+        c_indptr, c_indices = capi.csr_select_rows(graph, hot)
+        assert torch.equal(c_indptr[1:], torch.cumsum(deg[hot], 0)) and c_indices.numel() == int(c_indptr[-1])
+        hub = int(hot[0])                                              # the 2 M-edge hub row, copied by many workgroups
+        assert torch.equal(c_indices[:int(c_indptr[1])], indices[int(indptr[hub]):int(indptr[hub + 1])])
+        k = int(torch.randint(1, 1_000_000, (1,)))
+        assert torch.equal(c_indices[int(c_indptr[k]):int(c_indptr[k + 1])],
+                           indices[int(indptr[hot[k]]):int(indptr[hot[k] + 1])])
+        pos = -torch.arange(N, dtype=torch.int64, device=DEV) - 2
+        pos[hot] = torch.arange(hot.numel(), device=DEV)
+        cached_graph = capi.Graph(indptr, indices, cached_indptr=c_indptr, cached_indices=c_indices, adj_pos_map=pos)
+        frontier = torch.cat([hot[:20000], torch.randint(0, N, (50000,), generator=gen, device=DEV)])
+        a = capi.sample_neighbors(graph, frontier, 15, False, 99, 2)
+        b = capi.sample_neighbors(cached_graph, frontier, 15, False, 99, 2)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        del pos, c_indptr, c_indices
     del pipe, feats, indices, indptr
     torch.cuda.empty_cache()
