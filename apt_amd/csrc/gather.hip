@@ -139,7 +139,7 @@ int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int R = tuning_gather_rows();
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = 1;
   const int groups = kGatherBlock / LPR;
   // With a device-side count the host size is only an upper bound: a capped
   // grid that strides over the rows avoids dispatching workgroups that would
