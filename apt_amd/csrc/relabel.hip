@@ -6,11 +6,22 @@
 // occurrence; relabeled[j] = rank of neighbors[j]); different mechanics:
 //   * no torch::cat: the item list is addressed as seeds ++ neighbors;
 //   * one global open-addressing table (multiplicative hash, linear probing,
-//     load <= 1/2) whose slot is remembered per item, so the later passes do
-//     not probe again (the reference re-probes in each of its 3 passes);
+//     load <= 1/2) of 64-bit words (tag of the key, index of the key's first
+//     item so far).  A new key costs one load and one CAS, a repeated key a
+//     load and a look at the item the word points to; the reference (and a
+//     key column + index column layout) pays a CAS on the key and an atomicMin
+//     on the index for every item, and random atomics are the scarcest
+//     resource here (~24 G/s against ~50 G/s for loads);
+//   * who owns a key is settled inside the insert pass: a CAS that lowers a
+//     word's index knows which item it displaced and flags it, so afterwards
+//     "owner" = claimed or lowered a word and was never flagged, read from two
+//     byte arrays in item order; the reference re-probes the table in each of
+//     its 3 passes;
 //   * owner flags are compacted with wave ballots + popcounts and a two-level
 //     block prefix (no spin-waiting between workgroups, no temp allocation)
 //     instead of a device-wide cub scan over a materialised flag array;
+//   * the slot of every item is remembered, owners write their ids straight to
+//     the output and into their slot, so only repeated keys go back to the table;
 //   * the count stays on the device unless the caller asks for it.
 // Passes: fill -> insert -> count owners per block -> place owners -> relabel.
 #include "common.hpp"
@@ -23,7 +34,7 @@ constexpr int kRelTile = kRelBlock * kRelItemsPerThread;  // items per block in 
 constexpr int64_t kRelMaxItems = (1LL << 30);
 
 struct RelabelLayout {
-  size_t keys_off, minidx_off, val_off, slot_off, blockcnt_off, total;
+  size_t table_off, state_off, displaced_off, slot_off, blockcnt_off, total;
   uint64_t cap_max;
   int64_t blocks_max;
 };
@@ -41,10 +52,10 @@ static RelabelLayout relabel_layout(int64_t items) {
   L.cap_max = table_capacity(items);
   L.blocks_max = ceil_div(items > 0 ? items : 1, kRelTile);
   size_t off = 0;
-  L.keys_off = off;   off = align_up(off + L.cap_max * sizeof(int64_t), 256);
-  // minidx directly follows keys so one fill covers both (all bytes 0xFF).
-  L.minidx_off = off; off = align_up(off + L.cap_max * sizeof(uint32_t), 256);
-  L.val_off = off;    off = align_up(off + L.cap_max * sizeof(uint32_t), 256);
+  L.table_off = off;  off = align_up(off + L.cap_max * sizeof(uint64_t), 256);
+  // one byte per item each; separate arrays because different threads write them
+  L.state_off = off;  off = align_up(off + static_cast<size_t>(items > 0 ? items : 1), 256);
+  L.displaced_off = off; off = align_up(off + static_cast<size_t>(items > 0 ? items : 1), 256);
   L.slot_off = off;   off = align_up(off + static_cast<size_t>(items > 0 ? items : 1) * sizeof(uint32_t), 256);
   L.blockcnt_off = off; off = align_up(off + static_cast<size_t>(L.blocks_max) * sizeof(uint32_t), 256);
   L.total = off;
@@ -58,9 +69,9 @@ struct RelabelParams {
   const int64_t* neighbors;
   int64_t nn;               // host-side (upper bound)
   int64_t stride;           // neighbours per seed when ns_dev != NULL
-  int64_t* keys;
-  uint32_t* minidx;
-  uint32_t* val;
+  unsigned long long* table;  // per slot: (tag << 32) | item index, later (tag << 32) | id
+  uint8_t* state;             // per item, written by its own thread
+  uint8_t* displaced;         // per item, written by the thread that took its key over
   uint32_t* slot_of;
   uint32_t* block_cnt;
   int64_t* unique;
@@ -102,55 +113,86 @@ __device__ __forceinline__ uint64_t hash_slot(int64_t key, const RelSizes& s) {
   return (static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> s.shift;
 }
 
-// keys := -1 and minidx := 0xFFFFFFFF, over the actual capacity only.
+constexpr unsigned long long kEmptyWord = ~0ull;
+constexpr uint8_t kItemPadding = 0;   // negative id: takes no part
+constexpr uint8_t kItemFirst = 1;     // claimed or lowered its key's word: owner unless displaced later
+constexpr uint8_t kItemRepeat = 2;    // an item with a smaller index holds the key
+
+__device__ __forceinline__ uint32_t key_tag(int64_t key) {
+  return static_cast<uint32_t>((static_cast<uint64_t>(key) * 0xD6E8FEB86659FD93ull) >> 32);
+}
+
+// table := empty, displaced := 0, over the actual sizes only.
 __global__ __launch_bounds__(kRelBlock) void relabel_fill_kernel(RelabelParams p) {
   const RelSizes s = rel_sizes(p);
-  const uint64_t cap = s.mask + 1;
-  // keys: cap * 8 bytes, minidx: cap * 4 bytes; both as 16-byte stores.
-  const uint64_t key_vecs = cap / 2;      // 2 int64 per 16 B
-  const uint64_t idx_vecs = cap / 4;      // 4 uint32 per 16 B
-  const uint64_t total = key_vecs + idx_vecs;
+  const uint64_t table_vecs = (s.mask + 1) / 2;                                  // 2 words per 16 B
+  const uint64_t flag_vecs = (static_cast<uint64_t>(s.items) + 15) / 16;         // the array is padded to 256 B
+  const uint64_t total = table_vecs + flag_vecs;
   const uint4 ones = make_uint4(~0u, ~0u, ~0u, ~0u);
-  uint4* kv = reinterpret_cast<uint4*>(p.keys);
-  uint4* iv = reinterpret_cast<uint4*>(p.minidx);
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  uint4* tv = reinterpret_cast<uint4*>(p.table);
+  uint4* fv = reinterpret_cast<uint4*>(p.displaced);
   for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kRelBlock + threadIdx.x; i < total;
        i += static_cast<uint64_t>(gridDim.x) * kRelBlock) {
-    if (i < key_vecs) kv[i] = ones;
-    else iv[i - key_vecs] = ones;
+    if (i < table_vecs) tv[i] = ones;
+    else fv[i - table_vecs] = zero;
   }
 }
 
-// Insert every item; the smallest item index per key wins (reference
-// relabel.cu:12-24: CAS on the key, AtomicMin on the index).
+// Insert every item; the smallest item index per key ends up in the key's word
+// (reference relabel.cu:12-24: CAS on the key, AtomicMin on the index).
 __global__ __launch_bounds__(kRelBlock) void relabel_insert_kernel(RelabelParams p) {
   const RelSizes s = rel_sizes(p);
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kRelBlock + threadIdx.x; i < s.items;
        i += static_cast<int64_t>(gridDim.x) * kRelBlock) {
     const int64_t key = item_at(p, s, i);
-    if (key < 0) continue;  // padding
-    uint64_t slot = hash_slot(key, s);
-    unsigned long long* keys = reinterpret_cast<unsigned long long*>(p.keys);
-    while (true) {
-      // Plain look first: repeated ids (hubs) mostly find their key in place
-      // and skip the atomic.
-      int64_t cur = __builtin_nontemporal_load(&p.keys[slot]);
-      if (cur == -1)
-        cur = static_cast<int64_t>(atomicCAS(&keys[slot], ~0ull, static_cast<unsigned long long>(key)));
-      if (cur == -1 || cur == key) break;
-      slot = (slot + 1) & s.mask;
+    if (key < 0) {  // padding
+      p.state[i] = kItemPadding;
+      continue;
     }
-    const uint32_t me = static_cast<uint32_t>(i);
-    // Indices only decrease, so a stale larger value costs one extra atomic
-    // and a smaller one means this item cannot be the owner.
-    if (__builtin_nontemporal_load(&p.minidx[slot]) > me) atomicMin(&p.minidx[slot], me);
+    const uint32_t tag = key_tag(key);
+    const unsigned long long mine = (static_cast<unsigned long long>(tag) << 32) | static_cast<uint32_t>(i);
+    uint64_t slot = hash_slot(key, s);
+    uint8_t state;
+    // A read may be stale; it then shows the slot empty or its key with an
+    // older, larger index, and the CAS that follows fails and returns the truth.
+    unsigned long long w = __builtin_nontemporal_load(&p.table[slot]);
+    while (true) {
+      if (w == kEmptyWord) {
+        w = atomicCAS(&p.table[slot], kEmptyWord, mine);
+        if (w == kEmptyWord) {
+          state = kItemFirst;
+          break;
+        }
+      }
+      const uint32_t other = static_cast<uint32_t>(w);
+      if (static_cast<uint32_t>(w >> 32) == tag && item_at(p, s, other) == key) {
+        if (other < static_cast<uint32_t>(i)) {
+          state = kItemRepeat;
+          break;
+        }
+        // the word points at a later item of this key: take it over
+        const unsigned long long seen = atomicCAS(&p.table[slot], w, mine);
+        if (seen == w) {
+          p.displaced[other] = 1;
+          state = kItemFirst;
+          break;
+        }
+        w = seen;  // somebody else lowered it meanwhile: look again at the same slot
+        continue;
+      }
+      slot = (slot + 1) & s.mask;
+      w = __builtin_nontemporal_load(&p.table[slot]);
+    }
+    p.state[i] = state;
     p.slot_of[i] = static_cast<uint32_t>(slot);
   }
 }
 
+// Every lowering of a word is a CAS that flags the item it replaces, so the one
+// item of a key that is never flagged is the one with the smallest index.
 __device__ __forceinline__ bool is_owner(const RelabelParams& p, const RelSizes& s, int64_t i) {
-  if (i >= s.items) return false;
-  if (item_at(p, s, i) < 0) return false;
-  return p.minidx[p.slot_of[i]] == static_cast<uint32_t>(i);
+  return i < s.items && p.state[i] == kItemFirst && p.displaced[i] == 0;
 }
 
 // Owners per tile of kRelTile consecutive items.
@@ -174,7 +216,8 @@ __global__ __launch_bounds__(kRelBlock) void relabel_count_kernel(RelabelParams 
   }
 }
 
-// Exclusive prefix of owner flags -> unique[] and the table's value column.
+// Exclusive prefix of owner flags -> unique[], the owners' own outputs, and the
+// id in the key's word for the repeats.
 __global__ __launch_bounds__(kRelBlock) void relabel_place_kernel(RelabelParams p) {
   const RelSizes s = rel_sizes(p);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kRelTile;
@@ -219,19 +262,25 @@ __global__ __launch_bounds__(kRelBlock) void relabel_place_kernel(RelabelParams 
       const int64_t i = base + it * kRelBlock + threadIdx.x;
       const int64_t rank = before + rank_below(mask[it]);
       p.unique[rank] = item_at(p, s, i);
-      p.val[p.slot_of[i]] = static_cast<uint32_t>(rank);
+      if (i >= s.ns) p.relabeled[i - s.ns] = rank;
+      // low half of the word: the id, for the key's other items
+      reinterpret_cast<uint32_t*>(&p.table[p.slot_of[i]])[0] = static_cast<uint32_t>(rank);
     }
   }
   if (blockIdx.x == tiles - 1 && threadIdx.x == 0) *p.num_unique = running;
 }
 
-// relabeled[j] = rank of neighbors[j] (reference relabel.cu:153-173).
+// relabeled[j] for the neighbours that are not the first item of their key
+// (reference relabel.cu:153-173); padding passes through.
 __global__ __launch_bounds__(kRelBlock) void relabel_lookup_kernel(RelabelParams p) {
   const RelSizes s = rel_sizes(p);
   for (int64_t j = static_cast<int64_t>(blockIdx.x) * kRelBlock + threadIdx.x; j < s.nn;
        j += static_cast<int64_t>(gridDim.x) * kRelBlock) {
-    const int64_t key = p.neighbors[j];
-    p.relabeled[j] = key < 0 ? key : static_cast<int64_t>(p.val[p.slot_of[s.ns + j]]);
+    const int64_t i = s.ns + j;
+    const uint8_t st = p.state[i];
+    if (st == kItemPadding) p.relabeled[j] = p.neighbors[j];
+    else if (st == kItemRepeat || p.displaced[i] != 0)
+      p.relabeled[j] = static_cast<int64_t>(static_cast<uint32_t>(p.table[p.slot_of[i]]));
   }
 }
 
@@ -277,9 +326,9 @@ extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
   p.neighbors = neighbors;
   p.nn = num_neighbors;
   p.stride = neighbor_stride;
-  p.keys = reinterpret_cast<int64_t*>(ws + L.keys_off);
-  p.minidx = reinterpret_cast<uint32_t*>(ws + L.minidx_off);
-  p.val = reinterpret_cast<uint32_t*>(ws + L.val_off);
+  p.table = reinterpret_cast<unsigned long long*>(ws + L.table_off);
+  p.state = reinterpret_cast<uint8_t*>(ws + L.state_off);
+  p.displaced = reinterpret_cast<uint8_t*>(ws + L.displaced_off);
   p.slot_of = reinterpret_cast<uint32_t*>(ws + L.slot_off);
   p.block_cnt = reinterpret_cast<uint32_t*>(ws + L.blockcnt_off);
   p.unique = unique;
@@ -288,7 +337,7 @@ extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   const unsigned fill_blocks =
-      static_cast<unsigned>(std::min<int64_t>(ceil_div((int64_t)(L.cap_max * 3 / 4), kRelBlock), 8192));
+      static_cast<unsigned>(std::min<int64_t>(ceil_div((int64_t)(L.cap_max / 2 + (items + 15) / 16), kRelBlock), 8192));
   const unsigned item_blocks =
       static_cast<unsigned>(std::min<int64_t>(ceil_div(items > 0 ? items : 1, kRelBlock), 65536));
   const unsigned tile_blocks = static_cast<unsigned>(L.blocks_max);
