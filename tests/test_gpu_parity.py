@@ -146,6 +146,23 @@ def test_relabel_random_sizes(orc, capi):
         _relabel_case(orc, capi, seeds, nbrs)
 
 
+def test_relabel_equal_tags_and_reversed_duplicates(orc, capi):
+    """Different ids whose 32-bit table tags are equal (the tag only filters; the
+    id itself decides), and duplicates laid out so that later items tend to reach
+    the table first (a word is then lowered and its item displaced)."""
+    C2 = 0xD6E8FEB86659FD93
+    inv = pow(C2, -1, 1 << 64)
+    same_tag = [t * inv % (1 << 64) for t in range(1, 4000)]
+    same_tag = np.array([0] + [d for d in same_tag if d < (1 << 62)][:700], dtype=np.int64)
+    assert len({(int(k) * C2 % (1 << 64)) >> 32 for k in same_tag}) == 1 and len(same_tag) > 300
+    rng = np.random.default_rng(9)
+    nbrs = same_tag[rng.integers(0, len(same_tag), size=5000)]
+    _relabel_case(orc, capi, same_tag[:100][::-1].copy(), nbrs)
+    # every id many times, spread over the whole item range
+    ids = rng.permutation(5000)[:2000].astype(np.int64)
+    _relabel_case(orc, capi, ids[:256], np.tile(ids, 300))
+
+
 def test_relabel_specials(orc, capi):
     rng = np.random.default_rng(1)
     e = np.array([], dtype=np.int64)
