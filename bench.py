@@ -459,8 +459,8 @@ def main():
             pass
         cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
                    sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
-                          f"with fresh rng keys) in {tc:.1f} s: sampling and gather on {threads} "
-                          f"OpenMP threads, relabel on 1 thread",
+                          f"with fresh rng keys) in {tc:.1f} s: sampling, relabel and gather on {threads} "
+                          f"OpenMP threads",
                    one_thread=one, host_cpu=model, host_logical_cpus=os.cpu_count())
         del h_indices, h_feats, og, ofs
 

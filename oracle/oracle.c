@@ -19,7 +19,8 @@
  *                       The reference's exact draws (XORWOW, constant seed) are
  *                       not reproduced: parity of draw values is unpinned and
  *                       not claimed.
- *   orc_relabel         numpy closed form (np.unique first-occurrence order).
+ *   orc_relabel         numpy closed form (np.unique first-occurrence order), for the
+ *                       one-thread and the threaded variant alike.
  *   orc_gather_rows     numpy fancy indexing through the position map.
  *   orc_cluster_*       numpy searchsorted + stable argsort closed form; the
  *                       inputs of tests/test_shuffle_seeds.cc:19-26.
@@ -229,8 +230,8 @@ static inline uint64_t mix64(uint64_t x) {
   return x;
 }
 
-int64_t orc_relabel(const int64_t* seeds, int64_t ns, const int64_t* neighbors,
-                    int64_t nn, int64_t* unique, int64_t* relabeled) {
+static int64_t relabel_serial(const int64_t* seeds, int64_t ns, const int64_t* neighbors,
+                              int64_t nn, int64_t* unique, int64_t* relabeled) {
   int64_t items = ns + nn;
   uint64_t cap = 16;
   while (cap < (uint64_t)items * 2) cap <<= 1;
@@ -256,6 +257,94 @@ int64_t orc_relabel(const int64_t* seeds, int64_t ns, const int64_t* neighbors,
   free(keys);
   free(vals);
   return u;
+}
+
+/* The same result on several threads, the way the reference's kernels get it
+ * (relabel.cu:12-24,100-116): concurrent insert with a CAS on the key and an
+ * atomic minimum on the item index, owners = items whose index is their key's
+ * minimum, ranks = exclusive prefix of the owner flags in item order. */
+static int64_t relabel_threads(const int64_t* seeds, int64_t ns, const int64_t* neighbors,
+                               int64_t nn, int64_t* unique, int64_t* relabeled, int threads) {
+  const int64_t items = ns + nn;
+  uint64_t cap = 16;
+  while (cap < (uint64_t)items * 2) cap <<= 1;
+  int64_t* keys = (int64_t*)malloc(sizeof(int64_t) * cap);
+  int64_t* minidx = (int64_t*)malloc(sizeof(int64_t) * cap);   /* later: the key's rank */
+  uint32_t* slot_of = (uint32_t*)malloc(sizeof(uint32_t) * (size_t)(items > 0 ? items : 1));
+  uint8_t* owner = (uint8_t*)malloc((size_t)(items > 0 ? items : 1));
+  int64_t* part = (int64_t*)calloc((size_t)threads + 1, sizeof(int64_t));
+  int64_t total = 0;
+#pragma omp parallel num_threads(threads)
+  {
+#pragma omp for schedule(static)
+    for (uint64_t q = 0; q < cap; ++q) {
+      keys[q] = -1;
+      minidx[q] = INT64_MAX;
+    }
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < items; ++i) {
+      const int64_t k = i < ns ? seeds[i] : neighbors[i - ns];
+      if (k < 0) continue;
+      uint64_t pos = mix64((uint64_t)k) & (cap - 1);
+      for (;;) {
+        int64_t cur = __atomic_load_n(&keys[pos], __ATOMIC_RELAXED);
+        if (cur == -1) {
+          int64_t expect = -1;
+          if (__atomic_compare_exchange_n(&keys[pos], &expect, k, 0, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) break;
+          cur = expect;
+        }
+        if (cur == k) break;
+        pos = (pos + 1) & (cap - 1);
+      }
+      int64_t seen = __atomic_load_n(&minidx[pos], __ATOMIC_RELAXED);
+      while (seen > i && !__atomic_compare_exchange_n(&minidx[pos], &seen, i, 1, __ATOMIC_RELAXED, __ATOMIC_RELAXED)) {
+      }
+      slot_of[i] = (uint32_t)pos;
+    }
+    /* owners per thread chunk -> offsets -> ranks (static schedule: the same chunks both times) */
+    const int t = omp_get_thread_num();
+    int64_t mine = 0;
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < items; ++i) {
+      const int64_t k = i < ns ? seeds[i] : neighbors[i - ns];
+      owner[i] = k >= 0 && minidx[slot_of[i]] == i;
+      mine += owner[i];
+    }
+    part[t + 1] = mine;
+#pragma omp barrier
+#pragma omp single
+    {
+      for (int q = 0; q < threads; ++q) part[q + 1] += part[q];
+      total = part[threads];
+    }
+    int64_t rank = part[t];
+#pragma omp for schedule(static)
+    for (int64_t i = 0; i < items; ++i) {
+      if (!owner[i]) continue;
+      unique[rank] = i < ns ? seeds[i] : neighbors[i - ns];
+      keys[slot_of[i]] = rank++;   /* the slot's key is no longer needed: it now holds the rank */
+    }
+#pragma omp for schedule(static)
+    for (int64_t j = 0; j < nn; ++j) {
+      const int64_t k = neighbors[j];
+      relabeled[j] = k < 0 ? k : keys[slot_of[ns + j]];
+    }
+  }
+  free(keys);
+  free(minidx);
+  free(slot_of);
+  free(owner);
+  free(part);
+  return total;
+}
+
+int64_t orc_relabel(const int64_t* seeds, int64_t ns, const int64_t* neighbors,
+                    int64_t nn, int64_t* unique, int64_t* relabeled) {
+#ifdef _OPENMP
+  if (g_threads > 1 && ns + nn >= 4096)
+    return relabel_threads(seeds, ns, neighbors, nn, unique, relabeled, g_threads);
+#endif
+  return relabel_serial(seeds, ns, neighbors, nn, unique, relabeled);
 }
 
 /* ------------------------------------------------------------------ */

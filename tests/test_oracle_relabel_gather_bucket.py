@@ -38,6 +38,25 @@ def test_relabel_specials(orc):
     assert uniq.tolist() == [3, 1, 7] and rel.tolist() == [1, -1, 2, -1, 0]
 
 
+def test_relabel_threaded_variant(orc):
+    """Beyond 4096 items and with more than one thread the oracle inserts
+    concurrently (CAS + atomic minimum, as the reference's kernels do): the same
+    closed form must hold, whatever the interleaving."""
+    rng = np.random.default_rng(2)
+    orc.set_threads(4)
+    try:
+        for rep in range(5):
+            for ns, f, hi in [(4096, 1, 5000), (6144, 10, 100000), (3000, 15, 300), (70000, 15, 2_000_000)]:
+                seeds = rng.integers(0, hi, size=ns)                       # repeated seeds too
+                nbrs = rng.integers(0, hi, size=ns * f)
+                nbrs[rng.random(nbrs.size) < 0.1] = -1
+                _check_relabel(orc, seeds, nbrs)
+        uniq, rel = orc.relabel(np.array([4]), np.full(9000, 4))          # every item the same key
+        assert uniq.tolist() == [4] and not rel.any()
+    finally:
+        orc.set_threads(1)
+
+
 @pytest.mark.parametrize("dtype,dim", [(np.float32, 128), (np.float32, 100), (np.uint16, 128),
                                        (np.float32, 7), (np.uint16, 5)])
 def test_gather_identity(orc, dtype, dim):
