@@ -81,8 +81,10 @@ class MiniBatchPipeline:
         if formats:
             self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=formats != "csc", device=dev)
                             for h, f in enumerate(self.fanouts)]
-            # a hop's formats are a string of small dependent launches: the hops run beside each other
-            # (and beside the gather) on streams of their own
+            # with CSR a hop's formats are a string of ~10 small dependent launches: the hops then run beside
+            # each other (and beside the gather) on streams of their own; COO + CSC alone are 2 launches per
+            # hop, less than what the cross-stream joins cost, and stay on the caller's stream
+            self.format_side_streams = formats != "csc"
             self.format_streams = [torch.cuda.Stream(device=dev) for _ in self.fanouts]
             self.format_fork = torch.cuda.Event()
             self.format_done = [torch.cuda.Event() for _ in self.fanouts]
@@ -147,6 +149,10 @@ class MiniBatchPipeline:
         gather) and the caller joins later with join_formats()."""
         if self.formats is None:
             return
+        if not self.format_side_streams:
+            for h, fmt in enumerate(self.formats):
+                fmt.emit(self.relabeled[h], self._size(h))
+            return
         self.format_fork.record()
         for h, fmt in enumerate(self.formats):
             with torch.cuda.stream(self.format_streams[h]):
@@ -158,7 +164,7 @@ class MiniBatchPipeline:
 
     def join_formats(self):
         """The current stream waits for the formats (before the buffers are reused)."""
-        if self.formats is not None:
+        if self.formats is not None and self.format_side_streams:
             cur = torch.cuda.current_stream()
             for e in self.format_done:
                 cur.wait_event(e)

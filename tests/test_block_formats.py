@@ -108,8 +108,8 @@ def test_gpu_pipeline_blocks_in_all_formats(orc, capi):
     feats = torch.randn(20000, 32, device="cuda:0")
     graph = capi.Graph(dev(indptr), dev(indices))
     rng = np.random.default_rng(5)
-    for use_graph in (False, True):
-        pipe = MiniBatchPipeline(graph, capi.FeatStore(feats), 256, [4, 8, 12], formats=True, use_graph=use_graph)
+    for use_graph, what in ((False, True), (True, True), (False, "csc"), (True, "csc")):
+        pipe = MiniBatchPipeline(graph, capi.FeatStore(feats), 256, [4, 8, 12], formats=what, use_graph=use_graph)
         for key in (77, 78, 79):                              # buffers and streams are reused batch after batch
             seeds = rng.permutation(20000)[:256]
             pipe.run(dev(seeds), key)
@@ -121,5 +121,11 @@ def test_gpu_pipeline_blocks_in_all_formats(orc, capi):
                 f = got["formats"]
                 num_dst, num_src = len(want["seeds"]), len(want["unique"])
                 ref = orc.block_formats(want["relabeled"], num_dst, want["fanout"], num_src)
-                assert f["csc_indptr"].numel() == num_dst + 1 and f["csr_indptr"].numel() == num_src + 1
+                assert f["csc_indptr"].numel() == num_dst + 1
+                if what == "csc":
+                    assert "csr_indptr" not in f
+                    _same({k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in f.items()}, ref,
+                          keys=("coo_row", "coo_col", "csc_indptr"))
+                    continue
+                assert f["csr_indptr"].numel() == num_src + 1
                 _same({k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in f.items()}, ref)
