@@ -102,7 +102,10 @@ __device__ __forceinline__ bool in_table(const HopParams& p, int64_t v) {
 constexpr int kBeginBlocks = 64;
 
 __global__ __launch_bounds__(kMbBlock) void mb_begin_kernel(uint4* table, int64_t vecs, uint32_t* state,
-                                                            uint32_t payload_bits) {
+                                                            uint32_t payload_bits, int64_t* sizes,
+                                                            int num_sizes, int64_t batch) {
+  // per-batch counters: sizes[0] = batch, the rest 0
+  if (blockIdx.x == 0 && static_cast<int>(threadIdx.x) < num_sizes) sizes[threadIdx.x] = threadIdx.x == 0 ? batch : 0;
   const bool refill = state[1] != payload_bits || state[0] == 0;
   if (refill) {
     const uint4 ones = make_uint4(kEmpty, kEmpty, kEmpty, kEmpty);
@@ -124,7 +127,8 @@ __global__ __launch_bounds__(kMbBlock) void mb_begin_kernel(uint4* table, int64_
 }
 
 // First hop only: seeds may repeat, so they race like everything else; the
-// smallest seed index owns the node.  Also clears the per-batch counters.
+// smallest seed index owns the node.  (Also sets the per-batch counters, as the
+// first kernel of the batch already has.)
 __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, int64_t* sizes,
                                                                  int num_sizes) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x;
@@ -441,7 +445,7 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     // next epoch; refills only when the epochs are used up (or the table is new)
     const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
     hipLaunchKernelGGL(mb_begin_kernel, dim3(kBeginBlocks), dim3(kMbBlock), 0, st,
-                       static_cast<uint4*>(rank_table), vecs, state, L.payload_bits);
+                       static_cast<uint4*>(rank_table), vecs, state, L.payload_bits, sizes, num_hops + 2, batch);
     APT_LAUNCH_CHECK("mb_begin_kernel");
   }
 
@@ -457,8 +461,9 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   hp.ns_cap = batch;
   hp.ns_dev = nullptr;
 
-  // sizes[0] = batch, the rest 0; first-hop seeds bid for their nodes.
-  {
+  // First-hop seeds bid for their nodes: inside the sampling kernel when it does
+  // the marking, else in a pass of their own.
+  if (!(hop_fanouts[0] <= kWave && tuning_fuse_mark() != 0)) {
     const int64_t work = std::max<int64_t>(batch, num_hops + 2);
     hipLaunchKernelGGL(mb_mark_seeds_kernel, dim3(static_cast<unsigned>(ceil_div(work, kMbBlock))),
                        dim3(kMbBlock), 0, st, hp, sizes, num_hops + 2);

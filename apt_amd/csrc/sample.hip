@@ -185,6 +185,10 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
             node = s_node[t];
             src[u] = s_nbrs[t];
           }
+          // First hop of the fused driver: the row's seed bids for its node with
+          // its own index, like its neighbours below (seeds may repeat).
+          if (p.first_hop != 0 && p.table.entries != nullptr && l == 0 && node >= 0 && node < p.table.len)
+            atomicMin(&p.table.entries[node], table_base(p.table.state) + static_cast<uint32_t>(gis[u]));
           pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, node, seed, p.hop);
           if (l == 0) {
             const int64_t cnt = REPLACE ? (deg > 0 ? fanout : 0) : (deg < fanout ? deg : fanout);
