@@ -194,9 +194,9 @@ def load_partition(rank, min_vids, localnode_feats_idx, localnode_feats, labels,
     graph = capi.Graph(indptr, indices, row_begin=row_begin, num_total_nodes=num_total_nodes)
     c_indptr, c_indices = build_graph_cache(graph, cache_graph_node_idx)
     if row_begin:
-        ops.register_graph_partition(indptr, indices, row_begin, num_total_nodes)
         if cache_graph_node_idx.numel():
             raise ValueError("a graph cache on top of a range partition is not supported")
+        ops.register_graph_partition(indptr, indices, row_begin, num_total_nodes)
     else:
         ops.mix_cache_graphs(cache_graph_node_idx.numel(), cache_graph_node_idx, c_indptr, c_indices, indptr, indices)
     # feature cache
