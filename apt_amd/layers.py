@@ -63,6 +63,33 @@ class SAGEConv(nn.Module):
         return self.activation(rst) if self.activation is not None else rst
 
 
+class GraphConv(nn.Module):
+    """GCN layer with the reference's arithmetic (python/npc/model/graphconv.py:
+    159-232, MPGraphConv): the fanout stands in for the degrees in the
+    normalisation ("both": fanout^-1/2 on either side, "left"/"right": 1/fanout
+    on one), the weight is applied before the sum."""
+
+    def __init__(self, in_feats, out_feats, norm="both", bias=True, activation=None):
+        super().__init__()
+        if norm not in ("none", "both", "right", "left"):
+            raise KeyError(f'Invalid norm value. Must be either "none", "both", "right" or "left". But got "{norm}".')
+        self.norm, self.activation = norm, activation
+        self.weight = nn.Parameter(torch.empty(in_feats, out_feats))
+        self.bias = nn.Parameter(torch.zeros(out_feats)) if bias else None
+        nn.init.xavier_uniform_(self.weight)
+
+    def forward(self, block, feat):
+        fanout = float(block.fanout)
+        if self.norm in ("left", "both"):
+            feat = feat * (fanout ** -0.5 if self.norm == "both" else 1.0 / fanout)
+        rst = BlockAggregate.apply(block, torch.matmul(feat, self.weight), False)
+        if self.norm in ("right", "both"):
+            rst = rst * (fanout ** -0.5 if self.norm == "both" else 1.0 / fanout)
+        if self.bias is not None:
+            rst = rst + self.bias
+        return self.activation(rst) if self.activation is not None else rst
+
+
 class GATConv(nn.Module):
     """GAT layer forward (python/npc/model/gatconv.py:207-236: fc, attention
     logits, LeakyReLU, edge softmax, weighted sum, bias) in two kernels.

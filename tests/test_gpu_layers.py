@@ -46,6 +46,25 @@ def test_block_aggregate_gradients():
             assert torch.equal(out3, out) and torch.equal(X3.grad, X.grad)
 
 
+def test_graphconv_matches_dense_statement():
+    import apt_amd as npc
+    from apt_amd.layers import GraphConv
+    _setup_graph(seed=4)
+    sampler = npc.MixedPSNeighborSampler(0, 1, [5], "DP", replace=True, rng_seed=6)
+    seeds = torch.from_numpy(np.random.default_rng(2).permutation(6000)[:150]).to(DEV)
+    _, _, (blk,) = sampler.sample(None, seeds)
+    for norm, scale in (("both", 1 / 5.0), ("right", 1 / 5.0), ("left", 1 / 5.0), ("none", 1.0)):
+        layer = GraphConv(12, 7, norm=norm).to(DEV)
+        feat = torch.randn(blk.num_src, 12, device=DEV, requires_grad=True)
+        got = layer(blk, feat)
+        h = feat @ layer.weight
+        want = torch.zeros(blk.num_dst, 7, device=DEV).index_add(0, blk.col, h[blk.row]) * scale + layer.bias
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-5), norm
+        g1, = torch.autograd.grad(got.sum(), feat, retain_graph=True)
+        g2, = torch.autograd.grad(want.sum(), feat)
+        assert torch.allclose(g1, g2, rtol=1e-5, atol=1e-5), norm
+
+
 def test_gat_layer_matches_dense_statement():
     import apt_amd as npc
     from apt_amd.layers import GATConv
