@@ -72,6 +72,8 @@ SYMBOLS = {
     "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
     "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
     "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
+    "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
+    "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _I, _I64, _I, _P, _I64, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
@@ -625,4 +627,32 @@ def vir_send_offset(world_size, base, sorted_nodes, unique_nodes, with_dst=False
     out = torch.empty(world_size * (3 if with_dst else 2) + 1, dtype=torch.int64, device=sorted_nodes.device)
     check(lib().apt_vir_send_offset(int(world_size), int(base), _ptr(sorted_nodes), sorted_nodes.numel(),
                                     _ptr(unique_nodes), unique_nodes.numel(), int(with_dst), _ptr(out), _stream()))
+    return out
+
+
+def gat_block_backward(neighbors, num_dst, fanout, ft, el, er, negative_slope, attn, d_out, csc_indptr, num_edges):
+    """Edge half of the backward pass of gat_block -> (a_edge [E, heads], dz_edge [E, heads], d_er [num_dst, heads])."""
+    num_src, heads, dim = ft.shape
+    dev = ft.device
+    a_edge = torch.empty((num_edges, heads), dtype=torch.float32, device=dev)
+    dz_edge = torch.empty((num_edges, heads), dtype=torch.float32, device=dev)
+    d_er = torch.empty((num_dst, heads), dtype=torch.float32, device=dev)
+    check(lib().apt_gat_block_backward(_ptr(_dev_i64(neighbors, "neighbors")), int(num_dst), int(fanout), _ptr(ft),
+                                       num_src, heads, dim, ft.element_size(), _ptr(_f32(el, "el")),
+                                       _ptr(_f32(er, "er")), float(negative_slope), _ptr(_f32(attn, "attn")),
+                                       _ptr(_f32(d_out, "d_out")), _ptr(_dev_i64(csc_indptr, "csc_indptr")),
+                                       _ptr(a_edge), _ptr(dz_edge), _ptr(d_er), _stream()))
+    return a_edge, dz_edge, d_er
+
+
+def spmm_heads(row, col, x, head_weights, num_out):
+    """out[col[e], h, :] += head_weights[e, h] * x[row[e], h, :]; x [n, heads, head_dim] -> fp32 [num_out, heads, head_dim]."""
+    row, col = _dev_i64(row, "row"), _dev_i64(col, "col")
+    n, heads, hd = x.shape
+    w = _f32(head_weights, "head_weights")
+    if tuple(w.shape) != (row.numel(), heads) or not x.is_contiguous():
+        raise AptError("spmm_heads: head_weights must be [E, heads] and x contiguous")
+    out = torch.zeros((num_out, heads, hd), dtype=torch.float32, device=x.device)
+    check(lib().apt_spmm_heads(_ptr(row), _ptr(col), row.numel(), _ptr(x), n, _ptr(w), heads, heads * hd,
+                               x.element_size(), _ptr(out), num_out, _stream()))
     return out

@@ -34,6 +34,9 @@ struct AggParams {
   int num_seg;
   int64_t dim;
   int64_t num_in_rows, num_e_rows, num_out_rows;
+  const float* head_w;      // MODE 3: [E, heads] scalar per edge and head
+  int heads;
+  int64_t head_dim;         // dim / heads
 };
 
 template <typename T> __device__ __forceinline__ float to_float(T v);
@@ -71,6 +74,7 @@ __device__ __forceinline__ void load_vec(const T* base, int64_t elem, float (&v)
 // MODE 0: copy_u  acc += in[in_off + src]
 // MODE 1: copy_e  acc += in[e]
 // MODE 2: u_mul_e acc += in[in_off + src] * edata[e]
+// MODE 3: acc += in[in_off + src] * head_w[e, head of the feature] (VEC divides head_dim)
 // A lane owns VEC consecutive features; kUnroll edges are loaded before they
 // are accumulated.
 template <typename T, int MODE, int VEC>
@@ -78,7 +82,7 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
   constexpr int kUnroll = 4;
   __shared__ int64_t s_off[kMaxSegments + 1];
   __shared__ int64_t s_in[kMaxSegments], s_out[kMaxSegments];
-  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off[threadIdx.x];
+  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off != nullptr ? p.coo_off[threadIdx.x] : 0;  // NULL: one segment
   if (threadIdx.x < p.num_seg) {
     s_in[threadIdx.x] = p.in_off != nullptr ? p.in_off[threadIdx.x] : 0;
     s_out[threadIdx.x] = p.out_off != nullptr ? p.out_off[threadIdx.x] : 0;
@@ -128,6 +132,11 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) v[u][i] *= w[i];
               }
+              if (MODE == 3) {
+                const float w = p.head_w[e * p.heads + d / p.head_dim];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) v[u][i] *= w;
+              }
             }
           }
         }
@@ -155,7 +164,7 @@ template <typename T, int OP>
 __global__ __launch_bounds__(kAggBlock) void sddmm_kernel(AggParams p) {
   __shared__ int64_t s_off[kMaxSegments + 1];
   __shared__ int64_t s_l[kMaxSegments], s_r[kMaxSegments];
-  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off[threadIdx.x];
+  if (threadIdx.x <= p.num_seg) s_off[threadIdx.x] = p.coo_off != nullptr ? p.coo_off[threadIdx.x] : 0;  // NULL: one segment
   if (threadIdx.x < p.num_seg) {
     s_l[threadIdx.x] = p.in_off != nullptr ? p.in_off[threadIdx.x] : 0;
     s_r[threadIdx.x] = p.out_off != nullptr ? p.out_off[threadIdx.x] : 0;
@@ -401,6 +410,64 @@ static void launch_gat(const int64_t* nbr, int64_t num_dst, const int64_t* num_d
 #undef APT_GAT
 }
 
+// Backward of gat_ell_kernel, edge half.  A wavefront per (destination, head):
+// with a = softmax(e) and out = sum a_k ft[s_k],
+//   g_k  = dOut . ft[s_k]                     (gradient wrt a_k)
+//   de_k = a_k (g_k - sum_j a_j g_j)          (softmax)
+//   dz_k = de_k * (z_k > 0 ? 1 : slope)       (LeakyReLU, z_k = el[s_k] + er[i])
+// Lane k keeps slot k (fanout <= 64).  Written in the block's COO order (edge
+// id = csc_indptr[i] + rank of the slot among the row's edges): the attention
+// weight a and dz per edge and head, and der[i, h] = sum_k dz_k.  The source half
+// (d ft[s] = sum a dOut[dst], d el[s] = sum dz) is a sum over the edges of a
+// source and runs through the SpMM kernels on the block's CSR order.
+template <typename T>
+__global__ __launch_bounds__(kAggBlock) void gat_bwd_edge_kernel(
+    const int64_t* __restrict__ nbr, int64_t num_dst, int fanout, const T* __restrict__ ft, int64_t num_src,
+    int heads, int64_t dim, const float* __restrict__ el, const float* __restrict__ er, float slope,
+    const float* __restrict__ attn, const float* __restrict__ d_out, const int64_t* __restrict__ csc_indptr,
+    float* __restrict__ a_edge, float* __restrict__ dz_edge, float* __restrict__ d_er) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t items = num_dst * heads;
+  for (int64_t it = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave; it < items;
+       it += static_cast<int64_t>(gridDim.x) * kAggWaves) {
+    const int64_t i = it / heads;
+    const int h = static_cast<int>(it % heads);
+    const int64_t* ids = nbr + i * fanout;
+    const int64_t mine = lane < fanout ? ids[lane] : -1;
+    const bool valid = mine >= 0 && mine < num_src;
+    float g = 0.f;   // lane k: dOut[i, h] . ft[s_k, h]
+    for (int k = 0; k < fanout; ++k) {
+      const int64_t src = __shfl(mine, k, kWave);
+      if (src < 0 || src >= num_src) continue;   // wave-uniform
+      float part = 0.f;
+      for (int64_t d = lane; d < dim; d += kWave)
+        part += d_out[it * dim + d] * to_float<T>(ft[(src * heads + h) * dim + d]);
+#pragma unroll
+      for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+      if (lane == k) g = part;
+    }
+    const float a = valid ? attn[(i * fanout + lane) * heads + h] : 0.f;
+    float s = a * g;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, kWave);
+    float dz = 0.f;
+    if (valid) {
+      const float z = el[mine * heads + h] + er[it];
+      dz = a * (g - s) * (z > 0.f ? 1.f : slope);
+    }
+    float sum_dz = dz;
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) sum_dz += __shfl_xor(sum_dz, off, kWave);
+    const uint64_t m = ballot(valid);
+    if (valid) {
+      const int64_t e = csc_indptr[i] + rank_below(m);
+      a_edge[e * heads + h] = a;
+      dz_edge[e * heads + h] = dz;
+    }
+    if (lane == 0) d_er[it] = sum_dz;
+  }
+}
+
 static int agg_check(const char* who, const int64_t* row, const int64_t* col, int64_t E, const void* in,
                      float* out, const int64_t* coo_off, int num_seg, int64_t dim, int elem_size) {
   APT_REQUIRE(E >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (E %lld, dim %lld)", who, (long long)E,
@@ -587,5 +654,71 @@ extern "C" int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const in
     else launch_gat<uint16_t, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
   }
   APT_LAUNCH_CHECK("gat_ell_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+                              const void* input, int64_t num_in_rows, const float* head_weights, int heads,
+                              int64_t dim, int elem_size, float* out, int64_t num_out_rows, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_edges >= 0 && heads > 0 && dim > 0 && dim % heads == 0, APT_EINVAL,
+              "apt_spmm_heads: bad shape (E %lld, heads %d, dim %lld)", (long long)num_edges, heads,
+              (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_spmm_heads: elem_size %d (4 = fp32, 2 = bf16)",
+              elem_size);
+  APT_REQUIRE(num_out_rows >= 0 && num_in_rows >= 0, APT_EINVAL, "apt_spmm_heads: negative row count");
+  if (num_edges == 0) return APT_OK;
+  APT_REQUIRE(coo_row != nullptr && coo_col != nullptr && input != nullptr && head_weights != nullptr &&
+                  out != nullptr,
+              APT_EINVAL, "apt_spmm_heads: a tensor is NULL");
+  AggParams p{};
+  p.row = coo_row; p.col = coo_col; p.num_edges = num_edges; p.in = input; p.out = out;
+  p.num_seg = 1;  // no segment tables: every edge in segment 0, offsets 0
+  p.coo_off = nullptr;
+  p.dim = dim; p.num_in_rows = num_in_rows; p.num_e_rows = num_edges; p.num_out_rows = num_out_rows;
+  p.head_w = head_weights; p.heads = heads; p.head_dim = dim / heads;
+  const int64_t waves = ceil_div(num_edges, kEdgesPerWave);
+  const dim3 grid(static_cast<unsigned>(ceil_div(waves, kAggWaves))), block(kAggBlock);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec4 = p.head_dim % 4 == 0 && (reinterpret_cast<uintptr_t>(input) & 15) == 0;
+  if (elem_size == 4) {
+    if (vec4) hipLaunchKernelGGL((spmm_kernel<float, 3, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((spmm_kernel<float, 3, 1>), grid, block, 0, st, p);
+  } else {
+    if (vec4) hipLaunchKernelGGL((spmm_kernel<uint16_t, 3, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((spmm_kernel<uint16_t, 3, 1>), grid, block, 0, st, p);
+  }
+  APT_LAUNCH_CHECK("spmm_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst, int fanout, const void* ft,
+                                      int64_t num_src, int heads, int64_t dim, int elem_size, const float* el,
+                                      const float* er, float negative_slope, const float* attn,
+                                      const float* d_out, const int64_t* csc_indptr, float* a_edge,
+                                      float* dz_edge, float* d_er, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_dst >= 0 && fanout > 0 && fanout <= kWave && heads > 0 && dim > 0 && num_src >= 0, APT_EINVAL,
+              "apt_gat_block_backward: bad shape (num_dst %lld, fanout %d (1..64), heads %d, dim %lld)",
+              (long long)num_dst, fanout, heads, (long long)dim);
+  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL,
+              "apt_gat_block_backward: elem_size %d (4 = fp32, 2 = bf16)", elem_size);
+  if (num_dst == 0) return APT_OK;
+  APT_REQUIRE(neighbors != nullptr && ft != nullptr && el != nullptr && er != nullptr && attn != nullptr &&
+                  d_out != nullptr && csc_indptr != nullptr && a_edge != nullptr && dz_edge != nullptr &&
+                  d_er != nullptr,
+              APT_EINVAL, "apt_gat_block_backward: a tensor is NULL");
+  const unsigned blocks =
+      static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst * heads, kAggWaves), 1 << 20));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (elem_size == 4)
+    hipLaunchKernelGGL(gat_bwd_edge_kernel<float>, dim3(blocks), dim3(kAggBlock), 0, st, neighbors, num_dst,
+                       fanout, static_cast<const float*>(ft), num_src, heads, dim, el, er, negative_slope, attn,
+                       d_out, csc_indptr, a_edge, dz_edge, d_er);
+  else
+    hipLaunchKernelGGL(gat_bwd_edge_kernel<uint16_t>, dim3(blocks), dim3(kAggBlock), 0, st, neighbors, num_dst,
+                       fanout, static_cast<const uint16_t*>(ft), num_src, heads, dim, el, er, negative_slope, attn,
+                       d_out, csc_indptr, a_edge, dz_edge, d_er);
+  APT_LAUNCH_CHECK("gat_bwd_edge_kernel");
   return APT_OK;
 }

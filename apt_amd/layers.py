@@ -90,10 +90,43 @@ class GraphConv(nn.Module):
         return self.activation(rst) if self.activation is not None else rst
 
 
+class GATAggregate(torch.autograd.Function):
+    """out[d, h] = sum over the block's edges (s -> d) of softmax_d(LeakyReLU(el[s, h] + er[d, h])) * ft[s, h]
+    (python/npc/model/gatconv.py:118-126), forward and backward fused over the
+    block: forward = one kernel from the fixed-stride layout; backward = one
+    kernel per (destination, head) for the logit gradients, then the two sums
+    over the edges of a source on the block's CSR order."""
+
+    @staticmethod
+    def forward(ctx, block, ft, el, er, negative_slope):
+        ft, el, er = ft.contiguous(), el.contiguous().float(), er.contiguous().float()
+        out, attn = capi.gat_block(block.relabeled, block.num_dst, block.fanout, ft, el, er, negative_slope,
+                                   want_attn=True)
+        ctx.block, ctx.slope = block, negative_slope
+        ctx.save_for_backward(ft, el, er, attn)
+        return out.to(ft.dtype) if ft.dtype != torch.float32 else out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        block = ctx.block
+        ft, el, er, attn = ctx.saved_tensors
+        d_out = d_out.contiguous().float()
+        csc_indptr = block.csc()[0]
+        _, dst, eids = block.csr()
+        E = eids.numel()
+        a_edge, dz_edge, d_er = capi.gat_block_backward(block.relabeled, block.num_dst, block.fanout, ft, el, er,
+                                                        ctx.slope, attn, d_out, csc_indptr, E)
+        src = block.row[eids]                                   # edges grouped by source
+        d_ft = capi.spmm_heads(dst, src, d_out, a_edge[eids].contiguous(), block.num_src)
+        d_el = capi.spmm_sum(1, dst, src, dz_edge[eids].contiguous(), block.num_src)
+        return None, d_ft.to(ft.dtype), d_el, d_er, None
+
+
 class GATConv(nn.Module):
-    """GAT layer forward (python/npc/model/gatconv.py:207-236: fc, attention
-    logits, LeakyReLU, edge softmax, weighted sum, bias) in two kernels.
-    Inference only: the fused aggregation has no backward pass."""
+    """GAT layer (python/npc/model/gatconv.py:207-236: fc, attention logits,
+    LeakyReLU, edge softmax, weighted sum, bias).  Under torch.no_grad() the
+    logits come from the library's kernel too; otherwise from torch, so that
+    autograd carries them, and the aggregation is GATAggregate."""
 
     def __init__(self, in_feats, out_feats, num_heads, negative_slope=0.2, bias=True, activation=None):
         super().__init__()
@@ -108,12 +141,16 @@ class GATConv(nn.Module):
         nn.init.xavier_normal_(self.attn_l, gain=gain)
         nn.init.xavier_normal_(self.attn_r, gain=gain)
 
-    @torch.no_grad()
     def forward(self, block, feat):
         ft = self.fc(feat).view(block.num_src, self.num_heads, self.out_feats).contiguous()
-        el = capi.gat_scores(ft, self.attn_l.detach().float().contiguous())
-        er = capi.gat_scores(ft[:block.num_dst].contiguous(), self.attn_r.detach().float().contiguous())
-        rst = capi.gat_block(block.relabeled, block.num_dst, block.fanout, ft, el, er, self.negative_slope)
+        if torch.is_grad_enabled() and (ft.requires_grad or self.attn_l.requires_grad):
+            el = (ft * self.attn_l).sum(-1)
+            er = (ft[:block.num_dst] * self.attn_r).sum(-1)
+            rst = GATAggregate.apply(block, ft, el, er, self.negative_slope)
+        else:
+            el = capi.gat_scores(ft, self.attn_l.detach().float().contiguous())
+            er = capi.gat_scores(ft[:block.num_dst].contiguous(), self.attn_r.detach().float().contiguous())
+            rst = capi.gat_block(block.relabeled, block.num_dst, block.fanout, ft, el, er, self.negative_slope)
         if self.bias is not None:
             rst = rst + self.bias.view(1, self.num_heads, self.out_feats)
         return self.activation(rst) if self.activation is not None else rst

@@ -431,6 +431,28 @@ int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_
                   const float* el, const float* er, float negative_slope, float* out,
                   float* attn_out, void* stream);
 
+/* Backward pass of apt_gat_block (no counterpart in the reference, whose GAT layer
+ * gets its gradients from DGL's autograd).  Edge half, one wavefront per
+ * (destination, head), fanout <= 64: from dOut [num_dst, heads, dim] and the
+ * forward's attention weights attn [num_dst * fanout, heads] it writes, in the
+ * block's COO order (edge id = csc_indptr[d] + rank of the slot among d's edges,
+ * see apt_block_formats), a_edge and dz_edge [E, heads] (attention weight;
+ * gradient of the logit before LeakyReLU) and d_er [num_dst, heads] = sum of dz
+ * over a destination's edges.  The source half is two sums over the edges of a
+ * source: d el = segment sum of dz_edge, d ft = apt_spmm_heads below.
+ *   apt_spmm_heads  out[col[e], h, :] += head_weights[e, h] * input[row[e], h, :]
+ *                   (dim = heads * head_dim features per row; out fp32, zero-filled
+ *                   by the caller; one segment).  With the edges in the block's CSR
+ *                   order it is deterministic, like apt_spmm_sum. */
+int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst, int fanout, const void* ft,
+                           int64_t num_src, int heads, int64_t dim, int elem_size, const float* el,
+                           const float* er, float negative_slope, const float* attn,
+                           const float* d_out, const int64_t* csc_indptr, float* a_edge,
+                           float* dz_edge, float* d_er, void* stream);
+int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
+                   const void* input, int64_t num_in_rows, const float* head_weights, int heads,
+                   int64_t dim, int elem_size, float* out, int64_t num_out_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,8 +74,8 @@ def test_gat_layer_matches_dense_statement():
     _, _, (blk,) = sampler.sample(None, seeds)
     layer = GATConv(16, 8, 3).to(DEV)
     feat = torch.randn(blk.num_src, 16, device=DEV)
-    got = layer(blk, feat)
     with torch.no_grad():
+        got = layer(blk, feat)
         ft = layer.fc(feat).view(-1, 3, 8)
         el, er = (ft * layer.attn_l).sum(-1), (ft[:blk.num_dst] * layer.attn_r).sum(-1)
         e = torch.nn.functional.leaky_relu(el[blk.row] + er[blk.col], 0.2)            # [E, H]
@@ -86,6 +86,43 @@ def test_gat_layer_matches_dense_statement():
         want = torch.zeros(blk.num_dst, 3, 8, device=DEV).index_add(0, blk.col, a[:, :, None] * ft[blk.row])
         want = want + layer.bias.view(1, 3, 8)
     assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+def _gat_dense(layer, blk, feat):
+    """The layer's textbook statement in plain torch (autograd gives the reference gradients)."""
+    H, D = layer.num_heads, layer.out_feats
+    ft = layer.fc(feat).view(-1, H, D)
+    el, er = (ft * layer.attn_l).sum(-1), (ft[:blk.num_dst] * layer.attn_r).sum(-1)
+    e = torch.nn.functional.leaky_relu(el[blk.row] + er[blk.col], layer.negative_slope)
+    top = torch.full((blk.num_dst, H), -1e30, device=DEV).scatter_reduce(0, blk.col[:, None].expand(-1, H), e.detach(), "amax")
+    w = torch.exp(e - top[blk.col])
+    den = torch.zeros(blk.num_dst, H, device=DEV).index_add(0, blk.col, w)
+    a = w / den[blk.col]
+    out = torch.zeros(blk.num_dst, H, D, device=DEV).index_add(0, blk.col, a[:, :, None] * ft[blk.row])
+    return out + layer.bias.view(1, H, D)
+
+
+@pytest.mark.parametrize("heads,dim", [(3, 8), (4, 64), (1, 5), (2, 100)])
+def test_gat_layer_gradients(heads, dim):
+    import apt_amd as npc
+    from apt_amd.layers import GATConv
+    _setup_graph(seed=5)
+    sampler = npc.MixedPSNeighborSampler(0, 1, [9], "DP", replace=False, rng_seed=8)
+    seeds = torch.from_numpy(np.random.default_rng(3).permutation(6000)[:300]).to(DEV)
+    _, _, (blk,) = sampler.sample(None, seeds)
+    torch.manual_seed(1)
+    layer = GATConv(20, dim, heads).to(DEV)
+    feat = torch.randn(blk.num_src, 20, device=DEV, requires_grad=True)
+    w = torch.randn(blk.num_dst, heads, dim, device=DEV)
+    got = layer(blk, feat)
+    params = [feat, layer.fc.weight, layer.attn_l, layer.attn_r]
+    g_got = torch.autograd.grad((got * w).sum(), params)
+    want = _gat_dense(layer, blk, feat)
+    g_want = torch.autograd.grad((want * w).sum(), params)
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+    for a, b, name in zip(g_got, g_want, ("feat", "fc", "attn_l", "attn_r")):
+        scale = b.abs().max().item() + 1e-12
+        assert (a - b).abs().max().item() <= 2e-4 * scale, (name, (a - b).abs().max().item(), scale)
 
 
 def test_sage_trains_on_sampled_batches():
