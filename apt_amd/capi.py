@@ -73,7 +73,7 @@ SYMBOLS = {
     "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
     "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
     "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
-    "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _I, _I64, _I, _P, _I64, _P]),
+    "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
@@ -645,14 +645,26 @@ def gat_block_backward(neighbors, num_dst, fanout, ft, el, er, negative_slope, a
     return a_edge, dz_edge, d_er
 
 
-def spmm_heads(row, col, x, head_weights, num_out):
-    """out[col[e], h, :] += head_weights[e, h] * x[row[e], h, :]; x [n, heads, head_dim] -> fp32 [num_out, heads, head_dim]."""
+def spmm_heads(row, col, x, head_weights, num_out, weight_row=None, grouped=False, head_weights2=None):
+    """out[col[e], h, :] += head_weights[w(e), h] * x[row[e], h, :], w(e) = weight_row[e] or e;
+    x [n, heads, head_dim] -> fp32 [num_out, heads, head_dim].  grouped: edges with equal col are consecutive.
+    head_weights2: also returns out2[col[e], h] += head_weights2[w(e), h]."""
     row, col = _dev_i64(row, "row"), _dev_i64(col, "col")
+    weight_row = _dev_i64(weight_row, "weight_row")
     n, heads, hd = x.shape
     w = _f32(head_weights, "head_weights")
-    if tuple(w.shape) != (row.numel(), heads) or not x.is_contiguous():
-        raise AptError("spmm_heads: head_weights must be [E, heads] and x contiguous")
+    if w.dim() != 2 or w.shape[1] != heads or not x.is_contiguous():
+        raise AptError("spmm_heads: head_weights must be [*, heads] and x contiguous")
+    if weight_row is None and w.shape[0] != row.numel():
+        raise AptError("spmm_heads: head_weights needs one row per edge")
     out = torch.zeros((num_out, heads, hd), dtype=torch.float32, device=x.device)
-    check(lib().apt_spmm_heads(_ptr(row), _ptr(col), row.numel(), _ptr(x), n, _ptr(w), heads, heads * hd,
-                               x.element_size(), _ptr(out), num_out, _stream()))
-    return out
+    out2 = None
+    if head_weights2 is not None:
+        head_weights2 = _f32(head_weights2, "head_weights2")
+        if head_weights2.shape != w.shape:
+            raise AptError("spmm_heads: head_weights2 must have the shape of head_weights")
+        out2 = torch.zeros((num_out, heads), dtype=torch.float32, device=x.device)
+    check(lib().apt_spmm_heads(_ptr(row), _ptr(col), row.numel(), _ptr(x), n, _ptr(w), _ptr(weight_row), heads,
+                               heads * hd, x.element_size(), int(grouped), _ptr(out), num_out, _ptr(head_weights2),
+                               _ptr(out2), _stream()))
+    return out if out2 is None else (out, out2)

@@ -35,8 +35,12 @@ struct AggParams {
   int64_t dim;
   int64_t num_in_rows, num_e_rows, num_out_rows;
   const float* head_w;      // MODE 3: [E, heads] scalar per edge and head
+  const int64_t* head_w_row;  // MODE 3: row of head_w for edge e (NULL = e)
+  const float* head_w2;     // MODE 3, optional: second [*, heads] table, summed per output row and head ...
+  float* out2;              // ... into out2 [num_out, heads]
   int heads;
   int64_t head_dim;         // dim / heads
+  int grouped;              // edges with equal col are consecutive: rows inside a wavefront's range are stored, not added
 };
 
 template <typename T> __device__ __forceinline__ float to_float(T v);
@@ -102,19 +106,33 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     int64_t cur = -1;
-    auto flush = [&]() {
+    bool first_row = true;  // the row at the start of the range may have begun in the previous wavefront's range
+    // MODE 3: the lane holding a head's first features also sums the second weight table
+    const bool second = MODE == 3 && p.head_w2 != nullptr && live && d % p.head_dim == 0;
+    float acc2 = 0.f;
+    auto flush = [&](bool last_row) {
       if (cur >= 0 && cur < p.num_out_rows && live) {
+        if (p.grouped && !first_row && !last_row) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) atomicAdd(&p.out[cur * p.dim + d + i], acc[i]);
+          for (int i = 0; i < VEC; ++i) p.out[cur * p.dim + d + i] = acc[i];
+          if (second) p.out2[cur * p.heads + d / p.head_dim] = acc2;
+        } else {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) atomicAdd(&p.out[cur * p.dim + d + i], acc[i]);
+          if (second) atomicAdd(&p.out2[cur * p.heads + d / p.head_dim], acc2);
+        }
       }
+      if (cur >= 0) first_row = false;
     };
     for (int64_t eb = e0; eb < e1; eb += kUnroll) {
       float v[kUnroll][VEC];
+      float v2[kUnroll];
       int64_t dst[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
         const int64_t e = eb + u;
         dst[u] = -1;
+        v2[u] = 0.f;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v[u][i] = 0.f;
         if (e < e1) {
@@ -133,9 +151,11 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
                 for (int i = 0; i < VEC; ++i) v[u][i] *= w[i];
               }
               if (MODE == 3) {
-                const float w = p.head_w[e * p.heads + d / p.head_dim];
+                const int64_t we = p.head_w_row != nullptr ? p.head_w_row[e] : e;
+                const float w = p.head_w[we * p.heads + d / p.head_dim];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) v[u][i] *= w;
+                if (second) v2[u] = p.head_w2[we * p.heads + d / p.head_dim];
               }
             }
           }
@@ -145,17 +165,19 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
       for (int u = 0; u < kUnroll; ++u) {
         if (eb + u < e1) {
           if (dst[u] != cur) {
-            flush();
+            flush(false);
 #pragma unroll
             for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+            acc2 = 0.f;
             cur = dst[u];
           }
 #pragma unroll
           for (int i = 0; i < VEC; ++i) acc[i] += v[u][i];
+          acc2 += v2[u];
         }
       }
     }
-    flush();
+    flush(true);
   }
 }
 
@@ -468,6 +490,109 @@ __global__ __launch_bounds__(kAggBlock) void gat_bwd_edge_kernel(
   }
 }
 
+// The same on a lane group per destination row, for rows that fit one pass of
+// the group: LPH = dim / VEC lanes per head (a power of two), heads * LPH <= G
+// lanes.  The row's source features are read once, VEC per lane; the dot of a
+// slot is reduced over the head's lanes with xor shuffles and parked in
+// dz_edge until the row's sum is known.
+template <typename T, int VEC, int G>
+__global__ __launch_bounds__(kAggBlock) void gat_bwd_edge_group_kernel(
+    const int64_t* __restrict__ nbr, int64_t num_dst, int fanout, const T* __restrict__ ft, int64_t num_src,
+    int heads, int64_t dim, const float* __restrict__ el, const float* __restrict__ er, float slope,
+    const float* __restrict__ attn, const float* __restrict__ d_out, const int64_t* __restrict__ csc_indptr,
+    float* __restrict__ a_edge, float* __restrict__ dz_edge, float* __restrict__ d_er) {
+  constexpr int kGroups = kAggBlock / G;
+  constexpr int kUnroll = 5;
+  const int lph = static_cast<int>(dim / VEC);
+  const int64_t row_len = static_cast<int64_t>(heads) * dim;
+  const int grp = threadIdx.x / G, l = threadIdx.x % G;
+  const bool live = l < heads * lph;
+  const int h = live ? l / lph : 0;
+  const bool leader = live && l % lph == 0;
+  const int64_t d = static_cast<int64_t>(l) * VEC;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kGroups + grp; i < num_dst;
+       i += static_cast<int64_t>(gridDim.x) * kGroups) {
+    const int64_t* ids = nbr + i * fanout;
+    const int64_t e0 = csc_indptr[i];
+    float go[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) go[q] = live ? d_out[i * row_len + d + q] : 0.f;
+    float s = 0.f;
+    int64_t e = e0;
+    for (int k0 = 0; k0 < fanout; k0 += kUnroll) {
+      float v[kUnroll][VEC];
+      bool ok[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        ok[u] = false;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) v[u][q] = 0.f;
+        if (k0 + u < fanout) {
+          const int64_t src = ids[k0 + u];
+          if (src >= 0 && src < num_src) {
+            ok[u] = true;
+            if (live) load_vec<T, VEC>(ft, src * row_len + d, v[u]);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        if (!ok[u]) continue;  // group-uniform
+        float part = 0.f;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) part += go[q] * v[u][q];
+        for (int off = lph / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+        if (leader) {
+          s += attn[(i * fanout + k0 + u) * heads + h] * part;
+          dz_edge[e * heads + h] = part;
+        }
+        ++e;
+      }
+    }
+    if (leader) {
+      const float er_i = er[i * heads + h];
+      float sum_dz = 0.f;
+      e = e0;
+      for (int k = 0; k < fanout; ++k) {
+        const int64_t src = ids[k];
+        if (src < 0 || src >= num_src) continue;
+        const float a = attn[(i * fanout + k) * heads + h];
+        const float z = el[src * heads + h] + er_i;
+        const float dz = a * (dz_edge[e * heads + h] - s) * (z > 0.f ? 1.f : slope);
+        a_edge[e * heads + h] = a;
+        dz_edge[e * heads + h] = dz;
+        sum_dz += dz;
+        ++e;
+      }
+      d_er[i * heads + h] = sum_dz;
+    }
+  }
+}
+
+template <typename T, int VEC>
+static bool launch_gat_bwd_group(const int64_t* nbr, int64_t num_dst, int fanout, const void* ft, int64_t num_src,
+                                 int heads, int64_t dim, const float* el, const float* er, float slope,
+                                 const float* attn, const float* d_out, const int64_t* csc_indptr, float* a_edge,
+                                 float* dz_edge, float* d_er, hipStream_t st) {
+  if (dim % VEC != 0) return false;
+  const int64_t lph = dim / VEC;
+  if (lph > kWave || (lph & (lph - 1)) != 0 || heads * lph > kWave) return false;
+  if ((reinterpret_cast<uintptr_t>(ft) & 15) != 0) return false;
+  const int64_t lanes = heads * lph;
+  const T* x = static_cast<const T*>(ft);
+#define APT_GATB(G)                                                                                   \
+  hipLaunchKernelGGL((gat_bwd_edge_group_kernel<T, VEC, G>),                                          \
+                     dim3(static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst, kAggBlock / G), 1 << 20))), \
+                     dim3(kAggBlock), 0, st, nbr, num_dst, fanout, x, num_src, heads, dim, el, er, slope, attn, \
+                     d_out, csc_indptr, a_edge, dz_edge, d_er)
+  if (lanes <= 8) APT_GATB(8);
+  else if (lanes <= 16) APT_GATB(16);
+  else if (lanes <= 32) APT_GATB(32);
+  else APT_GATB(64);
+#undef APT_GATB
+  return true;
+}
+
 static int agg_check(const char* who, const int64_t* row, const int64_t* col, int64_t E, const void* in,
                      float* out, const int64_t* coo_off, int num_seg, int64_t dim, int elem_size) {
   APT_REQUIRE(E >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (E %lld, dim %lld)", who, (long long)E,
@@ -658,8 +783,10 @@ extern "C" int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const in
 }
 
 extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
-                              const void* input, int64_t num_in_rows, const float* head_weights, int heads,
-                              int64_t dim, int elem_size, float* out, int64_t num_out_rows, void* stream) {
+                              const void* input, int64_t num_in_rows, const float* head_weights,
+                              const int64_t* weight_row, int heads, int64_t dim, int elem_size, int grouped,
+                              float* out, int64_t num_out_rows, const float* head_weights2, float* out2,
+                              void* stream) {
   using namespace apt;
   APT_REQUIRE(num_edges >= 0 && heads > 0 && dim > 0 && dim % heads == 0, APT_EINVAL,
               "apt_spmm_heads: bad shape (E %lld, heads %d, dim %lld)", (long long)num_edges, heads,
@@ -676,7 +803,11 @@ extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, in
   p.num_seg = 1;  // no segment tables: every edge in segment 0, offsets 0
   p.coo_off = nullptr;
   p.dim = dim; p.num_in_rows = num_in_rows; p.num_e_rows = num_edges; p.num_out_rows = num_out_rows;
-  p.head_w = head_weights; p.heads = heads; p.head_dim = dim / heads;
+  p.head_w = head_weights; p.head_w_row = weight_row; p.heads = heads; p.head_dim = dim / heads;
+  p.grouped = grouped != 0;
+  APT_REQUIRE((head_weights2 == nullptr) == (out2 == nullptr), APT_EINVAL,
+              "apt_spmm_heads: head_weights2 and out2 go together");
+  p.head_w2 = head_weights2; p.out2 = out2;
   const int64_t waves = ceil_div(num_edges, kEdgesPerWave);
   const dim3 grid(static_cast<unsigned>(ceil_div(waves, kAggWaves))), block(kAggBlock);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -711,6 +842,18 @@ extern "C" int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst,
   const unsigned blocks =
       static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst * heads, kAggWaves), 1 << 20));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool grouped =
+      elem_size == 4
+          ? launch_gat_bwd_group<float, 4>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,
+                                           negative_slope, attn, d_out, csc_indptr, a_edge, dz_edge, d_er, st)
+          : (launch_gat_bwd_group<uint16_t, 8>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,
+                                               negative_slope, attn, d_out, csc_indptr, a_edge, dz_edge, d_er, st) ||
+             launch_gat_bwd_group<uint16_t, 4>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,
+                                               negative_slope, attn, d_out, csc_indptr, a_edge, dz_edge, d_er, st));
+  if (grouped) {
+    APT_LAUNCH_CHECK("gat_bwd_edge_group_kernel");
+    return APT_OK;
+  }
   if (elem_size == 4)
     hipLaunchKernelGGL(gat_bwd_edge_kernel<float>, dim3(blocks), dim3(kAggBlock), 0, st, neighbors, num_dst,
                        fanout, static_cast<const float*>(ft), num_src, heads, dim, el, er, negative_slope, attn,

@@ -117,8 +117,8 @@ class GATAggregate(torch.autograd.Function):
         a_edge, dz_edge, d_er = capi.gat_block_backward(block.relabeled, block.num_dst, block.fanout, ft, el, er,
                                                         ctx.slope, attn, d_out, csc_indptr, E)
         src = block.row[eids]                                   # edges grouped by source
-        d_ft = capi.spmm_heads(dst, src, d_out, a_edge[eids].contiguous(), block.num_src)
-        d_el = capi.spmm_sum(1, dst, src, dz_edge[eids].contiguous(), block.num_src)
+        d_ft, d_el = capi.spmm_heads(dst, src, d_out, a_edge, block.num_src, weight_row=eids, grouped=True,
+                                     head_weights2=dz_edge)
         return None, d_ft.to(ft.dtype), d_el, d_er, None
 
 

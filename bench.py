@@ -357,7 +357,28 @@ def main():
                 t = e0.elapsed_time(e1) / 10 * 1e-3
                 agg[f"{tag}_{name}_us"] = t * 1e6
                 agg[f"{tag}_{name}_GBps"] = nbytes / t / 1e9
-            del ft, el, er
+            # backward of the aggregation: logit gradients per (destination, head), then the sums over the
+            # edges of a source on the block's CSR order
+            fmt_b = capi.block_formats(rel, n_dst, f, n_src)
+            _, attn_w = capi.gat_block(rel, n_dst, f, ft, el, er, 0.2, want_attn=True)
+            d_out = torch.randn(n_dst, heads, hdim, device=dev)
+            src_csr = fmt_b["coo_row"][fmt_b["csr_eids"]].contiguous()
+
+            def gat_bwd():
+                a_e, dz_e, d_er = capi.gat_block_backward(rel, n_dst, f, ft, el, er, 0.2, attn_w, d_out,
+                                                          fmt_b["csc_indptr"], fmt_b["num_edges"])
+                capi.spmm_heads(fmt_b["csr_indices"], src_csr, d_out, a_e, n_src, weight_row=fmt_b["csr_eids"],
+                                grouped=True, head_weights2=dz_e)
+            for _ in range(3):
+                gat_bwd()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(10):
+                gat_bwd()
+            e1.record()
+            torch.cuda.synchronize()
+            agg[f"gat_block_backward_{name}_us"] = e0.elapsed_time(e1) / 10 * 1e3
+            del ft, el, er, fmt_b, attn_w, d_out
         hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
         h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)
         fn = lambda: capi.sddmm(0, row_e, col_e, h, hd)

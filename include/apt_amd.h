@@ -440,18 +440,26 @@ int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_
  * gradient of the logit before LeakyReLU) and d_er [num_dst, heads] = sum of dz
  * over a destination's edges.  The source half is two sums over the edges of a
  * source: d el = segment sum of dz_edge, d ft = apt_spmm_heads below.
- *   apt_spmm_heads  out[col[e], h, :] += head_weights[e, h] * input[row[e], h, :]
- *                   (dim = heads * head_dim features per row; out fp32, zero-filled
- *                   by the caller; one segment).  With the edges in the block's CSR
- *                   order it is deterministic, like apt_spmm_sum. */
+ *   apt_spmm_heads  out[col[e], h, :] += head_weights[w(e), h] * input[row[e], h, :],
+ *                   w(e) = weight_row[e] or e when weight_row is NULL (dim = heads *
+ *                   head_dim features per row; out fp32, zero-filled by the caller;
+ *                   one segment).  grouped != 0: the caller guarantees that edges
+ *                   with equal col are consecutive (the block's CSR order); rows that
+ *                   lie inside a wavefront's 64 edges are then stored without
+ *                   atomics and the result is deterministic.  head_weights2 / out2
+ *                   (both or neither): out2[col[e], h] += head_weights2[w(e), h], a
+ *                   second, scalar sum per row and head in the same pass (d el of
+ *                   the GAT backward); out2 fp32 [num_out_rows, heads], zero-filled. */
 int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst, int fanout, const void* ft,
                            int64_t num_src, int heads, int64_t dim, int elem_size, const float* el,
                            const float* er, float negative_slope, const float* attn,
                            const float* d_out, const int64_t* csc_indptr, float* a_edge,
                            float* dz_edge, float* d_er, void* stream);
 int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
-                   const void* input, int64_t num_in_rows, const float* head_weights, int heads,
-                   int64_t dim, int elem_size, float* out, int64_t num_out_rows, void* stream);
+                   const void* input, int64_t num_in_rows, const float* head_weights,
+                   const int64_t* weight_row, int heads, int64_t dim, int elem_size, int grouped,
+                   float* out, int64_t num_out_rows, const float* head_weights2, float* out2,
+                   void* stream);
 
 #ifdef __cplusplus
 }

@@ -125,6 +125,29 @@ def test_gat_layer_gradients(heads, dim):
         assert (a - b).abs().max().item() <= 2e-4 * scale, (name, (a - b).abs().max().item(), scale)
 
 
+@pytest.mark.parametrize("heads,dim", [(4, 64), (2, 16), (3, 24), (1, 40)])
+def test_gat_backward_bf16_matches_fp32_on_rounded_inputs(capi, heads, dim):
+    """bf16 features take other kernel variants (8 per lane); on the same (rounded)
+    values they must give what the fp32 variants give."""
+    rng = np.random.default_rng(heads * 100 + dim)
+    n_dst, fanout, n_src = 2000, 11, 9000
+    nbr = rng.integers(0, n_src, size=(n_dst, fanout)).astype(np.int64)
+    nbr[rng.random(nbr.shape) < 0.2] = -1
+    nbr = torch.from_numpy(nbr.reshape(-1)).to(DEV)
+    ft16 = torch.randn(n_src, heads, dim, device=DEV).to(torch.bfloat16)
+    ft32 = ft16.float()
+    el, er = torch.randn(n_src, heads, device=DEV), torch.randn(n_dst, heads, device=DEV)
+    d_out = torch.randn(n_dst, heads, dim, device=DEV)
+    fmt = capi.block_formats(nbr, n_dst, fanout, n_src, want_csr=False)
+    outs = []
+    for ft in (ft32, ft16):
+        _, attn = capi.gat_block(nbr, n_dst, fanout, ft, el, er, 0.2, want_attn=True)
+        outs.append(capi.gat_block_backward(nbr, n_dst, fanout, ft, el, er, 0.2, attn, d_out, fmt["csc_indptr"],
+                                            fmt["num_edges"]))
+    for a, b in zip(*outs):
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-5)
+
+
 def test_sage_trains_on_sampled_batches():
     """Two SAGE layers on sampled blocks + gathered features learn a label that
     depends on the neighbourhood: the loss falls well below its start."""
