@@ -89,6 +89,7 @@ class MiniBatchPipeline:
             self.format_fork = torch.cuda.Event()
             self.format_done = [torch.cuda.Event() for _ in self.fanouts]
         self.seeds = None
+        self.sizes_host = None
         self.graph_exec = None
         if use_graph:
             if not self.fused:
@@ -199,10 +200,24 @@ class MiniBatchPipeline:
             self.gather()
         self.join_formats()
 
-    def result(self):
+    def stage_sizes(self):
+        """Asynchronous copy of the batch's sizes (and request bucket sizes) to pinned
+        host memory on the current stream; result(staged=True) reads them once the
+        caller has waited for that stream, without a synchronous device read."""
+        if self.sizes_host is None:
+            self.sizes_host = torch.empty(self.sizes.numel(), dtype=torch.int64, pin_memory=True)
+            if self.requests is not None:
+                self.request_sizes_host = torch.empty(self.request_sizes.numel(), dtype=torch.int64,
+                                                      pin_memory=True)
+        self.sizes_host.copy_(self.sizes, non_blocking=True)
+        if self.requests is not None:
+            self.request_sizes_host.copy_(self.request_sizes, non_blocking=True)
+
+    def result(self, staged=False):
         """Waits for the batch and narrows the buffers to their real sizes ->
-        dict(input_nodes, blocks (outermost first), features, num_edges)."""
-        sizes = self.sizes.cpu().tolist()
+        dict(input_nodes, blocks (outermost first), features, num_edges).
+        staged: the sizes were copied by stage_sizes() and that copy has finished."""
+        sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
         H = len(self.fanouts)
         blocks = []
         for h, f in enumerate(self.fanouts):
@@ -222,7 +237,7 @@ class MiniBatchPipeline:
         out = dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],
                    sizes=sizes[:-1])
         if self.requests is not None:
-            rs = self.request_sizes.cpu().tolist()
+            rs = self.request_sizes_host.tolist() if staged else self.request_sizes.cpu().tolist()
             out.update(request_sizes=rs, request_ids=self.request_ids[:sizes[H]],
                        request_perm=self.request_perm[:sizes[H]],
                        features=None if self.features is None else self.features[:rs[0]])

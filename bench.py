@@ -291,6 +291,22 @@ def main():
         in_flight = {"batches_in_flight": len(pipes), "ms_per_step": t_fl / K * 1e3,
                      "edges_per_s": edges / t_fl}
         del pipes[1:]
+        # the same through the epoch loader a trainer would use (MiniBatchLoader): the consumer receives
+        # every batch narrowed to its sizes, which costs one host read-back per batch
+        if args.driver == "fused":
+            from apt_amd.loader import MiniBatchLoader
+            loader = MiniBatchLoader(graph, store, torch.cat(seed_sets), B, hops, in_flight=args.inflight,
+                                     shuffle=False, replace=args.replace, seed=args.seed, requests=requests)
+            it = iter(loader)
+            for _ in range(W):
+                next(it)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            loader_edges = sum(batch["num_edges"] for batch in it)
+            torch.cuda.synchronize()
+            t_ld = time.perf_counter() - t0
+            in_flight["loader"] = {"ms_per_step": t_ld / K * 1e3, "edges_per_s": loader_edges / t_ld}
+            del loader, it
     assert int(pipe.misses.item()) == 0 and int(stage_pipe.misses.item()) == 0
 
     # ---- optional aggregation stage on the outermost block of the last batch

@@ -1,0 +1,82 @@
+"""Epoch loader with mini-batches in flight: every batch equals what one
+pipeline builds alone from the same seeds and rng key (bit-exact), an epoch
+visits every index once, and buffers are not reused under the consumer."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(capi, n=30000, dim=32):
+    import torch
+
+    from apt_amd import synth
+    g = capi.Graph(*synth.rmat_csr_gpu(n, 12 * n, seed=9))
+    table = synth.random_features(n, dim, torch.float32, seed=4)
+    return g, capi.FeatStore(table), table
+
+
+@pytest.mark.parametrize("in_flight,drop_last,formats", [(1, True, False), (3, True, "csc"), (4, False, False),
+                                                         (8, False, True)])
+def test_loader_matches_single_pipeline(capi, in_flight, drop_last, formats):
+    import torch
+
+    from apt_amd.loader import MiniBatchLoader
+    from apt_amd.pipeline import MiniBatchPipeline
+    g, store, table = _setup(capi)
+    ids = torch.from_numpy(np.random.default_rng(0).choice(30000, 1100, replace=False)).cuda()
+    B, hops = 256, [3, 4]
+    loader = MiniBatchLoader(g, store, ids, B, hops, in_flight=in_flight, shuffle=True, drop_last=drop_last, seed=5,
+                             formats=formats)
+    assert len(loader) == (4 if drop_last else 5)
+    ref = {B: MiniBatchPipeline(g, store, B, hops)}
+    if not drop_last:
+        ref[1100 - 4 * B] = MiniBatchPipeline(g, store, 1100 - 4 * B, hops)
+    for epoch in range(2):
+        seen, kept = [], []
+        for i, batch in enumerate(loader):
+            seeds = batch["output_nodes"]
+            seen.append(seeds.cpu())
+            # consumer work on its own stream that reads the yielded buffers
+            kept.append((batch["features"].double().sum(), batch["input_nodes"].sum()))
+            pipe = ref[seeds.numel()]
+            pipe.run(seeds, (5 * 7919 + epoch) * len(loader) + i)
+            want = pipe.result()
+            assert torch.equal(batch["input_nodes"], want["input_nodes"])
+            assert torch.equal(batch["features"], want["features"])
+            assert torch.equal(batch["features"], table[want["input_nodes"]])
+            assert batch["num_edges"] == want["num_edges"]
+            for b, w in zip(batch["blocks"], want["blocks"]):
+                assert torch.equal(b["relabeled"], w["relabeled"]) and torch.equal(b["unique"], w["unique"])
+                if formats:
+                    assert b["formats"]["num_edges"] == int((w["relabeled"] >= 0).sum())
+            kept[-1] += (want["features"].double().sum(), want["input_nodes"].sum())
+        assert i + 1 == len(loader)
+        got = torch.cat(seen)
+        if drop_last:
+            assert got.numel() == 4 * B and len(set(got.tolist())) == 4 * B and set(got.tolist()) <= set(ids.tolist())
+        else:
+            assert sorted(got.tolist()) == sorted(ids.tolist())
+        for fs, ns, wf, wn in kept:                      # sums enqueued before the buffers were reused
+            assert float(fs) == float(wf) and int(ns) == int(wn)
+        if epoch == 0:
+            first = got
+    assert not torch.equal(first, got)                   # epochs are shuffled differently
+
+
+def test_loader_without_shuffle_and_early_exit(capi):
+    import torch
+
+    from apt_amd.loader import MiniBatchLoader
+    g, store, table = _setup(capi)
+    ids = torch.arange(100, 100 + 640).cuda()
+    loader = MiniBatchLoader(g, store, ids, 128, [5], in_flight=3, shuffle=False)
+    for i, batch in enumerate(loader):
+        assert torch.equal(batch["output_nodes"], ids[i * 128:(i + 1) * 128])
+        assert torch.equal(batch["input_nodes"][:128], batch["output_nodes"])
+        if i == 1:
+            break                                        # batches 2..4 are in flight; the next epoch starts over
+    out = [b["output_nodes"].clone() for b in loader]
+    assert torch.equal(torch.cat(out), ids)
+    with pytest.raises(ValueError):
+        MiniBatchLoader(g, store, ids[:10], 128, [5])
