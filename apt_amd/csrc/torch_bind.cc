@@ -233,7 +233,11 @@ std::tuple<Tensor, Tensor> SampleNeighbors(Tensor seeds, IdType fanout, bool rep
 // with neighbors / relabeled in the fixed-stride layout [rows_h * fanout_h], -1 = no edge.
 // The rank table and workspace live in the registry and are reused: calls must be
 // ordered on one stream.
-std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts, bool replace, IdType rng_seed) {
+// with_formats: each hop's block is also emitted as COO + CSC before that one wait;
+// appended per hop: coo_row_h, coo_col_h, csc_indptr_h (sizes then carries the hops'
+// edge counts after its H + 2 entries).
+std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts, bool replace, IdType rng_seed,
+                                 bool with_formats) {
   auto& s = S();
   TORCH_CHECK(s.has_graph, "npc: no graph registered (mix_cache_graphs)");
   const int H = static_cast<int>(hop_fanouts.size());
@@ -267,7 +271,7 @@ std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts,
     TORCH_CHECK(cap[h] > 0, "npc: sample_blocks: unsupported batch / fanouts");
   }
   auto nodes = torch::empty({cap[H]}, i64_opts());
-  auto sizes = torch::empty({H + 2}, i64_opts());
+  auto sizes = torch::zeros({H + 2 + (with_formats ? H : 0)}, i64_opts());
   std::vector<Tensor> nb(H), rl(H), ct(H);
   std::vector<int64_t*> nbp(H), rlp(H), ctp(H);
   for (int h = 0; h < H; ++h) {
@@ -285,6 +289,25 @@ std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts,
                                       static_cast<size_t>(s.mb_workspace.numel()), stream());
   if (rc != APT_OK) s.mb_workspace = Tensor();  // re-initialised by the next call
   check(rc);
+  std::vector<Tensor> row(H), col(H), csc(H);
+  if (with_formats) {
+    size_t need = 256;
+    for (int h = 0; h < H; ++h) {
+      const size_t b = apt_block_workspace_bytes(cap[h], fan[h], cap[h + 1], 0);
+      TORCH_CHECK(b > 0, "npc: sample_blocks: block sizes out of range");
+      need = std::max(need, b);
+    }
+    auto ws = torch::empty({static_cast<int64_t>(need)}, u8);   // the hops run one after the other
+    int64_t* dev_sizes = sizes.data_ptr<int64_t>();
+    for (int h = 0; h < H; ++h) {
+      row[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+      col[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+      csc[h] = torch::empty({cap[h] + 1}, i64_opts());
+      check(apt_block_formats(rlp[h], cap[h], dev_sizes + h, fan[h], cap[h + 1], row[h].data_ptr<int64_t>(),
+                              col[h].data_ptr<int64_t>(), csc[h].data_ptr<int64_t>(), dev_sizes + H + 2 + h, nullptr,
+                              nullptr, nullptr, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream()));
+    }
+  }
   auto host = sizes.cpu();  // the one wait of the batch
   const int64_t* hs = host.data_ptr<int64_t>();
   std::vector<Tensor> out{host, nodes.narrow(0, 0, hs[H])};
@@ -293,6 +316,12 @@ std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts,
     out.push_back(rl[h].narrow(0, 0, hs[h] * fan[h]));
     out.push_back(ct[h].narrow(0, 0, hs[h]));
   }
+  if (with_formats)
+    for (int h = 0; h < H; ++h) {
+      out.push_back(row[h].narrow(0, 0, hs[H + 2 + h]));
+      out.push_back(col[h].narrow(0, 0, hs[H + 2 + h]));
+      out.push_back(csc[h].narrow(0, 0, hs[h] + 1));
+    }
   return out;
 }
 

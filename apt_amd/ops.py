@@ -75,14 +75,23 @@ def sample_neighbors(seeds: torch.Tensor, fanout: int, replace: bool, rng_seed: 
     return _npc.sample_neighbors(seeds, fanout, replace, rng_seed, hop)
 
 
-def sample_blocks(seeds: torch.Tensor, hop_fanouts, replace: bool, rng_seed: int):
+def sample_blocks(seeds: torch.Tensor, hop_fanouts, replace: bool, rng_seed: int, formats: bool = False):
     """Every hop of a batch in one operator call (sample -> relabel -> next
     frontier; reference python/npc/sampler.py:187-203,358-364), one host wait.
-    hop_fanouts: from the seeds outward.
-    -> (sizes list[H + 2], input_nodes, [(neighbors, relabeled, counts) per hop])"""
-    out = _npc.sample_blocks(seeds, [int(f) for f in hop_fanouts], bool(replace), int(rng_seed))
-    hops = [tuple(out[2 + 3 * h:5 + 3 * h]) for h in range(len(hop_fanouts))]
-    return out[0].tolist(), out[1], hops
+    hop_fanouts: from the seeds outward.  formats: every hop's block also as
+    COO + CSC, emitted before that wait.
+    -> (sizes list[H + 2], input_nodes, [(neighbors, relabeled, counts) per hop])
+       (+ [dict(coo_row, coo_col, csc_indptr, num_edges) per hop] with formats)"""
+    H = len(hop_fanouts)
+    out = _npc.sample_blocks(seeds, [int(f) for f in hop_fanouts], bool(replace), int(rng_seed), bool(formats))
+    hops = [tuple(out[2 + 3 * h:5 + 3 * h]) for h in range(H)]
+    sizes = out[0].tolist()
+    if not formats:
+        return sizes, out[1], hops
+    base = 2 + 3 * H
+    fmts = [dict(coo_row=out[base + 3 * h], coo_col=out[base + 3 * h + 1], csc_indptr=out[base + 3 * h + 2],
+                 num_edges=sizes[H + 2 + h]) for h in range(H)]
+    return sizes[:H + 2], out[1], hops, fmts
 
 
 def block_formats(relabeled: torch.Tensor, num_dst: int, fanout: int, num_src: int, want_csr: bool = True):

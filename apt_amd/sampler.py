@@ -1,41 +1,49 @@
 """Multi-hop mini-batch driver, the DP branch of MixedPSNeighborSampler
 (reference python/npc/sampler.py:159-203,358-364) and create_dgl_block
-(:76-91), without DGL: a block is a plain record of COO tensors."""
-from dataclasses import dataclass, field
-from typing import Optional
-
+(:76-91), without DGL: a block is a plain record of tensors."""
 import torch
 
 from . import ops
 
 
-@dataclass
 class Block:
     """Bipartite block of one hop.  Edge e goes from source row[e] (index into
     src_ids) to destination col[e] (index into the hop's seeds); the first
     num_dst source ids are the destination ids (reference sampler.py:76-91).
     relabeled / fanout: the same edges in the sampler's fixed-stride layout
     (relabeled[d * fanout + k], -1 = no edge), which the block aggregations read
-    directly; csc() / csr() give DGL's other two formats on demand."""
-    row: torch.Tensor
-    col: torch.Tensor
-    num_src: int
-    num_dst: int
-    src_ids: torch.Tensor
-    relabeled: Optional[torch.Tensor] = None
-    fanout: int = 0
-    formats: Optional[dict] = field(default=None, repr=False)
+    directly.  row / col (COO), csc() and csr(), DGL's three formats, are derived
+    from it on first use: a forward pass over the fixed-stride layout never pays
+    for them."""
+
+    def __init__(self, num_src, num_dst, src_ids, relabeled, fanout, formats=None):
+        self.num_src, self.num_dst = int(num_src), int(num_dst)
+        self.src_ids = src_ids
+        self.relabeled = relabeled
+        self.fanout = int(fanout)
+        self.formats = formats
+
+    def __repr__(self):
+        return f"Block(num_src={self.num_src}, num_dst={self.num_dst}, fanout={self.fanout})"
 
     def _formats(self, want_csr):
         if self.formats is None or (want_csr and "csr_indptr" not in self.formats):
             self.formats = ops.block_formats(self.relabeled, self.num_dst, self.fanout, self.num_src, want_csr)
         return self.formats
 
+    @property
+    def row(self):
+        return self._formats(False)["coo_row"]
+
+    @property
+    def col(self):
+        return self._formats(False)["coo_col"]
+
     def csc(self):
         """-> (indptr over destinations, source per edge, edge ids): the arguments
         of the reference's create_block_from_csc (sampler.py:44-56)."""
         f = self._formats(False)
-        return f["csc_indptr"], f["coo_row"], torch.arange(f["num_edges"], device=self.row.device)
+        return f["csc_indptr"], f["coo_row"], torch.arange(f["num_edges"], device=self.relabeled.device)
 
     def csr(self):
         """-> (indptr over sources, destination per edge, edge ids)."""
@@ -56,9 +64,8 @@ def create_block(seeds, neighbors, fanout):
     return _block(seeds.numel(), unique, relabeled, fanout)
 
 
-def _block(num_dst, unique, relabeled, fanout):
-    f = ops.block_formats(relabeled, num_dst, fanout, unique.numel(), False)
-    return Block(f["coo_row"], f["coo_col"], unique.numel(), num_dst, unique, relabeled, fanout, f)
+def _block(num_dst, unique, relabeled, fanout, f=None):
+    return Block(unique.numel(), num_dst, unique, relabeled, fanout, f)
 
 
 class MixedPSNeighborSampler:
@@ -67,7 +74,7 @@ class MixedPSNeighborSampler:
     sampled with the last entry."""
 
     def __init__(self, rank, world_size, fanouts, system="DP", model=None, num_total_nodes=None,
-                 shuffle_with_dst=False, debug_info=None, replace=True, rng_seed=None, fused=True):
+                 shuffle_with_dst=False, debug_info=None, replace=True, rng_seed=None, fused=True, formats=False):
         if system != "DP":
             raise NotImplementedError(f"system {system!r} needs other GPUs; only 'DP' is available")
         self.rank, self.world_size = rank, world_size
@@ -77,6 +84,7 @@ class MixedPSNeighborSampler:
         self.replace = replace
         self.rng_seed = rng_seed
         self.fused = fused
+        self.formats = bool(formats)      # fused: COO + CSC of every block inside the one call, else on first use
         self.batches = 0
 
     def sample(self, graph, seeds):
@@ -89,9 +97,11 @@ class MixedPSNeighborSampler:
         if self.fused and (self.rng_seed is not None or not self.replace):
             seed = (self.rng_seed if self.rng_seed is not None else 0) + self.batches
             fan = list(reversed(self.fanouts))
-            sizes, nodes, hops = ops.sample_blocks(seeds, fan, self.replace, seed)
+            out = ops.sample_blocks(seeds, fan, self.replace, seed, formats=self.formats)
+            sizes, nodes, hops = out[:3]
             for h, (_, relabeled, _) in enumerate(hops):
-                blocks.insert(0, _block(sizes[h], nodes[:sizes[h + 1]], relabeled, fan[h]))
+                blocks.insert(0, _block(sizes[h], nodes[:sizes[h + 1]], relabeled, fan[h],
+                                        out[3][h] if self.formats else None))
             self.batches += 1
             return (nodes, output_nodes, blocks)
         for layer_id, fanout in enumerate(reversed(self.fanouts)):

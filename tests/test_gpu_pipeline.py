@@ -334,6 +334,13 @@ def test_operator_layer_fused_sampler(orc, capi):
     assert sizes[:2] == [50, len(want_in)] and np.array_equal(nodes.cpu().numpy(), want_in)
     assert np.array_equal(hops[0][0].cpu().numpy(), want_blocks[0]["neighbors"])
     assert np.array_equal(hops[0][2].cpu().numpy(), want_blocks[0]["counts"])
+    # the same call with the blocks' COO + CSC emitted before its one wait
+    sizes_f, nodes_f, hops_f, fmts = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9, formats=True)
+    assert sizes_f == sizes and torch.equal(nodes_f, nodes) and torch.equal(hops_f[0][1], hops[0][1])
+    alone = npc.ops.block_formats(hops[0][1], 50, 4, nodes.numel(), False)
+    assert fmts[0]["num_edges"] == alone["num_edges"] == int((hops[0][1] >= 0).sum())
+    for k in ("coo_row", "coo_col", "csc_indptr"):
+        assert torch.equal(fmts[0][k], alone[k]), k
     indptr2, indices2, _ = _setup(orc, capi, n=300, dim=4, seed=9)
     npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr2), torch.from_numpy(indices2))
     sizes, nodes, hops = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9)
