@@ -73,6 +73,8 @@ SYMBOLS = {
     "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
     "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
     "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
+    "apt_spmm_csr_workspace_bytes": (C.c_size_t, [_I64]),
+    "apt_spmm_csr": (_I, [_P, _P, _P, _I64, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P, _P, C.c_size_t, _P]),
     "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
@@ -567,6 +569,8 @@ def block_formats(relabeled, num_dst, fanout, num_src, want_csr=True, num_dst_de
 
 
 def _f32(t, name):
+    if t is None:
+        return None
     if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float32):
         raise TypeError(f"{name} must be a contiguous fp32 GPU tensor")
     return t
@@ -643,6 +647,39 @@ def gat_block_backward(neighbors, num_dst, fanout, ft, el, er, negative_slope, a
                                        _ptr(_f32(d_out, "d_out")), _ptr(_dev_i64(csc_indptr, "csc_indptr")),
                                        _ptr(a_edge), _ptr(dz_edge), _ptr(d_er), _stream()))
     return a_edge, dz_edge, d_er
+
+
+def spmm_csr(indptr, indices, x, eids=None, col_scale=None, head_weights=None, head_weights2=None):
+    """out[r] = sum over the edges e of CSR row r of col_scale[indices[e]] * head_weights[w(e), h] * x[indices[e]],
+    w(e) = eids[e] or e.  x [n, dim] or [n, heads, head_dim] -> fp32 of the same trailing shape with
+    len(indptr) - 1 rows, every row written once (no zero-fill, no atomics).  With head_weights2 also returns
+    out2[r, h] = sum of head_weights2[w(e), h]."""
+    indptr, indices = _dev_i64(indptr, "indptr"), _dev_i64(indices, "indices")
+    eids = _dev_i64(eids, "eids")
+    if x.dim() == 3:
+        n, heads, hd = x.shape
+    else:
+        x = _feat2d(x, "x")
+        (n, hd), heads = x.shape, 1
+    if not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
+        raise AptError("spmm_csr: x must be a contiguous fp32 or bf16 tensor")
+    rows, edges = indptr.numel() - 1, indices.numel()
+    if eids is not None and eids.numel() != edges:
+        raise AptError("spmm_csr: eids must have one entry per edge")
+    col_scale = _f32(col_scale, "col_scale")
+    head_weights, head_weights2 = _f32(head_weights, "head_weights"), _f32(head_weights2, "head_weights2")
+    for w in (head_weights, head_weights2):
+        if w is not None and (w.dim() != 2 or w.shape[1] != heads):
+            raise AptError("spmm_csr: head weights must be [*, heads]")
+    if col_scale is not None and col_scale.numel() != n:
+        raise AptError("spmm_csr: col_scale must have one entry per row of x")
+    out = torch.empty((rows,) + tuple(x.shape[1:]), dtype=torch.float32, device=x.device)
+    out2 = torch.empty((rows, heads), dtype=torch.float32, device=x.device) if head_weights2 is not None else None
+    ws = torch.empty(int(lib().apt_spmm_csr_workspace_bytes(edges)), dtype=torch.uint8, device=x.device)
+    check(lib().apt_spmm_csr(_ptr(indptr), _ptr(indices), _ptr(eids), rows, edges, _ptr(x), n, heads * hd,
+                             x.element_size(), _ptr(col_scale), _ptr(head_weights), _ptr(head_weights2), heads,
+                             _ptr(out), _ptr(out2), _ptr(ws), ws.numel(), _stream()))
+    return out if out2 is None else (out, out2)
 
 
 def spmm_heads(row, col, x, head_weights, num_out, weight_row=None, grouped=False, head_weights2=None):

@@ -27,14 +27,13 @@ class BlockAggregate(torch.autograd.Function):
     def backward(ctx, dZ):
         block = ctx.block
         dZ = dZ.contiguous()
+        scale = None
         if ctx.mean:
             indptr = block.csc()[0]
-            cnt = (indptr[1:] - indptr[:-1]).clamp(min=1).to(dZ.dtype)
-            dZ = dZ / cnt[:, None]
-        _, dst, eids = block.csr()                     # edges grouped by source, by increasing edge id
-        src = block.row[eids]
-        dX = capi.spmm_sum(0, dst, src, dZ, block.num_src)
-        return None, dX, None
+            scale = 1.0 / (indptr[1:] - indptr[:-1]).clamp(min=1).to(torch.float32)
+        indptr, dst, _ = block.csr()                   # edges grouped by source, by increasing edge id
+        dX = capi.spmm_csr(indptr, dst, dZ, col_scale=scale)    # every source row written once, in edge order
+        return None, dX.to(dZ.dtype), None
 
 
 class SAGEConv(nn.Module):
@@ -116,7 +115,10 @@ class GATAggregate(torch.autograd.Function):
         E = eids.numel()
         a_edge, dz_edge, d_er = capi.gat_block_backward(block.relabeled, block.num_dst, block.fanout, ft, el, er,
                                                         ctx.slope, attn, d_out, csc_indptr, E)
-        src = block.row[eids]                                   # edges grouped by source
+        # sums over the edges of a source, in the block's CSR order; the per-edge weights stay in COO order.
+        # (capi.spmm_csr computes the same without a zero-fill, but its extra per-edge loads make it the
+        # slower of the two here.)
+        src = block.row[eids]
         d_ft, d_el = capi.spmm_heads(dst, src, d_out, a_edge, block.num_src, weight_row=eids, grouped=True,
                                      head_weights2=dz_edge)
         return None, d_ft.to(ft.dtype), d_el, d_er, None

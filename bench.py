@@ -378,22 +378,30 @@ def main():
             fmt_b = capi.block_formats(rel, n_dst, f, n_src)
             _, attn_w = capi.gat_block(rel, n_dst, f, ft, el, er, 0.2, want_attn=True)
             d_out = torch.randn(n_dst, heads, hdim, device=dev)
+            csr_ip = fmt_b["csr_indptr"][:n_src + 1].contiguous()
             src_csr = fmt_b["coo_row"][fmt_b["csr_eids"]].contiguous()
+            d2 = d_out.view(n_dst, heads * hdim)
 
             def gat_bwd():
                 a_e, dz_e, d_er = capi.gat_block_backward(rel, n_dst, f, ft, el, er, 0.2, attn_w, d_out,
                                                           fmt_b["csc_indptr"], fmt_b["num_edges"])
                 capi.spmm_heads(fmt_b["csr_indices"], src_csr, d_out, a_e, n_src, weight_row=fmt_b["csr_eids"],
                                 grouped=True, head_weights2=dz_e)
-            for _ in range(3):
-                gat_bwd()
-            e0, e1 = ev(), ev()
-            e0.record()
-            for _ in range(10):
-                gat_bwd()
-            e1.record()
-            torch.cuda.synchronize()
-            agg[f"gat_block_backward_{name}_us"] = e0.elapsed_time(e1) / 10 * 1e3
+
+            # backward of the plain sum / mean (SAGE, GCN): one row-owned pass over the CSR order
+            for tag, fn in (("gat_block_backward", gat_bwd),
+                            ("spmm_block_backward", lambda: capi.spmm_csr(csr_ip, fmt_b["csr_indices"], d2))):
+                if tag == "spmm_block_backward" and name != "fp32":
+                    continue
+                for _ in range(3):
+                    fn()
+                e0, e1 = ev(), ev()
+                e0.record()
+                for _ in range(10):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                agg[f"{tag}_{name}_us"] = e0.elapsed_time(e1) / 10 * 1e3
             del ft, el, er, fmt_b, attn_w, d_out
         hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
         h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)

@@ -30,6 +30,8 @@
  *   orc_map_to_vir, orc_vir_send_offset   numpy searchsorted closed forms.
  *   orc_block_formats   numpy nonzero / stable argsort / bincount + cumsum.
  *   orc_count_ids, orc_csr_select_rows   numpy bincount / concatenated slices.
+ *   orc_spmm_csr        scipy.sparse CSR matrix x dense product (float64), per head
+ *                       with the edge weights as the matrix data; empty rows are zero.
  *   orc_spmm_sum/sddmm  numpy closed forms (np.add.at over fancy-indexed rows,
  *                       in float64); a sum over a row of ones equals its
  *                       in-degree.
@@ -524,6 +526,40 @@ void orc_spmm_sum(int mode, const int64_t* row, const int64_t* col, int64_t E, c
   }
   for (int64_t i = 0; i < num_out * dim; ++i) out[i] = (float)acc[i];
   free(acc);
+}
+
+/* Row-owned SpMM over CSR, the backward direction of a block (the reference runs
+ * its COO operator with the edges reversed, python/npc/model/sageconv.py:100-114):
+ * out[r] = sum_e col_scale[idx[e]] * w[weid(e), head] * x[idx[e]], float64 accumulation. */
+void orc_spmm_csr(const int64_t* indptr, const int64_t* indices, const int64_t* eids, int64_t num_rows,
+                  const float* x, int64_t num_x_rows, int64_t dim, const float* col_scale, const float* w,
+                  const float* w2, int heads, float* out, float* out2) {
+  const int64_t hd = dim / heads;
+#pragma omp parallel for schedule(dynamic, 256) num_threads(g_threads)
+  for (int64_t r = 0; r < num_rows; ++r) {
+    for (int64_t d = 0; d < dim; ++d) {
+      double acc = 0.0;
+      for (int64_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+        const int64_t j = indices[e];
+        if (j < 0 || j >= num_x_rows) continue;
+        const int64_t we = eids ? eids[e] : e;
+        double f = col_scale ? (double)col_scale[j] : 1.0;
+        if (w) f *= (double)w[we * heads + d / hd];
+        acc += f * (double)x[j * dim + d];
+      }
+      out[r * dim + d] = (float)acc;
+    }
+    if (w2)
+      for (int h = 0; h < heads; ++h) {
+        double acc = 0.0;
+        for (int64_t e = indptr[r]; e < indptr[r + 1]; ++e) {
+          const int64_t j = indices[e];
+          if (j < 0 || j >= num_x_rows) continue;
+          acc += (double)w2[(eids ? eids[e] : e) * heads + h];
+        }
+        out2[r * heads + h] = (float)acc;
+      }
+  }
 }
 
 void orc_sddmm(int op, const int64_t* row, const int64_t* col, int64_t E, const float* lhs,

@@ -16,7 +16,7 @@ __all__ = [
     "build", "lib", "philox4x32_10", "draw64", "bounded", "Graph", "FeatStore",
     "sample_neighbors", "sample_positions", "relabel", "gather_rows",
     "permute_rows", "scatter_rows", "cluster_permute", "cluster_reqs",
-    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "sddmm", "count_ids", "csr_select_rows", "block_formats", "gat_scores", "gat_block", "map_to_vir", "vir_send_offset",
+    "set_threads", "max_threads", "sample_blocks", "spmm_sum", "spmm_csr", "sddmm", "count_ids", "csr_select_rows", "block_formats", "gat_scores", "gat_block", "map_to_vir", "vir_send_offset",
 ]
 
 
@@ -277,6 +277,22 @@ def spmm_sum(mode, row, col, x, num_out, edata=None, coo_offset=None, input_offs
     lib().orc_spmm_sum(C.c_int(mode), _p(row), _p(col), C.c_int64(E), _p(x), _p(ed), C.c_int64(dim),
                        _p(coo), _p(io), _p(oo), C.c_int(nseg), _p(out), C.c_int64(num_out))
     return out
+
+
+def spmm_csr(indptr, indices, x, eids=None, col_scale=None, head_weights=None, head_weights2=None, heads=1):
+    """out[r] = sum over CSR row r's edges of col_scale[idx] * head_weights[w(e), h] * x[idx]
+    -> float32 [rows, dim] (and [rows, heads] with head_weights2); x is [n, dim], dim = heads * head_dim."""
+    indptr, indices, x = _i64(indptr), _i64(indices), _f32(x)
+    rows, dim = len(indptr) - 1, x.shape[1]
+    ei = None if eids is None else _i64(eids)
+    cs = None if col_scale is None else _f32(col_scale)
+    w = None if head_weights is None else _f32(head_weights)
+    w2 = None if head_weights2 is None else _f32(head_weights2)
+    out = np.zeros((rows, dim), dtype=np.float32)
+    out2 = None if w2 is None else np.zeros((rows, heads), dtype=np.float32)
+    lib().orc_spmm_csr(_p(indptr), _p(indices), _p(ei), C.c_int64(rows), _p(x), C.c_int64(x.shape[0]),
+                       C.c_int64(dim), _p(cs), _p(w), _p(w2), C.c_int(heads), _p(out), _p(out2))
+    return out if out2 is None else (out, out2)
 
 
 def sddmm(op, row, col, lhs, rhs, coo_offset=None, lhs_offset=None, rhs_offset=None):

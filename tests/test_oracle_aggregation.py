@@ -112,3 +112,38 @@ def test_gat_scores_and_block_pins(orc):
     a = orc.gat_block(nbr, n_dst, fanout, ft, neg_l, neg_r, 0.2)
     b = orc.gat_block(nbr, n_dst, fanout, ft, (0.2 * neg_l).astype(np.float32), (0.2 * neg_r).astype(np.float32), 1.0)
     assert np.allclose(a, b, rtol=1e-5, atol=1e-6)
+
+
+def test_spmm_csr_is_the_sparse_matrix_product(orc):
+    """Row-owned SpMM over CSR = scipy's CSR matrix times the dense features, per
+    head with the edge weights as the matrix data (float64); rows without edges are
+    zero; the second sum is the matrix times a column of ones."""
+    import scipy.sparse as sp
+    rng = np.random.default_rng(5)
+    rows, n_x, heads, hd = 400, 150, 3, 8
+    deg = rng.integers(0, 6, rows)
+    deg[7] = 700                                              # a hub row
+    deg[11] = 0
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    E = int(indptr[-1])
+    indices = rng.integers(0, n_x, E)
+    eids = rng.permutation(E)
+    x = rng.standard_normal((n_x, heads * hd)).astype(np.float32)
+    scale = rng.random(n_x).astype(np.float32) + 0.5
+    w = rng.standard_normal((E, heads)).astype(np.float32)
+    w2 = rng.standard_normal((E, heads)).astype(np.float32)
+    # plain sum
+    A = sp.csr_matrix((np.ones(E), indices, indptr), shape=(rows, n_x))
+    got = orc.spmm_csr(indptr, indices, x)
+    assert np.allclose(got, A @ x.astype(np.float64), rtol=1e-6, atol=1e-6) and not got[11].any()
+    # scaled columns (the mean's backward)
+    got = orc.spmm_csr(indptr, indices, x, col_scale=scale)
+    assert np.allclose(got, A @ (x.astype(np.float64) * scale[:, None]), rtol=1e-6, atol=1e-6)
+    # per-head edge weights addressed through edge ids, and the second sum
+    got, got2 = orc.spmm_csr(indptr, indices, x, eids=eids, head_weights=w, head_weights2=w2, heads=heads)
+    for h in range(heads):
+        Ah = sp.csr_matrix((w[eids, h].astype(np.float64), indices, indptr), shape=(rows, n_x))
+        assert np.allclose(got[:, h * hd:(h + 1) * hd], Ah @ x[:, h * hd:(h + 1) * hd].astype(np.float64),
+                           rtol=1e-5, atol=1e-5)
+        want2 = np.add.reduceat(np.concatenate([w2[eids, h].astype(np.float64), [0.0]]), indptr[:-1]) * (deg > 0)
+        assert np.allclose(got2[:, h], want2, rtol=1e-5, atol=1e-5)
