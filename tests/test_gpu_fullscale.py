@@ -167,5 +167,25 @@ def test_full_scale_properties(capi, replace):
         b = capi.sample_neighbors(cached_graph, frontier, 15, False, 99, 2)
         assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
         del pos, c_indptr, c_indices
+        # an epoch of 1300 batches through the loader, two in flight: each pipeline's rank table runs out of
+        # epochs once on the way (511 per fill at this plan's id width) and is refilled; every 40th batch is
+        # rebuilt afterwards by a lone pipeline from the same seeds and key and must match bit for bit
+        from apt_amd.loader import MiniBatchLoader
+        ids = torch.randperm(N, generator=gen, device=DEV)[:1300 * 4096].contiguous()
+        loader = MiniBatchLoader(graph, store, ids, 4096, hops, in_flight=2, shuffle=False, seed=3)
+        kept, edges = {}, 0
+        for i, batch in enumerate(loader):
+            edges += batch["num_edges"]
+            if i % 40 == 0:
+                kept[i] = (batch["input_nodes"].clone(), batch["features"].view(torch.int16).clone(),
+                           batch["blocks"][0]["relabeled"].clone())
+        assert i == 1299 and edges > 1300 * 1_000_000
+        for i, (nodes_i, feats_i, rel_i) in kept.items():
+            pipe.run(ids[i * 4096:(i + 1) * 4096], 3 * 7919 * 1300 + i)
+            want = pipe.result()
+            assert torch.equal(want["input_nodes"], nodes_i), i
+            assert torch.equal(want["features"].view(torch.int16), feats_i), i
+            assert torch.equal(want["blocks"][0]["relabeled"], rel_i), i
+        del loader, kept
     del pipe, feats, indices, indptr
     torch.cuda.empty_cache()
