@@ -67,7 +67,8 @@ SYMBOLS = {
     "apt_vir_send_offset": (_I, [_I, _I64, _P, _I64, _P, _I64, _I, _P, _P]),
     "apt_block_workspace_bytes": (_SZ, [_I64, _I, _I64, _I]),
     "apt_block_formats": (_I, [_P, _I64, _P, _I, _I64, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
-    "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P]),
+    "apt_spmm_sum": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I, _P, _P, _P, _I, _P, _I64, _P, _P]),
+    "apt_coo_is_grouped": (_I, [_P, _I64, _P, _P]),
     "apt_spmm_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I64, _I, _I, _P, _P]),
     "apt_sddmm": (_I, [_I, _P, _P, _I64, _P, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P]),
     "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
@@ -435,8 +436,10 @@ def _segments(coo_offset, num_edges, device):
 
 
 def spmm_sum(mode, row, col, x, num_out, edata=None, coo_offset=None, input_offset=None,
-             output_offset=None):
-    """mode 0 copy_u, 1 copy_e, 2 u_mul_e -> fp32 [num_out, dim] (see apt_spmm_sum)."""
+             output_offset=None, detect_grouped=True):
+    """mode 0 copy_u, 1 copy_e, 2 u_mul_e -> fp32 [num_out, dim] (see apt_spmm_sum).
+    detect_grouped: check on the device whether col is non-decreasing and, if so, skip the atomics for
+    rows inside a wavefront's edges."""
     row, col, x = _dev_i64(row, "row"), _dev_i64(col, "col"), _feat2d(x, "input")
     if edata is not None:
         edata = _feat2d(edata, "edata")
@@ -448,10 +451,14 @@ def spmm_sum(mode, row, col, x, num_out, edata=None, coo_offset=None, input_offs
         raise AptError("spmm_sum: row and col differ in length")
     coo = _segments(coo_offset, row.numel(), x.device)
     out = torch.zeros((num_out, x.shape[1]), dtype=torch.float32, device=x.device)
+    grouped = None
+    if detect_grouped:
+        grouped = torch.empty(1, dtype=torch.int32, device=x.device)
+        check(lib().apt_coo_is_grouped(_ptr(col), col.numel(), _ptr(grouped), _stream()))
     check(lib().apt_spmm_sum(int(mode), _ptr(row), _ptr(col), row.numel(), _ptr(x), x.shape[0], _ptr(edata),
                              x.shape[1], x.element_size(), _ptr(coo), _ptr(_dev_i64(input_offset, "input_offset")),
                              _ptr(_dev_i64(output_offset, "output_offset")), coo.numel() - 1, _ptr(out),
-                             int(num_out), _stream()))
+                             int(num_out), _ptr(grouped), _stream()))
     return out
 
 

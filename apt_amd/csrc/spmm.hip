@@ -41,6 +41,7 @@ struct AggParams {
   int heads;
   int64_t head_dim;         // dim / heads
   int grouped;              // edges with equal col are consecutive: rows inside a wavefront's range are stored, not added
+  const int* grouped_dev;   // the same as a device flag (apt_coo_is_grouped), or NULL
 };
 
 template <typename T> __device__ __forceinline__ float to_float(T v);
@@ -107,12 +108,13 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     int64_t cur = -1;
     bool first_row = true;  // the row at the start of the range may have begun in the previous wavefront's range
+    const bool grouped = p.grouped || (p.grouped_dev != nullptr && *p.grouped_dev != 0);
     // MODE 3: the lane holding a head's first features also sums the second weight table
     const bool second = MODE == 3 && p.head_w2 != nullptr && live && d % p.head_dim == 0;
     float acc2 = 0.f;
     auto flush = [&](bool last_row) {
       if (cur >= 0 && cur < p.num_out_rows && live) {
-        if (p.grouped && !first_row && !last_row) {
+        if (grouped && !first_row && !last_row) {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) p.out[cur * p.dim + d + i] = acc[i];
           if (second) p.out2[cur * p.heads + d / p.head_dim] = acc2;
@@ -179,6 +181,18 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
     }
     flush(true);
   }
+}
+
+// flag = 1 iff col is non-decreasing (then edges with equal col are consecutive).
+__global__ void coo_grouped_init_kernel(int* flag) { *flag = 1; }
+
+__global__ __launch_bounds__(kAggBlock) void coo_grouped_check_kernel(const int64_t* __restrict__ col, int64_t n,
+                                                                      int* flag) {
+  bool bad = false;
+  for (int64_t e = static_cast<int64_t>(blockIdx.x) * kAggBlock + threadIdx.x; e + 1 < n;
+       e += static_cast<int64_t>(gridDim.x) * kAggBlock)
+    bad |= col[e] > col[e + 1];
+  if (bad) *flag = 0;
 }
 
 // OP 0: lhs[src] + rhs[dst]; OP 1: lhs[src] * rhs[dst]  -> out[e]
@@ -909,7 +923,7 @@ extern "C" int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo
                             const void* input, int64_t num_in_rows, const void* edata, int64_t dim,
                             int elem_size, const int64_t* coo_offset, const int64_t* input_offset,
                             const int64_t* output_offset, int num_segments, float* out,
-                            int64_t num_out_rows, void* stream) {
+                            int64_t num_out_rows, const int* grouped_dev, void* stream) {
   using namespace apt;
   APT_REQUIRE(mode >= 0 && mode <= 2, APT_EINVAL, "apt_spmm_sum: mode %d (0 copy_u, 1 copy_e, 2 u_mul_e)", mode);
   int rc = agg_check("apt_spmm_sum", coo_row, coo_col, num_edges, input, out, coo_offset, num_segments, dim,
@@ -922,6 +936,8 @@ extern "C" int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo
   p.row = coo_row; p.col = coo_col; p.num_edges = num_edges; p.in = input; p.edata = edata; p.out = out;
   p.coo_off = coo_offset; p.in_off = input_offset; p.out_off = output_offset; p.num_seg = num_segments;
   p.dim = dim; p.num_in_rows = num_in_rows; p.num_e_rows = num_edges; p.num_out_rows = num_out_rows;
+  // with several segments two segments may share output rows, so the flag only counts for plain COO
+  p.grouped_dev = num_segments == 1 ? grouped_dev : nullptr;
   const int64_t waves = ceil_div(num_edges, kEdgesPerWave);
   const dim3 grid(static_cast<unsigned>(ceil_div(waves, kAggWaves))), block(kAggBlock);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -941,6 +957,20 @@ extern "C" int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo
   }
 #undef APT_SPMM_LAUNCH
   APT_LAUNCH_CHECK("spmm_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_coo_is_grouped(const int64_t* coo_col, int64_t num_edges, int* flag, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_edges >= 0 && flag != nullptr && (coo_col != nullptr || num_edges == 0), APT_EINVAL,
+              "apt_coo_is_grouped: bad arguments");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(coo_grouped_init_kernel, dim3(1), dim3(1), 0, st, flag);
+  if (num_edges > 1) {
+    const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_edges, kAggBlock), 4096));
+    hipLaunchKernelGGL(coo_grouped_check_kernel, dim3(blocks), dim3(kAggBlock), 0, st, coo_col, num_edges, flag);
+  }
+  APT_LAUNCH_CHECK("coo_grouped_check_kernel");
   return APT_OK;
 }
 

@@ -551,10 +551,13 @@ Tensor spmm(int mode, Tensor coo_row, Tensor coo_col, Tensor input, const Tensor
   }
   if (mode == 1) TORCH_CHECK(x.size(0) == row.numel(), "npc: spmm_copy_e_sum needs one input row per edge");
   auto out = torch::zeros({out_num, x.size(1)}, x.options().dtype(torch::kFloat32));
+  // a block's COO is destination-major: found out on the device, rows inside a wavefront's edges skip the atomics
+  auto grouped = torch::empty({1}, torch::TensorOptions().dtype(torch::kInt32).device(device()));
+  check(apt_coo_is_grouped(i64(col), col.numel(), grouped.data_ptr<int>(), stream()));
   check(apt_spmm_sum(mode, i64(row), i64(col), row.numel(), x.data_ptr(), x.size(0),
                      edata ? ed.data_ptr() : nullptr, x.size(1), static_cast<int>(x.element_size()),
                      i64(coo), input_offset ? i64(io) : nullptr, i64(oo), nseg, out.data_ptr<float>(),
-                     out_num, stream()));
+                     out_num, grouped.data_ptr<int>(), stream()));
   return out.to(x.scalar_type());
 }
 

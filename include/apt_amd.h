@@ -381,7 +381,13 @@ int apt_block_formats(const int64_t* relabeled, int64_t num_dst, const int64_t* 
  *                 (the reference's u_mul_e kernel adds instead of multiplying,
  *                 src/cuda/spmm.cu:78, and has no caller; the product is
  *                 implemented).  `out` is fp32 [num_out_rows, dim] and must be
- *                 zero on entry.
+ *                 zero on entry.  grouped_dev, optional (NULL = unknown): device
+ *                 flag written by apt_coo_is_grouped; when it is set (and there
+ *                 is one segment) every row that lies inside a wavefront's 64
+ *                 edges is stored instead of added atomically, which is what a
+ *                 sampled block's destination-major COO gets.
+ *   apt_coo_is_grouped  *flag = 1 iff col is non-decreasing (edges with equal col
+ *                 are then consecutive), else 0; flag is a device int.
  *   apt_sddmm     out[e, :] = lhs[lhs_offset[k] + row[e], :] (+|*) rhs[rhs_offset[k] + col[e], :]
  *                 op 0 = u_add_v, 1 = u_mul_v; out is fp32 [num_edges, dim].
  * elem_size 4 = fp32 inputs (the reference), 2 = bf16 inputs; accumulation and
@@ -392,7 +398,8 @@ int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo_col, int64
                  const void* input, int64_t num_in_rows, const void* edata, int64_t dim,
                  int elem_size, const int64_t* coo_offset, const int64_t* input_offset,
                  const int64_t* output_offset, int num_segments, float* out,
-                 int64_t num_out_rows, void* stream);
+                 int64_t num_out_rows, const int* grouped_dev, void* stream);
+int apt_coo_is_grouped(const int64_t* coo_col, int64_t num_edges, int* flag, void* stream);
 /* SpMM over a sampled block in the layout the sampler and relabel emit
  * (apt_sample_neighbors / apt_relabel / apt_minibatch_sample): destination i
  * owns slots [i * fanout, (i+1) * fanout) of `neighbors` (compact source ids,

@@ -210,3 +210,32 @@ def test_spmm_csr_rows_written_once(orc, capi, heads, hd, dtype):
     assert empty.shape == (4, heads, hd) and not empty.any()
     with pytest.raises(capi.AptError):
         capi.spmm_csr(dev(indptr), dev(indices), xt, eids=dev(eids[:-1]))
+
+
+def test_spmm_grouped_detection(orc, capi):
+    """apt_coo_is_grouped: 1 for a destination-major COO, 0 once two edges are out of
+    order; with the flag the sum skips the atomics inside a wavefront's edges and
+    gives the oracle's result either way (and the same bits on every call when grouped)."""
+    import ctypes
+    rng = np.random.default_rng(31)
+    row, col = _block(rng, 4000, 9, 9000)
+    x = rng.standard_normal((9000, 96)).astype(np.float32)
+    flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for swap, want in ((False, 1), (True, 0)):
+        c = col.copy()
+        if swap:
+            c[[10, 20000]] = c[[20000, 10]]
+        assert capi.lib().apt_coo_is_grouped(ctypes.c_void_p(dev(c).data_ptr()), len(c),
+                                             ctypes.c_void_p(flag.data_ptr()), stream) == 0
+        assert int(flag.item()) == want
+        want_out = orc.spmm_sum(0, row, c, x, 4000)
+        a = capi.spmm_sum(0, dev(row), dev(c), dev(x), 4000)
+        b = capi.spmm_sum(0, dev(row), dev(c), dev(x), 4000, detect_grouped=False)
+        assert _close(a.cpu().numpy(), want_out, 1e-5) and _close(b.cpu().numpy(), want_out, 1e-5)
+        if not swap:
+            assert torch.equal(a, capi.spmm_sum(0, dev(row), dev(c), dev(x), 4000))
+    for n in (0, 1):                                         # nothing to compare: grouped
+        assert capi.lib().apt_coo_is_grouped(ctypes.c_void_p(dev(col).data_ptr()), n,
+                                             ctypes.c_void_p(flag.data_ptr()), stream) == 0
+        assert int(flag.item()) == 1
