@@ -82,6 +82,13 @@ __device__ __forceinline__ void load_vec(const T* base, int64_t elem, float (&v)
 // MODE 3: acc += in[in_off + src] * head_w[e, head of the feature] (VEC divides head_dim)
 // A lane owns VEC consecutive features; kUnroll edges are loaded before they
 // are accumulated.
+// Value of a 64-bit variable in lane `src` of the wavefront (src is the same in all lanes).
+__device__ __forceinline__ int64_t wave_read(int64_t v, int src) {
+  const int lo = __builtin_amdgcn_readlane(static_cast<int>(v), src);
+  const int hi = __builtin_amdgcn_readlane(static_cast<int>(v >> 32), src);
+  return (static_cast<int64_t>(hi) << 32) | static_cast<uint32_t>(lo);
+}
+
 template <typename T, int MODE, int VEC>
 __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
   constexpr int kUnroll = 4;
@@ -97,67 +104,79 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
   const int64_t wave = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave;
   const int64_t e0 = wave * kEdgesPerWave;
   if (e0 >= p.num_edges) return;
-  const int64_t e1 = min(e0 + kEdgesPerWave, p.num_edges);
+  const int n = static_cast<int>(min(static_cast<int64_t>(kEdgesPerWave), p.num_edges - e0));
   const T* in = static_cast<const T*>(p.in);
   const T* ed = static_cast<const T*>(p.edata);
+  // Lane i fetches what edge e0 + i needs (its rows, and where its weights are): three coalesced loads
+  // for the wavefront's 64 edges; the edge loop below reads them lane by lane.
+  int64_t my_dst = -1, my_src = -1, my_we = 0;
+  if (lane < n) {
+    const int64_t e = e0 + lane;
+    const int k = segment_of(s_off, p.num_seg, e);
+    my_dst = s_out[k] + p.col[e];
+    if (MODE != 1) {
+      my_src = s_in[k] + p.row[e];
+      if (my_src >= p.num_in_rows) my_src = -1;
+    }
+    if (MODE == 3) my_we = p.head_w_row != nullptr ? p.head_w_row[e] : e;
+  }
+  const bool grouped = p.grouped || (p.grouped_dev != nullptr && *p.grouped_dev != 0);
   for (int64_t d0 = 0; d0 < p.dim; d0 += kWave * VEC) {
     const int64_t d = d0 + static_cast<int64_t>(lane) * VEC;
     const bool live = d < p.dim;
+    const int64_t h = MODE == 3 ? d / p.head_dim : 0;
     float acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
     int64_t cur = -1;
     bool first_row = true;  // the row at the start of the range may have begun in the previous wavefront's range
-    const bool grouped = p.grouped || (p.grouped_dev != nullptr && *p.grouped_dev != 0);
     // MODE 3: the lane holding a head's first features also sums the second weight table
-    const bool second = MODE == 3 && p.head_w2 != nullptr && live && d % p.head_dim == 0;
+    const bool second = MODE == 3 && p.head_w2 != nullptr && live && d == h * p.head_dim;
     float acc2 = 0.f;
     auto flush = [&](bool last_row) {
       if (cur >= 0 && cur < p.num_out_rows && live) {
         if (grouped && !first_row && !last_row) {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) p.out[cur * p.dim + d + i] = acc[i];
-          if (second) p.out2[cur * p.heads + d / p.head_dim] = acc2;
+          if (second) p.out2[cur * p.heads + h] = acc2;
         } else {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) atomicAdd(&p.out[cur * p.dim + d + i], acc[i]);
-          if (second) atomicAdd(&p.out2[cur * p.heads + d / p.head_dim], acc2);
+          if (second) atomicAdd(&p.out2[cur * p.heads + h], acc2);
         }
       }
       if (cur >= 0) first_row = false;
     };
-    for (int64_t eb = e0; eb < e1; eb += kUnroll) {
+    for (int i0 = 0; i0 < n; i0 += kUnroll) {
       float v[kUnroll][VEC];
       float v2[kUnroll];
       int64_t dst[kUnroll];
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        const int64_t e = eb + u;
         dst[u] = -1;
         v2[u] = 0.f;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v[u][i] = 0.f;
-        if (e < e1) {
-          const int k = segment_of(s_off, p.num_seg, e);
-          dst[u] = s_out[k] + p.col[e];
-          if (live) {
-            if (MODE == 1) {
-              load_vec<T, VEC>(in, e * p.dim + d, v[u]);
-            } else {
-              const int64_t src = s_in[k] + p.row[e];
-              if (src >= 0 && src < p.num_in_rows) load_vec<T, VEC>(in, src * p.dim + d, v[u]);
-              if (MODE == 2) {
-                float w[VEC];
-                load_vec<T, VEC>(ed, e * p.dim + d, w);
+        if (i0 + u < n) {
+          dst[u] = wave_read(my_dst, i0 + u);
+          if (MODE == 1) {
+            if (live) load_vec<T, VEC>(in, (e0 + i0 + u) * p.dim + d, v[u]);
+          } else {
+            const int64_t src = wave_read(my_src, i0 + u);
+            if (live && src >= 0) load_vec<T, VEC>(in, src * p.dim + d, v[u]);
+            if (MODE == 2 && live) {
+              float w[VEC];
+              load_vec<T, VEC>(ed, (e0 + i0 + u) * p.dim + d, w);
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) v[u][i] *= w[i];
-              }
-              if (MODE == 3) {
-                const int64_t we = p.head_w_row != nullptr ? p.head_w_row[e] : e;
-                const float w = p.head_w[we * p.heads + d / p.head_dim];
+              for (int i = 0; i < VEC; ++i) v[u][i] *= w[i];
+            }
+            if (MODE == 3) {
+              const int64_t we = wave_read(my_we, i0 + u);
+              if (live) {
+                const float w = p.head_w[we * p.heads + h];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) v[u][i] *= w;
-                if (second) v2[u] = p.head_w2[we * p.heads + d / p.head_dim];
+                if (second) v2[u] = p.head_w2[we * p.heads + h];
               }
             }
           }
@@ -165,7 +184,7 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
       }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
-        if (eb + u < e1) {
+        if (i0 + u < n) {
           if (dst[u] != cur) {
             flush(false);
 #pragma unroll
