@@ -73,6 +73,9 @@ def parse_args():
     ap.add_argument("--aggregation", action="store_true",
                     help="also time GraphSAGE-style SpMM (hidden 256, fp32 and bf16) and SDDMM on the "
                          "outermost sampled block of the last batch")
+    ap.add_argument("--cache_build", action="store_true",
+                    help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
+                         "cached feature table) and one step of the all-strategies dry run")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
@@ -444,6 +447,54 @@ def main():
             fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
             del fp
 
+    # ---- optional: cache construction and the strategy dry run (the callers of the registries)
+    cache_build = None
+    if args.cache_build and requests is None:
+        from apt_amd import cache as cache_mod
+        from apt_amd import cost_model as cm
+
+        def time_ms(fn, reps=5):
+            fn()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps
+
+        stage_pipe.run(seed_sets[W], args.seed + 100 + W)
+        torch.cuda.synchronize()
+        H = len(hops)
+        n_in = int(stage_pipe.sizes[H].item())
+        counter = cache_mod.HotnessCounter(N, dev)
+        t_count = time_ms(lambda: counter.add(stage_pipe.nodes, n_dev=stage_pipe.sizes[H:H + 1], output_nodes=seed_sets[W]))
+        deg = indptr[1:] - indptr[:-1]
+        hot = torch.topk(deg, min(1_000_000, N // 4)).indices.contiguous()
+        t_csr = time_ms(lambda: cache_mod.build_graph_cache(graph, hot), reps=3)
+        c_edges = int(deg[hot].sum().item())
+        t_feat = time_ms(lambda: capi.gather_rows(store, hot), reps=3)
+        world = 8
+        mv = torch.linspace(0, N, world + 1).to(torch.int64)
+        run = cm.AllPSDryRun(graph, world, list(reversed(hops)), mv, rng_seed=args.seed)
+        per_rank = [seed_sets[i % len(seed_sets)] for i in range(world)]
+        run.sample(per_rank)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        res = run.sample(per_rank)
+        torch.cuda.synchronize()
+        t_dry = time.perf_counter() - t0
+        cache_build = {
+            "count_ids_us": t_count * 1e3, "count_ids_nodes": n_in + B,
+            "cached_csr_rows": int(hot.numel()), "cached_csr_edges": c_edges, "cached_csr_ms": t_csr,
+            "cached_csr_GBps": 16.0 * c_edges / (t_csr * 1e-3) / 1e9,          # every edge read and written once
+            "cached_features_ms": t_feat, "cached_features_GBps": hot.numel() * bytes_per_row / (t_feat * 1e-3) / 1e9,
+            "dry_run_all_strategies_ms_per_step": t_dry * 1e3, "dry_run_world_size": world,
+            "dry_run_input_nodes_rank0": {"DP": int(res[0].dp_seeds.numel()), "NP": int(res[0].np_seeds.numel()),
+                                          "SP": int(res[0].sp_seeds.numel()), "MP": int(res[0].mp_seeds.numel())},
+        }
+        del counter, hot, deg, run, res
+
     # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
     cpu = None
     budget = args.cpu_seconds
@@ -549,6 +600,7 @@ def main():
         "cpu_baseline": cpu,
         "aggregation": agg,
         "block_formats": fmt,
+        "cache_build": cache_build,
         "stages": {
             "in_flight": in_flight,
             "edges_per_step": edges / K,
