@@ -50,12 +50,19 @@ __device__ __forceinline__ int64_t owner_row(const int64_t* out_indptr, int64_t 
 }
 
 // out_indices[out_indptr[i] + k] = indices[indptr[rows[i]] + k].  Work is split
-// by output position, so a 2 M-edge hub row is copied by many workgroups.
+// by output position, so a 2 M-edge hub row is copied by many workgroups.  A
+// workgroup whose 4096 positions touch only a few rows (the usual case for hot
+// rows) copies them segment by segment, each thread streaming 8-byte elements
+// with nothing else to look up; one that spans many short rows finds every
+// element's row by binary search.
+constexpr int kCopySegRows = 16;
+
 __global__ __launch_bounds__(kCacheBlock) void copy_rows_kernel(
     const int64_t* __restrict__ indptr, const int64_t* __restrict__ indices, int64_t row_begin,
     const int64_t* __restrict__ rows, int64_t n, const int64_t* __restrict__ out_indptr,
     int64_t* __restrict__ out_indices) {
   __shared__ int64_t s_lo, s_hi;
+  __shared__ int64_t s_dst[kCopySegRows + 1], s_src[kCopySegRows];
   const int64_t total = out_indptr[n];
   const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kCopyEdgesPerBlock;
   if (e0 >= total) return;
@@ -64,6 +71,19 @@ __global__ __launch_bounds__(kCacheBlock) void copy_rows_kernel(
   if (threadIdx.x == 1) s_hi = owner_row(out_indptr, 0, n - 1, e1);
   __syncthreads();
   const int64_t lo = s_lo, hi = s_hi;
+  if (hi - lo < kCopySegRows) {
+    const int nseg = static_cast<int>(hi - lo + 1);
+    if (static_cast<int>(threadIdx.x) <= nseg) s_dst[threadIdx.x] = out_indptr[lo + threadIdx.x];
+    if (static_cast<int>(threadIdx.x) < nseg) s_src[threadIdx.x] = indptr[rows[lo + threadIdx.x] - row_begin];
+    __syncthreads();
+    for (int k = 0; k < nseg; ++k) {
+      const int64_t b = max(s_dst[k], e0), e = min(s_dst[k + 1], e1 + 1);
+      const int64_t* src = indices + s_src[k] - s_dst[k];   // src[pos] is the element for output position pos
+      for (int64_t pos = b + threadIdx.x; pos < e; pos += kCacheBlock)
+        out_indices[pos] = __builtin_nontemporal_load(src + pos);
+    }
+    return;
+  }
   for (int64_t e = e0 + threadIdx.x; e <= e1; e += kCacheBlock) {
     const int64_t i = owner_row(out_indptr, lo, hi, e);
     const int64_t r = rows[i] - row_begin;
