@@ -346,3 +346,44 @@ def test_operator_layer_fused_sampler(orc, capi):
     sizes, nodes, hops = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9)
     want_in, _ = orc.sample_blocks(orc.Graph(indptr2, indices2), np.arange(50), [4], False, 9)
     assert np.array_equal(nodes.cpu().numpy(), want_in)
+
+
+def test_fused_driver_random_configurations(orc, capi):
+    """Sixty random plans (1-4 hops, fanouts 1..70 incl. those wider than a wavefront,
+    batches 1..3000, with and without replacement, repeated / out-of-range / negative
+    seeds, graphs with isolated rows and hubs): fused driver, per-hop driver and oracle
+    agree on every array."""
+    from apt_amd.pipeline import MiniBatchPipeline
+    rng = np.random.default_rng(2024)
+    graphs = []
+    for seed, (n, deg) in enumerate([(500, 3), (5000, 12), (40000, 25)]):
+        indptr, indices = small_graph(n, deg, seed=50 + seed)
+        graphs.append((n, orc.Graph(indptr, indices), capi.Graph(dev(indptr), dev(indices))))
+    for case in range(60):
+        n, og, dg = graphs[case % 3]
+        H = int(rng.integers(1, 5))
+        hops = [int(rng.choice([1, 2, 3, 5, 8, 15, 16, 17, 33, 64, 70])) for _ in range(H)]
+        B = int(rng.choice([1, 2, 63, 64, 65, 300, 1000, 3000]))
+        while B * np.prod([1 + f for f in hops]) > 3e6:        # keep the upper-bound buffers small
+            hops = hops[:-1] if len(hops) > 1 else [min(hops[0], 15)]
+            B = min(B, 300)
+        replace = bool(rng.integers(0, 2))
+        seeds = rng.integers(0, n, size=B)
+        if case % 4 == 1 and B > 2:
+            seeds[1] = seeds[0]
+            seeds[-1] = -1
+        if case % 4 == 2:
+            seeds[0] = n + 5                                    # an id the graph does not have
+        key = 7000 + case
+        for fused in (True, False):
+            # the rank table of the fused driver treats an id it cannot hold as padding; the hash table of the
+            # per-hop driver keeps it as a node without neighbours
+            as_seen = np.where(seeds >= n, -1, seeds) if fused else seeds
+            want_in, want_blocks = orc.sample_blocks(og, as_seen, hops, replace, key)
+            pipe = MiniBatchPipeline(dg, None, B, hops, replace=replace, gather=False, fused=fused)
+            pipe.run(dev(seeds), key)
+            res = pipe.result()
+            assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in), (case, hops, B, replace, fused)
+            for got, want in zip(res["blocks"], want_blocks):
+                for k in ("neighbors", "relabeled", "counts", "unique"):
+                    assert np.array_equal(got[k].cpu().numpy(), want[k]), (case, hops, B, replace, fused, k)
