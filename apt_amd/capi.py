@@ -74,9 +74,7 @@ SYMBOLS = {
     "apt_gat_scores": (_I, [_P, _I64, _I, _I64, _I, _P, _P, _P]),
     "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
     "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
-    "apt_spmm_csr_workspace_bytes": (C.c_size_t, [_I64]),
-    "apt_spmm_csr": (_I, [_P, _P, _P, _I64, _I64, _P, _I64, _I64, _I, _P, _P, _P, _I, _P, _P, _P, C.c_size_t, _P]),
-    "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P]),
+    "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P, _P]),
     # include/apt_synth.h
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
@@ -656,59 +654,47 @@ def gat_block_backward(neighbors, num_dst, fanout, ft, el, er, negative_slope, a
     return a_edge, dz_edge, d_er
 
 
-def spmm_csr(indptr, indices, x, eids=None, col_scale=None, head_weights=None, head_weights2=None):
-    """out[r] = sum over the edges e of CSR row r of col_scale[indices[e]] * head_weights[w(e), h] * x[indices[e]],
-    w(e) = eids[e] or e.  x [n, dim] or [n, heads, head_dim] -> fp32 of the same trailing shape with
-    len(indptr) - 1 rows, every row written once (no zero-fill, no atomics).  With head_weights2 also returns
-    out2[r, h] = sum of head_weights2[w(e), h]."""
-    indptr, indices = _dev_i64(indptr, "indptr"), _dev_i64(indices, "indices")
-    eids = _dev_i64(eids, "eids")
-    if x.dim() == 3:
-        n, heads, hd = x.shape
-    else:
-        x = _feat2d(x, "x")
-        (n, hd), heads = x.shape, 1
-    if not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
-        raise AptError("spmm_csr: x must be a contiguous fp32 or bf16 tensor")
-    rows, edges = indptr.numel() - 1, indices.numel()
-    if eids is not None and eids.numel() != edges:
-        raise AptError("spmm_csr: eids must have one entry per edge")
-    col_scale = _f32(col_scale, "col_scale")
-    head_weights, head_weights2 = _f32(head_weights, "head_weights"), _f32(head_weights2, "head_weights2")
-    for w in (head_weights, head_weights2):
-        if w is not None and (w.dim() != 2 or w.shape[1] != heads):
-            raise AptError("spmm_csr: head weights must be [*, heads]")
-    if col_scale is not None and col_scale.numel() != n:
-        raise AptError("spmm_csr: col_scale must have one entry per row of x")
-    out = torch.empty((rows,) + tuple(x.shape[1:]), dtype=torch.float32, device=x.device)
-    out2 = torch.empty((rows, heads), dtype=torch.float32, device=x.device) if head_weights2 is not None else None
-    ws = torch.empty(int(lib().apt_spmm_csr_workspace_bytes(edges)), dtype=torch.uint8, device=x.device)
-    check(lib().apt_spmm_csr(_ptr(indptr), _ptr(indices), _ptr(eids), rows, edges, _ptr(x), n, heads * hd,
-                             x.element_size(), _ptr(col_scale), _ptr(head_weights), _ptr(head_weights2), heads,
-                             _ptr(out), _ptr(out2), _ptr(ws), ws.numel(), _stream()))
-    return out if out2 is None else (out, out2)
-
-
-def spmm_heads(row, col, x, head_weights, num_out, weight_row=None, grouped=False, head_weights2=None):
+def spmm_heads(row, col, x, head_weights, num_out, weight_row=None, grouped=False, head_weights2=None,
+               out_indptr=None, out=None, out2=None):
     """out[col[e], h, :] += head_weights[w(e), h] * x[row[e], h, :], w(e) = weight_row[e] or e;
-    x [n, heads, head_dim] -> fp32 [num_out, heads, head_dim].  grouped: edges with equal col are consecutive.
-    head_weights2: also returns out2[col[e], h] += head_weights2[w(e), h]."""
+    x [n, heads, head_dim] (or [n, dim]: one head) -> fp32 of the same trailing shape with num_out rows.
+    head_weights None = all ones.  grouped: edges with equal col are consecutive.  head_weights2: also
+    returns out2[col[e], h] += head_weights2[w(e), h].  out_indptr (with grouped): CSR offsets of col; the
+    outputs are then not zero-filled first (the library zeroes the rows it has to)."""
     row, col = _dev_i64(row, "row"), _dev_i64(col, "col")
-    weight_row = _dev_i64(weight_row, "weight_row")
+    weight_row, out_indptr = _dev_i64(weight_row, "weight_row"), _dev_i64(out_indptr, "out_indptr")
+    if x.dim() == 2:
+        x = x.unsqueeze(1)
+        flat = True
+    else:
+        flat = False
     n, heads, hd = x.shape
     w = _f32(head_weights, "head_weights")
-    if w.dim() != 2 or w.shape[1] != heads or not x.is_contiguous():
-        raise AptError("spmm_heads: head_weights must be [*, heads] and x contiguous")
-    if weight_row is None and w.shape[0] != row.numel():
-        raise AptError("spmm_heads: head_weights needs one row per edge")
-    out = torch.zeros((num_out, heads, hd), dtype=torch.float32, device=x.device)
-    out2 = None
+    if not x.is_contiguous() or x.dtype not in (torch.float32, torch.bfloat16):
+        raise AptError("spmm_heads: x must be a contiguous fp32 or bf16 tensor")
+    if w is not None:
+        if w.dim() != 2 or w.shape[1] != heads:
+            raise AptError("spmm_heads: head_weights must be [*, heads]")
+        if weight_row is None and w.shape[0] != row.numel():
+            raise AptError("spmm_heads: head_weights needs one row per edge")
+    if out_indptr is not None and (not grouped or out_indptr.numel() != num_out + 1):
+        raise AptError("spmm_heads: out_indptr needs grouped edges and num_out + 1 entries")
+    make = torch.empty if out_indptr is not None else torch.zeros
+    if out is None:
+        out = make((num_out, heads, hd), dtype=torch.float32, device=x.device)
+    elif out.numel() != num_out * heads * hd or out.dtype != torch.float32 or not out.is_contiguous():
+        raise AptError("spmm_heads: out must be a contiguous fp32 tensor of num_out rows")
+    else:
+        out = out.view(num_out, heads, hd)
     if head_weights2 is not None:
         head_weights2 = _f32(head_weights2, "head_weights2")
-        if head_weights2.shape != w.shape:
-            raise AptError("spmm_heads: head_weights2 must have the shape of head_weights")
-        out2 = torch.zeros((num_out, heads), dtype=torch.float32, device=x.device)
+        if head_weights2.dim() != 2 or head_weights2.shape[1] != heads:
+            raise AptError("spmm_heads: head_weights2 must be [*, heads]")
+        if out2 is None:
+            out2 = make((num_out, heads), dtype=torch.float32, device=x.device)
     check(lib().apt_spmm_heads(_ptr(row), _ptr(col), row.numel(), _ptr(x), n, _ptr(w), _ptr(weight_row), heads,
                                heads * hd, x.element_size(), int(grouped), _ptr(out), num_out, _ptr(head_weights2),
-                               _ptr(out2), _stream()))
+                               _ptr(out2), _ptr(out_indptr), _stream()))
+    if flat:
+        out = out.squeeze(1)
     return out if out2 is None else (out, out2)

@@ -42,6 +42,9 @@ struct AggParams {
   int64_t head_dim;         // dim / heads
   int grouped;              // edges with equal col are consecutive: rows inside a wavefront's range are stored, not added
   const int* grouped_dev;   // the same as a device flag (apt_coo_is_grouped), or NULL
+  const int64_t* out_indptr;  // grouped only, optional: offsets of the output rows in the edge list (CSR of col).
+                              // Rows inside a wavefront's range are then recognised exactly, the rest (rows that
+                              // span ranges, rows without edges) is zeroed by spmm_zero_rows_kernel: out need not be zero
 };
 
 template <typename T> __device__ __forceinline__ float to_float(T v);
@@ -135,7 +138,10 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
     float acc2 = 0.f;
     auto flush = [&](bool last_row) {
       if (cur >= 0 && cur < p.num_out_rows && live) {
-        if (grouped && !first_row && !last_row) {
+        bool inside = !first_row && !last_row;
+        if (!inside && p.out_indptr != nullptr)   // the range's first or last row: does it begin and end in here?
+          inside = p.out_indptr[cur] >= e0 && p.out_indptr[cur + 1] <= e0 + n;
+        if (grouped && inside) {
 #pragma unroll
           for (int i = 0; i < VEC; ++i) p.out[cur * p.dim + d + i] = acc[i];
           if (second) p.out2[cur * p.heads + h] = acc2;
@@ -173,9 +179,11 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
             if (MODE == 3) {
               const int64_t we = wave_read(my_we, i0 + u);
               if (live) {
-                const float w = p.head_w[we * p.heads + h];
+                if (p.head_w != nullptr) {
+                  const float w = p.head_w[we * p.heads + h];
 #pragma unroll
-                for (int i = 0; i < VEC; ++i) v[u][i] *= w;
+                  for (int i = 0; i < VEC; ++i) v[u][i] *= w;
+                }
                 if (second) v2[u] = p.head_w2[we * p.heads + h];
               }
             }
@@ -199,6 +207,23 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
       }
     }
     flush(true);
+  }
+}
+
+// Companion of spmm_kernel with out_indptr: zeroes the output rows that the main kernel does not store whole,
+// i.e. rows without edges and rows whose edges lie in more than one wavefront range (those are added
+// atomically).  A lane group of 16 per row.
+__global__ __launch_bounds__(kAggBlock) void spmm_zero_rows_kernel(const int64_t* __restrict__ out_indptr,
+                                                                   int64_t num_rows, int64_t dim, float* out,
+                                                                   float* out2, int heads) {
+  constexpr int kLanes = 16;
+  const int l = threadIdx.x % kLanes;
+  for (int64_t r = (static_cast<int64_t>(blockIdx.x) * kAggBlock + threadIdx.x) / kLanes; r < num_rows;
+       r += static_cast<int64_t>(gridDim.x) * (kAggBlock / kLanes)) {
+    const int64_t lo = out_indptr[r], hi = out_indptr[r + 1];
+    if (hi > lo && lo / kEdgesPerWave == (hi - 1) / kEdgesPerWave) continue;   // stored whole by one wavefront
+    for (int64_t d = l; d < dim; d += kLanes) out[r * dim + d] = 0.f;
+    if (out2 != nullptr && l < heads) out2[r * heads + l] = 0.f;
   }
 }
 
@@ -640,303 +665,7 @@ static int agg_check(const char* who, const int64_t* row, const int64_t* col, in
   return APT_OK;
 }
 
-// ---------------------------------------------------------------------------
-// Row-owned SpMM over CSR: out[r, :] = sum over the edges e of row r of
-//   col_scale[indices[e]] * head_w[w(e), head] * x[indices[e], :],  w(e) = eids[e] or e.
-// A lane group owns an output row and writes it exactly once (zeros for an empty
-// row), so there are no atomics, no zero-fill and the sum runs in edge order.
-// This is the backward direction of a sampled block (edges grouped by source):
-// most rows have one or two edges, a few hubs have thousands.  Rows above
-// kCsrLongRow edges are put on a list instead and summed by a whole workgroup
-// each in a second launch (edges dealt round-robin to its lane groups, partial
-// sums combined in LDS in a fixed order).
-constexpr int kCsrLongRow = 128;
-
-struct CsrParams {
-  const int64_t* indptr;     // [num_rows + 1]
-  const int64_t* indices;    // [E] row of x per edge
-  const int64_t* eids;       // [E] row of head_w per edge, or NULL (= e)
-  int64_t num_rows, num_x_rows, dim;
-  const void* x;
-  const float* col_scale;    // [num_x_rows] or NULL
-  const float* head_w;       // [*, heads] or NULL
-  const float* head_w2;      // [*, heads] or NULL: out2[r, h] = sum over the row's edges of head_w2[w(e), h]
-  float* out;                // [num_rows, dim]
-  float* out2;               // [num_rows, heads]
-  int heads;
-  int64_t head_dim;
-  int64_t* long_rows;        // rows left to the second launch
-  uint32_t* long_count;
-  int64_t long_cap;
-};
-
-// Streams VEC consecutive floats out (the output of a backward sum is not read again soon).
-template <int VEC>
-__device__ __forceinline__ void store_stream(float* dst, const float (&v)[VEC]) {
-  if constexpr (VEC % 4 == 0) {
-    typedef float f4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-    for (int i = 0; i < VEC; i += 4) {
-      f4 t = {v[i], v[i + 1], v[i + 2], v[i + 3]};
-      __builtin_nontemporal_store(t, reinterpret_cast<f4*>(dst + i));
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) __builtin_nontemporal_store(v[i], dst + i);
-  }
-}
-
-// One edge's contribution to the lane's VEC features (and to the second sum).
-template <typename T, int VEC>
-__device__ __forceinline__ void csr_edge(const CsrParams& p, const T* x, int64_t e, int64_t d, int h, bool second,
-                                         float (&v)[VEC], float& v2) {
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) v[i] = 0.f;
-  v2 = 0.f;
-  const int64_t j = p.indices[e];
-  if (j < 0 || j >= p.num_x_rows) return;
-  load_vec<T, VEC>(x, j * p.dim + d, v);
-  float w = p.col_scale != nullptr ? p.col_scale[j] : 1.f;
-  if (p.head_w != nullptr || second) {
-    const int64_t we = p.eids != nullptr ? p.eids[e] : e;
-    if (p.head_w != nullptr) w *= p.head_w[we * p.heads + h];
-    if (second) v2 = p.head_w2[we * p.heads + h];
-  }
-#pragma unroll
-  for (int i = 0; i < VEC; ++i) v[i] *= w;
-}
-
-// A lane group takes kCsrRows consecutive rows at a time and has the first
-// kCsrFirst edges of all of them in flight together (most rows of a block's
-// backward direction have one or two edges, so one row at a time would leave a
-// wavefront waiting on a single 1 KB load); what a row has beyond that follows
-// row by row.
-constexpr int kCsrRows = 4;
-constexpr int kCsrFirst = 2;
-
-template <typename T, int VEC, int LPR>
-__global__ __launch_bounds__(kAggBlock) void spmm_csr_kernel(CsrParams p) {
-  constexpr int kGroups = kAggBlock / LPR;
-  constexpr int kUnroll = 4;
-  const T* x = static_cast<const T*>(p.x);
-  const int grp = threadIdx.x / LPR, l = threadIdx.x % LPR;
-  for (int64_t r0 = (static_cast<int64_t>(blockIdx.x) * kGroups + grp) * kCsrRows; r0 < p.num_rows;
-       r0 += static_cast<int64_t>(gridDim.x) * kGroups * kCsrRows) {
-    int64_t lo[kCsrRows], hi[kCsrRows];
-    bool mine[kCsrRows];
-#pragma unroll
-    for (int rr = 0; rr < kCsrRows; ++rr) {
-      const bool in = r0 + rr < p.num_rows;
-      lo[rr] = in ? p.indptr[r0 + rr] : 0;
-      hi[rr] = in ? p.indptr[r0 + rr + 1] : 0;
-      mine[rr] = in && hi[rr] - lo[rr] <= kCsrLongRow;
-      if (in && !mine[rr] && l == 0) {
-        const uint32_t k = atomicAdd(p.long_count, 1u);
-        if (static_cast<int64_t>(k) < p.long_cap) p.long_rows[k] = r0 + rr;
-      }
-      if (!mine[rr]) hi[rr] = lo[rr];
-    }
-    for (int64_t d = static_cast<int64_t>(l) * VEC; d < p.dim; d += LPR * VEC) {
-      const int h = static_cast<int>(d / p.head_dim);
-      const bool second = p.head_w2 != nullptr && d == h * p.head_dim;
-      float acc[kCsrRows][VEC], acc2[kCsrRows];
-      {
-        float v[kCsrRows][kCsrFirst][VEC], v2[kCsrRows][kCsrFirst];
-#pragma unroll
-        for (int rr = 0; rr < kCsrRows; ++rr)
-#pragma unroll
-          for (int u = 0; u < kCsrFirst; ++u) {
-            if (lo[rr] + u < hi[rr]) {
-              csr_edge<T, VEC>(p, x, lo[rr] + u, d, h, second, v[rr][u], v2[rr][u]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < VEC; ++i) v[rr][u][i] = 0.f;
-              v2[rr][u] = 0.f;
-            }
-          }
-#pragma unroll
-        for (int rr = 0; rr < kCsrRows; ++rr) {
-#pragma unroll
-          for (int i = 0; i < VEC; ++i) acc[rr][i] = 0.f;
-          acc2[rr] = 0.f;
-#pragma unroll
-          for (int u = 0; u < kCsrFirst; ++u) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[rr][i] += v[rr][u][i];
-            acc2[rr] += v2[rr][u];
-          }
-        }
-      }
-#pragma unroll
-      for (int rr = 0; rr < kCsrRows; ++rr) {
-        for (int64_t e0 = lo[rr] + kCsrFirst; e0 < hi[rr]; e0 += kUnroll) {
-          float v[kUnroll][VEC], v2[kUnroll];
-#pragma unroll
-          for (int u = 0; u < kUnroll; ++u) {
-            if (e0 + u < hi[rr]) {
-              csr_edge<T, VEC>(p, x, e0 + u, d, h, second, v[u], v2[u]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < VEC; ++i) v[u][i] = 0.f;
-              v2[u] = 0.f;
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[rr][i] += v[u][i];
-            acc2[rr] += v2[u];
-          }
-        }
-        if (mine[rr]) {
-          store_stream<VEC>(p.out + (r0 + rr) * p.dim + d, acc[rr]);
-          if (second) p.out2[(r0 + rr) * p.heads + h] = acc2[rr];
-        }
-      }
-    }
-  }
-}
-
-// A workgroup of 1024 threads per listed row.  Lane group g sums edges lo + g,
-// lo + g + G, ... (kLongUnroll of them in flight); the G partial rows meet in LDS
-// and lane group 0 adds them up in order.
-constexpr int kCsrLongBlock = 1024;
-constexpr int kLongUnroll = 8;
-
-template <typename T, int VEC, int LPR>
-__global__ __launch_bounds__(kCsrLongBlock) void spmm_csr_long_kernel(CsrParams p) {
-  constexpr int kGroups = kCsrLongBlock / LPR;
-  __shared__ float s_part[kGroups][LPR * VEC];
-  __shared__ float s_part2[kGroups][LPR];
-  const T* x = static_cast<const T*>(p.x);
-  const int grp = threadIdx.x / LPR, l = threadIdx.x % LPR;
-  const int64_t listed = min(static_cast<int64_t>(*p.long_count), p.long_cap);
-  for (int64_t k = blockIdx.x; k < listed; k += gridDim.x) {
-    const int64_t r = p.long_rows[k];
-    const int64_t lo = p.indptr[r], hi = p.indptr[r + 1];
-    for (int64_t d0 = 0; d0 < p.dim; d0 += LPR * VEC) {
-      const int64_t d = d0 + static_cast<int64_t>(l) * VEC;
-      const bool live = d < p.dim;
-      const int h = static_cast<int>(d / p.head_dim);
-      const bool second = live && p.head_w2 != nullptr && d == h * p.head_dim;
-      float acc[VEC];
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
-      float acc2 = 0.f;
-      if (live) {
-        for (int64_t e0 = lo + grp; e0 < hi; e0 += static_cast<int64_t>(kLongUnroll) * kGroups) {
-          float v[kLongUnroll][VEC], v2[kLongUnroll];
-#pragma unroll
-          for (int u = 0; u < kLongUnroll; ++u) {
-            const int64_t e = e0 + static_cast<int64_t>(u) * kGroups;
-            if (e < hi) {
-              csr_edge<T, VEC>(p, x, e, d, h, second, v[u], v2[u]);
-            } else {
-#pragma unroll
-              for (int i = 0; i < VEC; ++i) v[u][i] = 0.f;
-              v2[u] = 0.f;
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < kLongUnroll; ++u) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] += v[u][i];
-            acc2 += v2[u];
-          }
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) s_part[grp][l * VEC + i] = acc[i];
-      s_part2[grp][l] = acc2;
-      __syncthreads();
-      if (grp == 0 && live) {
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          float t = 0.f;
-          for (int g = 0; g < kGroups; ++g) t += s_part[g][l * VEC + i];
-          p.out[r * p.dim + d + i] = t;
-        }
-        if (second) {
-          float t = 0.f;
-          for (int g = 0; g < kGroups; ++g) t += s_part2[g][l];
-          p.out2[r * p.heads + h] = t;
-        }
-      }
-      __syncthreads();
-    }
-  }
-}
-
-__global__ void csr_zero_count_kernel(uint32_t* c) { *c = 0; }
-
-template <typename T, int VEC, int LPR>
-static void launch_spmm_csr(const CsrParams& p, hipStream_t st) {
-  constexpr int kGroups = kAggBlock / LPR;
-  const unsigned blocks =
-      static_cast<unsigned>(std::min<int64_t>(ceil_div(p.num_rows, static_cast<int64_t>(kGroups) * kCsrRows), 1 << 20));
-  hipLaunchKernelGGL((spmm_csr_kernel<T, VEC, LPR>), dim3(blocks), dim3(kAggBlock), 0, st, p);
-  const unsigned long_blocks = static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(p.long_cap, 2048)));
-  hipLaunchKernelGGL((spmm_csr_long_kernel<T, VEC, LPR>), dim3(long_blocks), dim3(kCsrLongBlock), 0, st, p);
-}
-
-template <typename T, int VEC>
-static bool dispatch_spmm_csr(const CsrParams& p, hipStream_t st) {
-  if (p.dim % VEC != 0 || p.head_dim % VEC != 0) return false;
-  const int64_t lanes = p.dim / VEC;
-  if (lanes <= 8) launch_spmm_csr<T, VEC, 8>(p, st);
-  else if (lanes <= 16) launch_spmm_csr<T, VEC, 16>(p, st);
-  else if (lanes <= 32) launch_spmm_csr<T, VEC, 32>(p, st);
-  else launch_spmm_csr<T, VEC, 64>(p, st);
-  return true;
-}
-
 }  // namespace apt
-
-extern "C" size_t apt_spmm_csr_workspace_bytes(int64_t num_edges) {
-  if (num_edges < 0) return 0;
-  return 256 + sizeof(int64_t) * static_cast<size_t>(num_edges / apt::kCsrLongRow + 1);
-}
-
-extern "C" int apt_spmm_csr(const int64_t* indptr, const int64_t* indices, const int64_t* eids, int64_t num_rows,
-                            int64_t num_edges, const void* x, int64_t num_x_rows, int64_t dim, int elem_size,
-                            const float* col_scale, const float* head_weights, const float* head_weights2,
-                            int heads, float* out, float* out2, void* workspace, size_t workspace_bytes,
-                            void* stream) {
-  using namespace apt;
-  APT_REQUIRE(num_rows >= 0 && num_edges >= 0 && num_x_rows >= 0 && dim > 0 && heads > 0 && dim % heads == 0,
-              APT_EINVAL, "apt_spmm_csr: bad shape (rows %lld, E %lld, dim %lld, heads %d)", (long long)num_rows,
-              (long long)num_edges, (long long)dim, heads);
-  APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_spmm_csr: elem_size %d (4 = fp32, 2 = bf16)",
-              elem_size);
-  APT_REQUIRE((head_weights2 == nullptr) == (out2 == nullptr), APT_EINVAL,
-              "apt_spmm_csr: head_weights2 and out2 go together");
-  if (num_rows == 0) return APT_OK;
-  APT_REQUIRE(indptr != nullptr && out != nullptr && (num_edges == 0 || (indices != nullptr && x != nullptr)),
-              APT_EINVAL, "apt_spmm_csr: a tensor is NULL");
-  APT_REQUIRE(workspace != nullptr && workspace_bytes >= apt_spmm_csr_workspace_bytes(num_edges) &&
-                  (reinterpret_cast<uintptr_t>(workspace) & 7) == 0,
-              APT_EINVAL, "apt_spmm_csr: workspace too small or not 8-byte aligned (see apt_spmm_csr_workspace_bytes)");
-  CsrParams p{};
-  p.indptr = indptr; p.indices = indices; p.eids = eids;
-  p.num_rows = num_rows; p.num_x_rows = num_x_rows; p.dim = dim;
-  p.x = x; p.col_scale = col_scale; p.head_w = head_weights; p.head_w2 = head_weights2;
-  p.out = out; p.out2 = out2; p.heads = heads; p.head_dim = dim / heads;
-  p.long_count = static_cast<uint32_t*>(workspace);
-  p.long_rows = reinterpret_cast<int64_t*>(static_cast<char*>(workspace) + 256);
-  p.long_cap = num_edges / kCsrLongRow + 1;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(csr_zero_count_kernel, dim3(1), dim3(1), 0, st, p.long_count);
-  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-  bool ok;
-  if (elem_size == 4) ok = (aligned && dispatch_spmm_csr<float, 4>(p, st)) || dispatch_spmm_csr<float, 1>(p, st);
-  else ok = (aligned && (dispatch_spmm_csr<uint16_t, 8>(p, st) || dispatch_spmm_csr<uint16_t, 4>(p, st))) ||
-            dispatch_spmm_csr<uint16_t, 1>(p, st);
-  APT_REQUIRE(ok, APT_EINVAL, "apt_spmm_csr: unsupported shape");
-  APT_LAUNCH_CHECK("spmm_csr_kernel");
-  return APT_OK;
-}
-
-
 
 extern "C" int apt_spmm_sum(int mode, const int64_t* coo_row, const int64_t* coo_col, int64_t num_edges,
                             const void* input, int64_t num_in_rows, const void* edata, int64_t dim,
@@ -1131,7 +860,7 @@ extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, in
                               const void* input, int64_t num_in_rows, const float* head_weights,
                               const int64_t* weight_row, int heads, int64_t dim, int elem_size, int grouped,
                               float* out, int64_t num_out_rows, const float* head_weights2, float* out2,
-                              void* stream) {
+                              const int64_t* out_indptr, void* stream) {
   using namespace apt;
   APT_REQUIRE(num_edges >= 0 && heads > 0 && dim > 0 && dim % heads == 0, APT_EINVAL,
               "apt_spmm_heads: bad shape (E %lld, heads %d, dim %lld)", (long long)num_edges, heads,
@@ -1139,10 +868,20 @@ extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, in
   APT_REQUIRE(elem_size == 2 || elem_size == 4, APT_EINVAL, "apt_spmm_heads: elem_size %d (4 = fp32, 2 = bf16)",
               elem_size);
   APT_REQUIRE(num_out_rows >= 0 && num_in_rows >= 0, APT_EINVAL, "apt_spmm_heads: negative row count");
+  APT_REQUIRE(out_indptr == nullptr || grouped != 0, APT_EINVAL, "apt_spmm_heads: out_indptr needs grouped edges");
+  APT_REQUIRE(heads <= 16 || out2 == nullptr || out_indptr == nullptr, APT_ELIMIT,
+              "apt_spmm_heads: out_indptr with a second sum supports at most 16 heads");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_indptr != nullptr && num_out_rows > 0) {
+    APT_REQUIRE(out != nullptr, APT_EINVAL, "apt_spmm_heads: out is NULL");
+    const unsigned zb = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_out_rows, kAggBlock / 16), 1 << 20));
+    hipLaunchKernelGGL(spmm_zero_rows_kernel, dim3(zb), dim3(kAggBlock), 0, st, out_indptr, num_out_rows, dim, out,
+                       out2, heads);
+    APT_LAUNCH_CHECK("spmm_zero_rows_kernel");
+  }
   if (num_edges == 0) return APT_OK;
-  APT_REQUIRE(coo_row != nullptr && coo_col != nullptr && input != nullptr && head_weights != nullptr &&
-                  out != nullptr,
-              APT_EINVAL, "apt_spmm_heads: a tensor is NULL");
+  APT_REQUIRE(coo_row != nullptr && coo_col != nullptr && input != nullptr && out != nullptr, APT_EINVAL,
+              "apt_spmm_heads: a tensor is NULL");
   AggParams p{};
   p.row = coo_row; p.col = coo_col; p.num_edges = num_edges; p.in = input; p.out = out;
   p.num_seg = 1;  // no segment tables: every edge in segment 0, offsets 0
@@ -1150,12 +889,12 @@ extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, in
   p.dim = dim; p.num_in_rows = num_in_rows; p.num_e_rows = num_edges; p.num_out_rows = num_out_rows;
   p.head_w = head_weights; p.head_w_row = weight_row; p.heads = heads; p.head_dim = dim / heads;
   p.grouped = grouped != 0;
+  p.out_indptr = out_indptr;
   APT_REQUIRE((head_weights2 == nullptr) == (out2 == nullptr), APT_EINVAL,
               "apt_spmm_heads: head_weights2 and out2 go together");
   p.head_w2 = head_weights2; p.out2 = out2;
   const int64_t waves = ceil_div(num_edges, kEdgesPerWave);
   const dim3 grid(static_cast<unsigned>(ceil_div(waves, kAggWaves))), block(kAggBlock);
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec4 = p.head_dim % 4 == 0 && (reinterpret_cast<uintptr_t>(input) & 15) == 0;
   if (elem_size == 4) {
     if (vec4) hipLaunchKernelGGL((spmm_kernel<float, 3, 4>), grid, block, 0, st, p);

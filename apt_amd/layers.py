@@ -27,12 +27,14 @@ class BlockAggregate(torch.autograd.Function):
     def backward(ctx, dZ):
         block = ctx.block
         dZ = dZ.contiguous()
-        scale = None
         if ctx.mean:
             indptr = block.csc()[0]
-            scale = 1.0 / (indptr[1:] - indptr[:-1]).clamp(min=1).to(torch.float32)
-        indptr, dst, _ = block.csr()                   # edges grouped by source, by increasing edge id
-        dX = capi.spmm_csr(indptr, dst, dZ, col_scale=scale)    # every source row written once, in edge order
+            dZ = dZ / (indptr[1:] - indptr[:-1]).clamp(min=1).to(dZ.dtype)[:, None]
+        indptr, dst, eids = block.csr()                # edges grouped by source, by increasing edge id
+        src = block.row[eids]
+        # every source row is stored whole by the wavefront that holds its edges (or zeroed and added when it
+        # spans two): no zero-fill, no atomics for the bulk, sums in edge order
+        dX = capi.spmm_heads(dst, src, dZ, None, block.num_src, grouped=True, out_indptr=indptr)
         return None, dX.to(dZ.dtype), None
 
 
@@ -111,16 +113,14 @@ class GATAggregate(torch.autograd.Function):
         ft, el, er, attn = ctx.saved_tensors
         d_out = d_out.contiguous().float()
         csc_indptr = block.csc()[0]
-        _, dst, eids = block.csr()
+        indptr, dst, eids = block.csr()
         E = eids.numel()
         a_edge, dz_edge, d_er = capi.gat_block_backward(block.relabeled, block.num_dst, block.fanout, ft, el, er,
                                                         ctx.slope, attn, d_out, csc_indptr, E)
-        # sums over the edges of a source, in the block's CSR order; the per-edge weights stay in COO order.
-        # (capi.spmm_csr computes the same without a zero-fill, but its extra per-edge loads make it the
-        # slower of the two here.)
+        # sums over the edges of a source, in the block's CSR order; the per-edge weights stay in COO order
         src = block.row[eids]
         d_ft, d_el = capi.spmm_heads(dst, src, d_out, a_edge, block.num_src, weight_row=eids, grouped=True,
-                                     head_weights2=dz_edge)
+                                     head_weights2=dz_edge, out_indptr=indptr)
         return None, d_ft.to(ft.dtype), d_el, d_er, None
 
 

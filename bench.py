@@ -389,12 +389,13 @@ def main():
                 a_e, dz_e, d_er = capi.gat_block_backward(rel, n_dst, f, ft, el, er, 0.2, attn_w, d_out,
                                                           fmt_b["csc_indptr"], fmt_b["num_edges"])
                 capi.spmm_heads(fmt_b["csr_indices"], src_csr, d_out, a_e, n_src, weight_row=fmt_b["csr_eids"],
-                                grouped=True, head_weights2=dz_e)
+                                grouped=True, head_weights2=dz_e, out_indptr=csr_ip)
 
-            # backward of the plain sum / mean (SAGE, GCN): one row-owned pass over the CSR order
+            # backward of the plain sum / mean (SAGE, GCN): the same sum over the CSR order, no weights
             for tag, fn in (("gat_block_backward", gat_bwd),
-                            ("spmm_block_backward", lambda: capi.spmm_csr(csr_ip, fmt_b["csr_indices"], d2))):
-                if tag == "spmm_block_backward" and name != "fp32":
+                            ("spmm_block_backward", lambda: capi.spmm_heads(
+                                fmt_b["csr_indices"], src_csr, d2, None, n_src, grouped=True, out_indptr=csr_ip))):
+                if tag.startswith("spmm_block_backward") and name != "fp32":
                     continue
                 for _ in range(3):
                     fn()

@@ -438,27 +438,6 @@ int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_
                   const float* el, const float* er, float negative_slope, float* out,
                   float* attn_out, void* stream);
 
-/* Row-owned SpMM over CSR: the backward direction of a sampled block (the
- * reference gets it from the same COO operator with the edges reversed,
- * python/npc/model/sageconv.py:100-114, one atomicAdd per edge and feature).
- *   out[r, :] = sum over e in [indptr[r], indptr[r+1]) of
- *               col_scale[indices[e]] * head_weights[w(e), head of the feature] * x[indices[e], :]
- * with w(e) = eids[e] (or e when eids is NULL); col_scale and head_weights are
- * optional (NULL = 1).  x [num_x_rows, dim] fp32 or bf16 (elem_size 4 / 2), dim =
- * heads * head_dim; out fp32 [num_rows, dim].  head_weights2 / out2 (both or
- * neither): out2[r, h] = sum over the row's edges of head_weights2[w(e), h].
- * Every row of out (and out2) is written exactly once, zeros for a row without
- * edges: no zero-fill by the caller, no atomics, summation in edge order, so the
- * result is reproducible.  workspace: apt_spmm_csr_workspace_bytes(num_edges)
- * bytes, 8-byte aligned (the list of rows with more than 128 edges, which a whole
- * workgroup sums in a second launch). */
-size_t apt_spmm_csr_workspace_bytes(int64_t num_edges);
-int apt_spmm_csr(const int64_t* indptr, const int64_t* indices, const int64_t* eids, int64_t num_rows,
-                 int64_t num_edges, const void* x, int64_t num_x_rows, int64_t dim, int elem_size,
-                 const float* col_scale, const float* head_weights, const float* head_weights2,
-                 int heads, float* out, float* out2, void* workspace, size_t workspace_bytes,
-                 void* stream);
-
 /* Backward pass of apt_gat_block (no counterpart in the reference, whose GAT layer
  * gets its gradients from DGL's autograd).  Edge half, one wavefront per
  * (destination, head), fanout <= 64: from dOut [num_dst, heads, dim] and the
@@ -477,7 +456,13 @@ int apt_spmm_csr(const int64_t* indptr, const int64_t* indices, const int64_t* e
  *                   atomics and the result is deterministic.  head_weights2 / out2
  *                   (both or neither): out2[col[e], h] += head_weights2[w(e), h], a
  *                   second, scalar sum per row and head in the same pass (d el of
- *                   the GAT backward); out2 fp32 [num_out_rows, heads], zero-filled. */
+ *                   the GAT backward); out2 fp32 [num_out_rows, heads], zero-filled.
+ *                   head_weights may be NULL (all ones).  out_indptr, optional, grouped
+ *                   only: int64[num_out_rows + 1], offsets of the output rows in the edge
+ *                   list (the CSR offsets that go with col).  The library then zeroes
+ *                   the rows it must (rows without edges, rows whose edges span two
+ *                   wavefront ranges) itself and stores every other row whole: out and
+ *                   out2 need not be initialised. */
 int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst, int fanout, const void* ft,
                            int64_t num_src, int heads, int64_t dim, int elem_size, const float* el,
                            const float* er, float negative_slope, const float* attn,
@@ -487,7 +472,7 @@ int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, int64_t num_e
                    const void* input, int64_t num_in_rows, const float* head_weights,
                    const int64_t* weight_row, int heads, int64_t dim, int elem_size, int grouped,
                    float* out, int64_t num_out_rows, const float* head_weights2, float* out2,
-                   void* stream);
+                   const int64_t* out_indptr, void* stream);
 
 #ifdef __cplusplus
 }

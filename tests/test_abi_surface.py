@@ -62,8 +62,7 @@ def test_argument_checks_need_no_gpu():
     assert L.apt_vir_send_offset(0, 5, None, 0, None, 0, 0, None, None) != 0
     assert L.apt_spmm_block(None, 5, None, 0, None, 5, 8, 4, 0, None, None) != 0
     assert L.apt_coo_is_grouped(None, 5, None, None) != 0
-    assert L.apt_spmm_csr_workspace_bytes(1000) >= 256 + 8 * 8
-    assert L.apt_spmm_csr(None, None, None, 5, 0, None, 0, 8, 4, None, None, None, 3, None, None, None, 0, None) != 0
+    assert L.apt_spmm_heads(None, None, 5, None, 5, None, None, 3, 8, 4, 1, None, 5, None, None, None, None) != 0
     assert b"heads" in L.apt_last_error()
     for key in (b"sample_min_workgroups", b"gather_vector_bytes", b"block_fused_scan"):
         assert L.apt_set_tuning(key, 0) == 0

@@ -172,46 +172,6 @@ def test_gat_bf16_config5_shape(orc, capi):
     assert _close(got.cpu().numpy(), want, 1e-2)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,hd", [(1, 256), (4, 64), (3, 8), (1, 7), (2, 150)])
-def test_spmm_csr_rows_written_once(orc, capi, heads, hd, dtype):
-    """apt_spmm_csr vs the oracle: hub rows (second launch), empty rows (zeros without a
-    zero-fill), column scales, per-head weights through edge
-    ids, the second sum; two calls give identical bits."""
-    rng = np.random.default_rng(heads * 100 + hd)
-    rows, n_x = 3000, 700
-    deg = rng.integers(0, 5, rows)
-    deg[[5, 1700]] = [129, 2500]                              # just above the long-row threshold, and far above
-    deg[[6, 2999]] = [128, 0]
-    indptr = np.concatenate([[0], np.cumsum(deg)])
-    E = int(indptr[-1])
-    indices = rng.integers(0, n_x, E)
-    eids = rng.permutation(E)
-    x = rng.standard_normal((n_x, heads, hd)).astype(np.float32)
-    xt = dev(x).to(dtype)
-    xf = xt.float().cpu().numpy().reshape(n_x, heads * hd)
-    scale = (rng.random(n_x) + 0.5).astype(np.float32)
-    w = rng.standard_normal((E, heads)).astype(np.float32)
-    w2 = rng.standard_normal((E, heads)).astype(np.float32)
-    rtol = 1e-5 if dtype == torch.float32 else 1e-2
-    got = capi.spmm_csr(dev(indptr), dev(indices), xt)
-    assert got.shape == (rows, heads, hd)
-    assert _close(got.cpu().numpy().reshape(rows, -1), orc.spmm_csr(indptr, indices, xf), rtol)
-    assert not got[2999].any()
-    got = capi.spmm_csr(dev(indptr), dev(indices), xt, col_scale=dev(scale))
-    assert _close(got.cpu().numpy().reshape(rows, -1), orc.spmm_csr(indptr, indices, xf, col_scale=scale), rtol)
-    got, got2 = capi.spmm_csr(dev(indptr), dev(indices), xt, eids=dev(eids), head_weights=dev(w), head_weights2=dev(w2))
-    want, want2 = orc.spmm_csr(indptr, indices, xf, eids=eids, head_weights=w, head_weights2=w2, heads=heads)
-    assert _close(got.cpu().numpy().reshape(rows, -1), want, rtol) and _close(got2.cpu().numpy(), want2, 1e-5)
-    again, again2 = capi.spmm_csr(dev(indptr), dev(indices), xt, eids=dev(eids), head_weights=dev(w), head_weights2=dev(w2))
-    assert torch.equal(got, again) and torch.equal(got2, again2)
-    # nothing to do, and argument checks
-    empty = capi.spmm_csr(dev(np.zeros(5, dtype=np.int64)), dev(np.zeros(0, dtype=np.int64)), xt)
-    assert empty.shape == (4, heads, hd) and not empty.any()
-    with pytest.raises(capi.AptError):
-        capi.spmm_csr(dev(indptr), dev(indices), xt, eids=dev(eids[:-1]))
-
-
 def test_spmm_grouped_detection(orc, capi):
     """apt_coo_is_grouped: 1 for a destination-major COO, 0 once two edges are out of
     order; with the flag the sum skips the atomics inside a wavefront's edges and
@@ -239,3 +199,37 @@ def test_spmm_grouped_detection(orc, capi):
         assert capi.lib().apt_coo_is_grouped(ctypes.c_void_p(dev(col).data_ptr()), n,
                                              ctypes.c_void_p(flag.data_ptr()), stream) == 0
         assert int(flag.item()) == 1
+
+
+@pytest.mark.parametrize("heads,hd", [(4, 64), (1, 256), (3, 8), (1, 5)])
+def test_spmm_heads_owns_its_rows(orc, capi, heads, hd):
+    """apt_spmm_heads with the CSR offsets of col: outputs that start as NaN come back
+    complete (rows without edges zero, rows inside one wavefront range stored, rows that
+    span ranges zeroed and added) and equal the oracle; weights optional."""
+    rng = np.random.default_rng(heads * 31 + hd)
+    rows, n_x = 5000, 900
+    deg = rng.integers(0, 4, rows)
+    deg[[0, 17, 4000]] = [0, 200, 70]
+    deg[-3:] = 0
+    indptr = np.concatenate([[0], np.cumsum(deg)])
+    E = int(indptr[-1])
+    col = np.repeat(np.arange(rows), deg)
+    row = rng.integers(0, n_x, E)
+    eids = rng.permutation(E)
+    x = rng.standard_normal((n_x, heads, hd)).astype(np.float32)
+    w = rng.standard_normal((E, heads)).astype(np.float32)
+    w2 = rng.standard_normal((E, heads)).astype(np.float32)
+    nan = lambda *shape: torch.full(shape, float("nan"), device=DEV)
+    got, got2 = capi.spmm_heads(dev(row), dev(col), dev(x), dev(w), rows, weight_row=dev(eids), grouped=True,
+                                head_weights2=dev(w2), out_indptr=dev(indptr), out=nan(rows, heads, hd),
+                                out2=nan(rows, heads))
+    want, want2 = orc.spmm_csr(indptr, row, x.reshape(n_x, -1), eids=eids, head_weights=w, head_weights2=w2,
+                               heads=heads)
+    assert not torch.isnan(got).any() and not torch.isnan(got2).any()
+    assert _close(got.cpu().numpy().reshape(rows, -1), want, 1e-5) and _close(got2.cpu().numpy(), want2, 1e-5)
+    assert not got[0].any() and not got[-1].any()
+    plain = capi.spmm_heads(dev(row), dev(col), dev(x), None, rows, grouped=True, out_indptr=dev(indptr),
+                            out=nan(rows, heads, hd))
+    assert _close(plain.cpu().numpy().reshape(rows, -1), orc.spmm_csr(indptr, row, x.reshape(n_x, -1)), 1e-5)
+    with pytest.raises(capi.AptError):
+        capi.spmm_heads(dev(row), dev(col), dev(x), None, rows, grouped=False, out_indptr=dev(indptr))
