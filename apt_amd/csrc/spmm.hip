@@ -627,6 +627,104 @@ __global__ __launch_bounds__(kAggBlock) void gat_bwd_edge_group_kernel(
   }
 }
 
+// The same edge half with a wavefront per destination and two lane layouts.
+// Feature layout: lane l holds VEC features of head l / lph (as above).  Slot
+// layout: lane j holds (slot j / heads, head j % heads), so everything that
+// exists once per (slot, head) -- the neighbour id, the attention weight, el, the
+// dot product, the logit gradient, the edge position -- is loaded, computed and
+// stored by all lanes at once (three coalesced loads and two coalesced stores per
+// destination instead of six accesses per slot and head by one lane in sixteen).
+// Needs heads and lph to be powers of two, heads * lph <= 64 and
+// heads * fanout <= 64.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kAggBlock) void gat_bwd_edge_wave_kernel(
+    const int64_t* __restrict__ nbr, int64_t num_dst, int fanout, const T* __restrict__ ft, int64_t num_src,
+    int heads, int log2_heads, int64_t dim, const float* __restrict__ el, const float* __restrict__ er, float slope,
+    const float* __restrict__ attn, const float* __restrict__ d_out, const int64_t* __restrict__ csc_indptr,
+    float* __restrict__ a_edge, float* __restrict__ dz_edge, float* __restrict__ d_er) {
+  constexpr int kUnroll = 5;
+  const int lane = threadIdx.x % kWave;
+  const int lph = static_cast<int>(dim / VEC);
+  const int64_t row_len = static_cast<int64_t>(heads) * dim;
+  const bool live = lane < heads * lph;
+  const int64_t d = static_cast<int64_t>(lane) * VEC;
+  const int k = lane >> log2_heads, hs = lane & (heads - 1);   // slot layout
+  const bool slot = k < fanout;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave; i < num_dst;
+       i += static_cast<int64_t>(gridDim.x) * kAggWaves) {
+    const int64_t id = slot ? nbr[i * fanout + k] : -1;
+    const bool valid = id >= 0 && id < num_src;
+    const float a = valid ? attn[(i * fanout + k) * heads + hs] : 0.f;
+    const float z = valid ? el[id * heads + hs] + er[i * heads + hs] : 0.f;
+    const int64_t e0 = csc_indptr[i];
+    float go[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) go[q] = live ? d_out[i * row_len + d + q] : 0.f;
+    float my_part = 0.f;   // slot layout: dOut[i, hs] . ft[id, hs]
+    for (int u0 = 0; u0 < fanout; u0 += kUnroll) {
+      float v[kUnroll][VEC];
+      bool ok[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        ok[u] = false;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) v[u][q] = 0.f;
+        if (u0 + u < fanout) {
+          const int64_t src = wave_read(id, (u0 + u) << log2_heads);
+          if (src >= 0 && src < num_src) {
+            ok[u] = true;
+            if (live) load_vec<T, VEC>(ft, src * row_len + d, v[u]);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        if (!ok[u]) continue;  // the same in all lanes
+        float part = 0.f;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) part += go[q] * v[u][q];
+        for (int off = lph / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+        const float got = __shfl(part, hs * lph, kWave);   // the dot product of head hs
+        if (k == u0 + u) my_part = got;
+      }
+    }
+    // sums over the slots of a head: lanes j, j ^ heads, j ^ 2 heads, ...
+    float s = a * my_part;
+    for (int off = heads; off < kWave; off <<= 1) s += __shfl_xor(s, off, kWave);
+    const float dz = a * (my_part - s) * (z > 0.f ? 1.f : slope);
+    float sum_dz = dz;
+    for (int off = heads; off < kWave; off <<= 1) sum_dz += __shfl_xor(sum_dz, off, kWave);
+    // position of the slot's edge: e0 + number of valid slots before it
+    const uint64_t vm = ballot(valid && hs == 0);
+    const int first = k << log2_heads;
+    const int rank = __popcll(vm & (first == 0 ? 0ull : (~0ull >> (kWave - first))));
+    if (valid) {
+      const int64_t e = e0 + rank;
+      a_edge[e * heads + hs] = a;
+      dz_edge[e * heads + hs] = dz;
+    }
+    if (lane < heads) d_er[i * heads + lane] = sum_dz;   // lanes 0 .. heads-1 are (slot 0, head lane)
+  }
+}
+
+template <typename T, int VEC>
+static bool launch_gat_bwd_wave(const int64_t* nbr, int64_t num_dst, int fanout, const void* ft, int64_t num_src,
+                                int heads, int64_t dim, const float* el, const float* er, float slope,
+                                const float* attn, const float* d_out, const int64_t* csc_indptr, float* a_edge,
+                                float* dz_edge, float* d_er, hipStream_t st) {
+  if (dim % VEC != 0 || (heads & (heads - 1)) != 0 || heads * fanout > kWave) return false;
+  const int64_t lph = dim / VEC;
+  if ((lph & (lph - 1)) != 0 || heads * lph > kWave) return false;
+  if ((reinterpret_cast<uintptr_t>(ft) & 15) != 0) return false;
+  int log2_heads = 0;
+  while ((1 << log2_heads) < heads) ++log2_heads;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst, kAggWaves), 1 << 20));
+  hipLaunchKernelGGL((gat_bwd_edge_wave_kernel<T, VEC>), dim3(blocks), dim3(kAggBlock), 0, st, nbr, num_dst, fanout,
+                     static_cast<const T*>(ft), num_src, heads, log2_heads, dim, el, er, slope, attn, d_out,
+                     csc_indptr, a_edge, dz_edge, d_er);
+  return true;
+}
+
 template <typename T, int VEC>
 static bool launch_gat_bwd_group(const int64_t* nbr, int64_t num_dst, int fanout, const void* ft, int64_t num_src,
                                  int heads, int64_t dim, const float* el, const float* er, float slope,
@@ -926,6 +1024,16 @@ extern "C" int apt_gat_block_backward(const int64_t* neighbors, int64_t num_dst,
   const unsigned blocks =
       static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst * heads, kAggWaves), 1 << 20));
   hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool by_wave =
+      elem_size == 4 ? launch_gat_bwd_wave<float, 4>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,
+                                                     negative_slope, attn, d_out, csc_indptr, a_edge, dz_edge, d_er, st)
+                     : launch_gat_bwd_wave<uint16_t, 4>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,
+                                                        negative_slope, attn, d_out, csc_indptr, a_edge, dz_edge, d_er,
+                                                        st);
+  if (by_wave) {
+    APT_LAUNCH_CHECK("gat_bwd_edge_wave_kernel");
+    return APT_OK;
+  }
   const bool grouped =
       elem_size == 4
           ? launch_gat_bwd_group<float, 4>(neighbors, num_dst, fanout, ft, num_src, heads, dim, el, er,

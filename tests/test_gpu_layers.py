@@ -102,12 +102,13 @@ def _gat_dense(layer, blk, feat):
     return out + layer.bias.view(1, H, D)
 
 
-@pytest.mark.parametrize("heads,dim", [(3, 8), (4, 64), (1, 5), (2, 100)])
-def test_gat_layer_gradients(heads, dim):
+@pytest.mark.parametrize("heads,dim,fanout", [(3, 8, 9), (4, 64, 9), (1, 5, 9), (2, 100, 9),      # lane-group kernels
+                                              (4, 64, 16), (8, 8, 8), (1, 256, 15), (2, 16, 3)])    # wavefront per destination
+def test_gat_layer_gradients(heads, dim, fanout):
     import apt_amd as npc
     from apt_amd.layers import GATConv
     _setup_graph(seed=5)
-    sampler = npc.MixedPSNeighborSampler(0, 1, [9], "DP", replace=False, rng_seed=8)
+    sampler = npc.MixedPSNeighborSampler(0, 1, [fanout], "DP", replace=False, rng_seed=8)
     seeds = torch.from_numpy(np.random.default_rng(3).permutation(6000)[:300]).to(DEV)
     _, _, (blk,) = sampler.sample(None, seeds)
     torch.manual_seed(1)
@@ -125,7 +126,7 @@ def test_gat_layer_gradients(heads, dim):
         assert (a - b).abs().max().item() <= 2e-4 * scale, (name, (a - b).abs().max().item(), scale)
 
 
-@pytest.mark.parametrize("heads,dim", [(4, 64), (2, 16), (3, 24), (1, 40)])
+@pytest.mark.parametrize("heads,dim", [(4, 64), (2, 16), (3, 24), (1, 40), (8, 8), (1, 256)])
 def test_gat_backward_bf16_matches_fp32_on_rounded_inputs(capi, heads, dim):
     """bf16 features take other kernel variants (8 per lane); on the same (rounded)
     values they must give what the fp32 variants give."""
