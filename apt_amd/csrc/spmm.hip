@@ -472,6 +472,92 @@ __global__ __launch_bounds__(kAggBlock) void gat_ell_kernel(const int64_t* __res
   }
 }
 
+// The same layer with a wavefront per destination and two lane layouts (needs
+// heads and lph = dim / VEC to be powers of two, heads * lph <= 64 and
+// heads * fanout <= 64).  Slot layout: lane j is (slot j / heads, head
+// j % heads) and holds that slot's logit, so ids, el and the attention weights
+// are one coalesced access each per destination and the softmax is three
+// cross-lane reductions.  Feature layout: lane l holds VEC features of head
+// l / lph and adds up the source rows, fetching each slot's weight from the slot
+// layout with one shuffle.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kAggBlock) void gat_ell_wave_kernel(
+    const int64_t* __restrict__ nbr, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+    const T* __restrict__ ft, int64_t num_src, int heads, int log2_heads, int64_t dim,
+    const float* __restrict__ el, const float* __restrict__ er, float slope, float* __restrict__ out,
+    float* __restrict__ attn_out) {
+  constexpr int kUnroll = 5;
+  const int64_t n = actual_count(num_dst, num_dst_dev);
+  const int lane = threadIdx.x % kWave;
+  const int lph = static_cast<int>(dim / VEC);
+  const int64_t row_len = static_cast<int64_t>(heads) * dim;
+  const bool live = lane < heads * lph;
+  const int hf = live ? lane / lph : 0;
+  const int64_t d = static_cast<int64_t>(lane) * VEC;
+  const int k = lane >> log2_heads, hs = lane & (heads - 1);
+  const bool slot = k < fanout;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kAggWaves) {
+    const int64_t id = slot ? nbr[i * fanout + k] : -1;
+    const bool valid = id >= 0 && id < num_src;
+    float e = -INFINITY;
+    if (valid) {
+      e = el[id * heads + hs] + er[i * heads + hs];
+      e = e > 0.f ? e : e * slope;
+    }
+    float top = e;
+    for (int off = heads; off < kWave; off <<= 1) top = fmaxf(top, __shfl_xor(top, off, kWave));
+    const float w = valid ? expf(e - top) : 0.f;
+    float denom = w;
+    for (int off = heads; off < kWave; off <<= 1) denom += __shfl_xor(denom, off, kWave);
+    const float a = denom > 0.f ? w / denom : 0.f;
+    if (attn_out != nullptr && slot) attn_out[(i * fanout + k) * heads + hs] = a;
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    for (int u0 = 0; u0 < fanout; u0 += kUnroll) {
+      float v[kUnroll][VEC];
+      float au[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        au[u] = 0.f;
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) v[u][q] = 0.f;
+        if (u0 + u < fanout) {
+          const int64_t src = wave_read(id, (u0 + u) << log2_heads);
+          if (src >= 0 && src < num_src) {
+            au[u] = __shfl(a, ((u0 + u) << log2_heads) + hf, kWave);
+            if (live) load_vec<T, VEC>(ft, src * row_len + d, v[u]);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int q = 0; q < VEC; ++q) acc[q] += au[u] * v[u][q];
+    }
+    if (live) {
+#pragma unroll
+      for (int q = 0; q < VEC; ++q) out[i * row_len + d + q] = acc[q];
+    }
+  }
+}
+
+template <typename T, int VEC>
+static bool launch_gat_wave(const int64_t* nbr, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
+                            const void* ft, int64_t num_src, int heads, int64_t dim, const float* el,
+                            const float* er, float slope, float* out, float* attn_out, hipStream_t st) {
+  if (dim % VEC != 0 || (heads & (heads - 1)) != 0 || heads * fanout > kWave) return false;
+  const int64_t lph = dim / VEC;
+  if ((lph & (lph - 1)) != 0 || heads * lph > kWave) return false;
+  int log2_heads = 0;
+  while ((1 << log2_heads) < heads) ++log2_heads;
+  const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_dst, kAggWaves), 1 << 20));
+  hipLaunchKernelGGL((gat_ell_wave_kernel<T, VEC>), dim3(blocks), dim3(kAggBlock), 0, st, nbr, num_dst, num_dst_dev,
+                     fanout, static_cast<const T*>(ft), num_src, heads, log2_heads, dim, el, er, slope, out, attn_out);
+  return true;
+}
+
 template <typename T, int VEC>
 static void launch_gat(const int64_t* nbr, int64_t num_dst, const int64_t* num_dst_dev, int fanout,
                        const void* ft, int64_t num_src, int heads, int64_t dim, const float* el,
@@ -942,6 +1028,14 @@ extern "C" int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const in
   hipStream_t st = static_cast<hipStream_t>(stream);
   const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(ft) & 15) == 0 &&
                     (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (vec4 && num_src > 0 &&
+      (elem_size == 4 ? launch_gat_wave<float, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el,
+                                                  er, negative_slope, out, attn_out, st)
+                      : launch_gat_wave<uint16_t, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim,
+                                                     el, er, negative_slope, out, attn_out, st))) {
+    APT_LAUNCH_CHECK("gat_ell_wave_kernel");
+    return APT_OK;
+  }
   if (elem_size == 4) {
     if (vec4) launch_gat<float, 4>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
     else launch_gat<float, 1>(neighbors, num_dst, num_dst_dev, fanout, ft, num_src, heads, dim, el, er, negative_slope, out, attn_out, st);
