@@ -289,7 +289,17 @@ __global__ __launch_bounds__(kAggBlock) void spmm_ell_kernel(const int64_t* __re
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * kGroups + grp; i < n;
        i += static_cast<int64_t>(gridDim.x) * kGroups) {
     const int64_t* ids = nbr + i * fanout;
-    for (int64_t d = static_cast<int64_t>(l) * VEC; d < dim; d += LPR * VEC) {
+    // lane s of the group fetches slot s's id (one coalesced load for the destination); the slot loop reads
+    // it with a shuffle.  (Ids that do not fit 32 bits, or more slots than lanes: every lane loads them itself.)
+    const bool shared_ids = fanout <= LPR && num_src <= 0x7fffffffLL;
+    int my_id = -1;
+    if (shared_ids && l < fanout) {
+      const int64_t v = ids[l];
+      my_id = (v >= 0 && v < num_src) ? static_cast<int>(v) : -1;
+    }
+    for (int64_t d0 = 0; d0 < dim; d0 += LPR * VEC) {   // every lane of the group stays in the loop (shuffles)
+      const int64_t d = d0 + static_cast<int64_t>(l) * VEC;
+      const bool live = d < dim;
       float acc[VEC];
 #pragma unroll
       for (int k = 0; k < VEC; ++k) acc[k] = 0.f;
@@ -301,9 +311,9 @@ __global__ __launch_bounds__(kAggBlock) void spmm_ell_kernel(const int64_t* __re
 #pragma unroll
           for (int k = 0; k < VEC; ++k) v[u][k] = 0.f;
           if (s0 + u < fanout) {
-            const int64_t src = ids[s0 + u];
+            const int64_t src = shared_ids ? static_cast<int64_t>(__shfl(my_id, s0 + u, LPR)) : ids[s0 + u];
             if (src >= 0 && src < num_src) {
-              load_vec<T, VEC>(x, src * dim + d, v[u]);
+              if (live) load_vec<T, VEC>(x, src * dim + d, v[u]);
               ++cnt;
             }
           }
@@ -314,8 +324,10 @@ __global__ __launch_bounds__(kAggBlock) void spmm_ell_kernel(const int64_t* __re
           for (int k = 0; k < VEC; ++k) acc[k] += v[u][k];
       }
       const float scale = (mean && cnt > 0) ? 1.0f / static_cast<float>(cnt) : 1.0f;
+      if (live) {
 #pragma unroll
-      for (int k = 0; k < VEC; ++k) out[i * dim + d + k] = acc[k] * scale;
+        for (int k = 0; k < VEC; ++k) out[i * dim + d + k] = acc[k] * scale;
+      }
     }
   }
 }
