@@ -549,6 +549,25 @@ def main():
             e1, b1, t1s = cpu_leg(budget * 0.25, cpu_batches)
             one = dict(value=e1 / t1s, batches=b1, seconds=t1s)
             orc.set_threads(threads)
+        # the gather stage alone, as the reference states it on the CPU (src/load_subtensor.cc:10-17: torch's
+        # index_select over the host table), on the input nodes of one batch
+        gather_cpu = None
+        if requests is None:
+            inp, _ = orc.sample_blocks(og, h_seeds[0], hops, args.replace, args.seed + 100 + W)
+            table = torch.from_numpy(h_feats.view(np.int16) if dtype == torch.bfloat16 else h_feats)
+            ids_t = torch.from_numpy(inp)
+            torch.set_num_threads(threads)
+            table.index_select(0, ids_t[:1000])
+            t1 = time.perf_counter()
+            reps = 0
+            while time.perf_counter() - t1 < 1.0:
+                table.index_select(0, ids_t)
+                reps += 1
+            tg = (time.perf_counter() - t1) / reps
+            gather_cpu = dict(GBps=len(inp) * bytes_per_row / tg / 1e9, ms=tg * 1e3, rows=int(len(inp)),
+                              what="torch.index_select on the host table (the reference's CPU gather), "
+                                   f"{threads} threads")
+            del table, ids_t
         model = ""
         try:
             model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
@@ -558,7 +577,7 @@ def main():
                    sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
                           f"with fresh rng keys) in {tc:.1f} s: sampling, relabel and gather on {threads} "
                           f"OpenMP threads",
-                   one_thread=one, host_cpu=model, host_logical_cpus=os.cpu_count())
+                   one_thread=one, gather_stage=gather_cpu, host_cpu=model, host_logical_cpus=os.cpu_count())
         del h_indices, h_feats, og, ofs
 
     out = {
