@@ -48,7 +48,8 @@ SYMBOLS = {
     "apt_gather_rows": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P]),
     "apt_time_next_gather": (_I, [_P, _P]),
     "apt_permute_rows": (_I, [_P, _I64, _P, _I64, _I64, _I, _P, _P]),
-    "apt_scatter_rows": (_I, [_P, _P, _I64, _I64, _I, _P, _I64, _P]),
+    "apt_scatter_workspace_bytes": (C.c_size_t, [_I64]),
+    "apt_scatter_rows": (_I, [_P, _P, _I64, _I64, _I, _P, _I64, _P, C.c_size_t, _P]),
     "apt_bucket_workspace_bytes": (_SZ, [_I64, _I]),
     "apt_cluster_permute": (_I, [_P, _I64, _P, _P, _I, _I64, _I, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_cluster_reqs": (_I, [_P, _I64, _P, _P, _I64, _P, _P, _I, _I, _P, _P, _P, _P, _P, _SZ, _P]),
@@ -282,10 +283,14 @@ def scatter_rows(table, perm, num_out_rows=None, out=None):
         raise AptError(f"scatter_rows: {table.shape[0]} rows but {n} destinations")
     if num_out_rows is None:
         num_out_rows = n
-    if out is None:
-        out = torch.zeros((num_out_rows, table.shape[1]), dtype=table.dtype, device=table.device)
+    ws = None
+    if out is None:   # rows nobody names are flagged by the scatter and zeroed afterwards: no fill of the whole output
+        out = torch.empty((num_out_rows, table.shape[1]), dtype=table.dtype, device=table.device)
+        ws = torch.empty(int(lib().apt_scatter_workspace_bytes(int(num_out_rows))), dtype=torch.uint8,
+                         device=table.device)
     check(lib().apt_scatter_rows(_ptr(table), _ptr(perm), n, table.shape[1], table.element_size(),
-                                 _ptr(out), int(num_out_rows), _stream()))
+                                 _ptr(out), int(num_out_rows), _ptr(ws), ws.numel() if ws is not None else 0,
+                                 _stream()))
     return out
 
 

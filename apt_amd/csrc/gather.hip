@@ -35,6 +35,7 @@ struct GatherParams {
   int64_t* miss_count;
   int scatter;               // 1: out[index[r]] = in[r] (pack); rows come from local_table
   int64_t num_out_rows;      // scatter only
+  uint8_t* named;            // scatter only, optional: named[v] = 1 for every output row v that is written
 };
 
 template <int V> struct VecT;
@@ -91,6 +92,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
           if (v >= 0 && v < p.num_out_rows) {
             src[k] = p.local_table + r * p.out_row_bytes;
             dst[k] = p.out + v * p.out_row_bytes;
+            if (p.named != nullptr && l == 0) p.named[v] = 1;
           }
         } else {
           src[k] = source_row(p, v);
@@ -250,6 +252,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.miss_count = miss_count;
   p.scatter = 0;
   p.num_out_rows = 0;
+  p.named = nullptr;
   arm.rearm();
   return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
 }
@@ -262,7 +265,7 @@ extern "C" int apt_time_next_gather(void* start_event, void* stop_event) {
 
 static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_t dim,
                           int elem_size, void* out, int scatter, int64_t num_rows_other,
-                          void* stream, const char* who) {
+                          void* stream, const char* who, uint8_t* named = nullptr) {
   using namespace apt;
   const TimingArm arm;
   APT_REQUIRE(n >= 0 && dim > 0, APT_EINVAL, "%s: bad shape (n %lld, dim %lld)", who,
@@ -289,6 +292,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
   p.miss_count = nullptr;
   p.scatter = scatter;
   p.num_out_rows = scatter ? num_rows_other : 0;
+  p.named = named;
   arm.rearm();
   return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
 }
@@ -301,10 +305,64 @@ extern "C" int apt_permute_rows(const void* in, int64_t num_in_rows, const int64
                         "apt_permute_rows");
 }
 
+namespace apt {
+
+__global__ __launch_bounds__(kGatherBlock) void zero_words_kernel(uint32_t* w, int64_t n) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kGatherBlock + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kGatherBlock)
+    w[i] = 0;
+}
+
+// rows whose flag is clear are zeroed, 16 lanes per row, 2 bytes per store (such rows are rare)
+__global__ __launch_bounds__(kGatherBlock) void zero_unnamed_kernel(const uint8_t* __restrict__ named,
+                                                                    int64_t num_rows, char* out, int64_t row_bytes) {
+  constexpr int kLanes = 16;
+  const int l = threadIdx.x % kLanes;
+  for (int64_t r = (static_cast<int64_t>(blockIdx.x) * kGatherBlock + threadIdx.x) / kLanes; r < num_rows;
+       r += static_cast<int64_t>(gridDim.x) * (kGatherBlock / kLanes)) {
+    if (named[r] != 0) continue;
+    uint16_t* row = reinterpret_cast<uint16_t*>(out + r * row_bytes);
+    for (int64_t c = l; c < row_bytes / 2; c += kLanes) row[c] = 0;
+  }
+}
+
+}  // namespace apt
+
+extern "C" size_t apt_scatter_workspace_bytes(int64_t num_out_rows) {
+  if (num_out_rows < 0) return 0;
+  return (static_cast<size_t>(num_out_rows) + 3) / 4 * 4 + 4;
+}
+
 extern "C" int apt_scatter_rows(const void* in, const int64_t* perm, int64_t n, int64_t dim,
-                                int elem_size, void* out, int64_t num_out_rows, void* stream) {
+                                int elem_size, void* out, int64_t num_out_rows, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  using namespace apt;
   APT_REQUIRE(num_out_rows >= 0, APT_EINVAL, "apt_scatter_rows: num_out_rows %lld < 0",
               (long long)num_out_rows);
-  return permute_common(in, perm, n, dim, elem_size, out, 1, num_out_rows, stream,
-                        "apt_scatter_rows");
+  if (workspace == nullptr)
+    return permute_common(in, perm, n, dim, elem_size, out, 1, num_out_rows, stream, "apt_scatter_rows");
+  // with scratch the library completes the output itself: a flag per output row, set by the scatter,
+  // tells which rows nobody named; only those are zeroed
+  APT_REQUIRE(workspace_bytes >= apt_scatter_workspace_bytes(num_out_rows) &&
+                  (reinterpret_cast<uintptr_t>(workspace) & 3) == 0,
+              APT_EWORKSPACE, "apt_scatter_rows: workspace too small or not 4-byte aligned "
+                              "(see apt_scatter_workspace_bytes)");
+  APT_REQUIRE(dim > 0 && (elem_size == 2 || elem_size == 4) && (out != nullptr || num_out_rows == 0), APT_EINVAL,
+              "apt_scatter_rows: bad shape or out is NULL");
+  if (num_out_rows == 0) return APT_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint8_t* named = static_cast<uint8_t*>(workspace);
+  const int64_t words = (num_out_rows + 3) / 4;
+  auto blocks_for = [](int64_t items) {
+    return dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(items, kGatherBlock), 4096))));
+  };
+  hipLaunchKernelGGL(zero_words_kernel, blocks_for(words), dim3(kGatherBlock), 0, st,
+                     reinterpret_cast<uint32_t*>(named), words);
+  APT_LAUNCH_CHECK("zero_words_kernel");
+  const int rc = permute_common(in, perm, n, dim, elem_size, out, 1, num_out_rows, stream, "apt_scatter_rows", named);
+  if (rc != APT_OK) return rc;
+  hipLaunchKernelGGL(zero_unnamed_kernel, blocks_for(num_out_rows * 16), dim3(kGatherBlock), 0, st, named,
+                     num_out_rows, static_cast<char*>(out), dim * elem_size);
+  APT_LAUNCH_CHECK("zero_unnamed_kernel");
+  return APT_OK;
 }

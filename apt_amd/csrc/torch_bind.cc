@@ -515,9 +515,13 @@ Tensor FeatShuffle(Tensor inputs, Tensor send_offset, Tensor recv_offset, Tensor
     return out;
   }
   TORCH_CHECK(perm.numel() == x.size(0), "npc: permutation must name every input row");
-  auto out = torch::zeros({n_out, feat_dim}, x.options());
-  check(apt_scatter_rows(x.data_ptr(), i64(perm), perm.numel(), feat_dim,
-                         static_cast<int>(x.element_size()), out.data_ptr(), n_out, stream()));
+  // rows that no permutation entry names (none when it is a bijection, as ShuffleSeeds makes it) are flagged by
+  // the scatter and zeroed afterwards: cheaper than zero-filling the whole output first
+  auto out = torch::empty({n_out, feat_dim}, x.options());
+  auto ws = torch::empty({static_cast<int64_t>(apt_scatter_workspace_bytes(n_out))},
+                         torch::TensorOptions().dtype(torch::kUInt8).device(device()));
+  check(apt_scatter_rows(x.data_ptr(), i64(perm), perm.numel(), feat_dim, static_cast<int>(x.element_size()),
+                         out.data_ptr(), n_out, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream()));
   return out;
 }
 

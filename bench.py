@@ -73,6 +73,9 @@ def parse_args():
     ap.add_argument("--aggregation", action="store_true",
                     help="also time GraphSAGE-style SpMM (hidden 256, fp32 and bf16) and SDDMM on the "
                          "outermost sampled block of the last batch")
+    ap.add_argument("--shuffle", action="store_true",
+                    help="also time the local halves of the feature shuffle on the batch's input nodes: bucketing by "
+                         "owner (cluster_permute) and pack / unpack of hidden rows")
     ap.add_argument("--cache_build", action="store_true",
                     help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
                          "cached feature table) and one step of the all-strategies dry run")
@@ -448,6 +451,39 @@ def main():
             fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
             del fp
 
+    # ---- optional: bucketing by owner and pack / unpack of hidden rows (the local halves of feat_shuffle)
+    shuffle = None
+    if args.shuffle:
+        def ms_of(fn, reps=10):
+            for _ in range(3):
+                fn()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps
+
+        stage_pipe.run(seed_sets[W], args.seed + 100 + W)
+        torch.cuda.synchronize()
+        H = len(hops)
+        n_in = int(stage_pipe.sizes[H].item())
+        ids = stage_pipe.nodes[:n_in].contiguous()
+        world, hid = 8, 256
+        mv = torch.linspace(0, N, world + 1).to(torch.int64).to(dev)
+        t_bucket = ms_of(lambda: capi.cluster_permute(ids, mv, world))
+        _, _, _, perm = capi.cluster_permute(ids, mv, world)
+        hrows = torch.randn(n_in, hid, device=dev)
+        t_unpack = ms_of(lambda: capi.permute_rows(hrows, perm))
+        t_pack = ms_of(lambda: capi.scatter_rows(hrows, perm))
+        row_bytes = 2 * hid * 4 + 8
+        shuffle = {"ids": n_in, "owners": world, "hidden": hid,
+                   "cluster_permute_us": t_bucket * 1e3, "cluster_permute_GBps": 24.0 * n_in / (t_bucket * 1e-3) / 1e9,
+                   "unpack_us": t_unpack * 1e3, "unpack_GBps": n_in * row_bytes / (t_unpack * 1e-3) / 1e9,
+                   "pack_us": t_pack * 1e3, "pack_GBps": n_in * row_bytes / (t_pack * 1e-3) / 1e9}
+        del hrows, perm, ids
+
     # ---- optional: cache construction and the strategy dry run (the callers of the registries)
     cache_build = None
     if args.cache_build and requests is None:
@@ -621,6 +657,7 @@ def main():
         "aggregation": agg,
         "block_formats": fmt,
         "cache_build": cache_build,
+        "shuffle": shuffle,
         "stages": {
             "in_flight": in_flight,
             "edges_per_step": edges / K,

@@ -199,14 +199,19 @@ int apt_time_next_gather(void* start_event, void* stop_event);
  *   pack   (bwd):  out[perm[i], :] = in[i, :], i < n   (index_select_backward
  *                  of a bijection, :14-16); rows of out that no perm[i] names
  *                  are left untouched, so the caller zero-fills out first when
- *                  perm is not onto; a perm[i] outside [0, num_out_rows) is
- *                  skipped. */
+ *                  perm is not onto -- or passes workspace
+ *                  (apt_scatter_workspace_bytes(num_out_rows) bytes, 4-byte
+ *                  aligned; NULL = none): the scatter then flags the rows it
+ *                  writes and the library zeroes exactly the others, far cheaper
+ *                  than a fill of wide rows; a perm[i] outside [0, num_out_rows)
+ *                  is skipped. */
 int apt_permute_rows(const void* in, int64_t num_in_rows, const int64_t* perm,
                      int64_t n, int64_t dim, int elem_size, void* out,
                      void* stream);
+size_t apt_scatter_workspace_bytes(int64_t num_out_rows);
 int apt_scatter_rows(const void* in, const int64_t* perm, int64_t n,
                      int64_t dim, int elem_size, void* out, int64_t num_out_rows,
-                     void* stream);
+                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* Stable bucketing of ids by owner.
  * Replaces ClusterAndPermute (src/cuda/npc_kernel.cu:318-382,434-470), the

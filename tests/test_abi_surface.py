@@ -62,6 +62,8 @@ def test_argument_checks_need_no_gpu():
     assert L.apt_vir_send_offset(0, 5, None, 0, None, 0, 0, None, None) != 0
     assert L.apt_spmm_block(None, 5, None, 0, None, 5, 8, 4, 0, None, None) != 0
     assert L.apt_coo_is_grouped(None, 5, None, None) != 0
+    assert L.apt_scatter_workspace_bytes(64) == 68 and L.apt_scatter_workspace_bytes(65) == 72
+    assert L.apt_scatter_rows(None, None, 3, 8, 4, None, 5, None, 0, None) != 0
     assert L.apt_spmm_heads(None, None, 5, None, 5, None, None, 3, 8, 4, 1, None, 5, None, None, None, None) != 0
     assert b"heads" in L.apt_last_error()
     for key in (b"sample_min_workgroups", b"gather_vector_bytes", b"block_fused_scan"):

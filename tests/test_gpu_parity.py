@@ -275,6 +275,20 @@ def test_permute_scatter_rows(orc, capi):
         assert np.array_equal(as_np(up), orc.permute_rows(x, perm))
         assert np.array_equal(as_np(pk), orc.scatter_rows(x, perm))
         assert np.array_equal(as_np(capi.permute_rows(pk, dev(perm))), x)       # round trip
+    # pack into more rows than are named (some ids out of range): the rows nobody names come back zero,
+    # on memory that held something else before
+    for dim, dtype in [(5, torch.float32), (256, torch.float32), (7, torch.bfloat16), (64, torch.bfloat16)]:
+        x = _rand_table(rng, 3000, dim, dtype)
+        dest = rng.permutation(5000)[:3000]
+        dest[[4, 77]] = [-1, 5000]
+        junk = torch.full((5000, dim), 3.0, device=DEV).to(dtype)     # recycled by the allocator below
+        del junk
+        pk = capi.scatter_rows(_to_dev_table(x, dtype), dev(dest), num_out_rows=5000)
+        as_np = lambda t: host(t.view(torch.int16) if dtype == torch.bfloat16 else t).view(x.dtype)
+        want = np.zeros((5000, dim), dtype=x.dtype)
+        ok = (dest >= 0) & (dest < 5000)
+        want[dest[ok]] = x[ok]
+        assert np.array_equal(as_np(pk), want), (dim, dtype)
     # un-unique gather: more outputs than inputs
     inv = rng.integers(0, 100, size=999)
     x = rng.standard_normal((100, 32)).astype(np.float32)
