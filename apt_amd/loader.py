@@ -15,13 +15,15 @@ from .pipeline import MiniBatchPipeline
 
 class MiniBatchLoader:
     def __init__(self, graph, feat, indices, batch_size, hop_fanouts, in_flight=4, shuffle=True, drop_last=True,
-                 replace=False, seed=0, formats=False, requests=None):
+                 replace=False, seed=0, formats=False, requests=None, use_graph=False):
         """indices: node ids to draw seeds from (the training ids).  hop_fanouts
         start from the seeds.  Yields MiniBatchPipeline.result() dicts with
         `output_nodes` (the batch's seeds) added.  A yielded batch lives in its
         pipeline's buffers: it stays valid until the loader is asked for the next
         one, and work the consumer has enqueued on its current stream by then is
-        waited for before the buffers are reused."""
+        waited for before the buffers are reused.  use_graph: every pipeline
+        replays a captured HIP graph, which costs the host less per batch (worth it
+        for small batches, where the host's launch calls are the limit)."""
         if in_flight < 1:
             raise ValueError("in_flight must be >= 1")
         dev = graph.device
@@ -34,7 +36,7 @@ class MiniBatchLoader:
         self.tail = 0 if drop_last else n - self.num_full * self.batch_size
         if self.num_full + (1 if self.tail else 0) == 0:
             raise ValueError(f"{n} indices give no batch of {self.batch_size}")
-        kw = dict(replace=replace, formats=formats, requests=requests)
+        kw = dict(replace=replace, formats=formats, requests=requests, use_graph=use_graph)
         self._make = lambda b: MiniBatchPipeline(graph, feat, b, hop_fanouts, **kw)
         self.pipes = [self._make(self.batch_size) for _ in range(min(in_flight, max(self.num_full, 1)))]
         self.streams = [torch.cuda.Stream(device=dev) for _ in self.pipes]

@@ -16,9 +16,10 @@ def _setup(capi, n=30000, dim=32):
     return g, capi.FeatStore(table), table
 
 
-@pytest.mark.parametrize("in_flight,drop_last,formats", [(1, True, False), (3, True, "csc"), (4, False, False),
-                                                         (8, False, True)])
-def test_loader_matches_single_pipeline(capi, in_flight, drop_last, formats):
+@pytest.mark.parametrize("in_flight,drop_last,formats,use_graph", [(1, True, False, False), (3, True, "csc", False),
+                                                                   (4, False, False, False), (8, False, True, False),
+                                                                   (3, False, False, True)])
+def test_loader_matches_single_pipeline(capi, in_flight, drop_last, formats, use_graph):
     import torch
 
     from apt_amd.loader import MiniBatchLoader
@@ -27,7 +28,7 @@ def test_loader_matches_single_pipeline(capi, in_flight, drop_last, formats):
     ids = torch.from_numpy(np.random.default_rng(0).choice(30000, 1100, replace=False)).cuda()
     B, hops = 256, [3, 4]
     loader = MiniBatchLoader(g, store, ids, B, hops, in_flight=in_flight, shuffle=True, drop_last=drop_last, seed=5,
-                             formats=formats)
+                             formats=formats, use_graph=use_graph)
     assert len(loader) == (4 if drop_last else 5)
     ref = {B: MiniBatchPipeline(g, store, B, hops)}
     if not drop_last:
