@@ -233,3 +233,70 @@ def test_spmm_heads_owns_its_rows(orc, capi, heads, hd):
     assert _close(plain.cpu().numpy().reshape(rows, -1), orc.spmm_csr(indptr, row, x.reshape(n_x, -1)), 1e-5)
     with pytest.raises(capi.AptError):
         capi.spmm_heads(dev(row), dev(col), dev(x), None, rows, grouped=False, out_indptr=dev(indptr))
+
+
+def test_gat_random_shapes(orc, capi):
+    """Forty random (heads, head_dim, fanout) shapes on both sides of what a wavefront
+    per destination can hold (heads a power of two, heads x fanout <= 64, lanes per
+    head a power of two): forward and attention weights against the oracle, fp32 and
+    bf16, and empty destinations."""
+    rng = np.random.default_rng(99)
+    for case in range(40):
+        heads = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        dim = int(rng.choice([4, 8, 12, 16, 32, 64, 128, 20]))
+        fanout = int(rng.choice([1, 2, 3, 4, 8, 15, 16, 17, 32, 33]))
+        n_dst, n_src = 700, 3000
+        nbr = _ell(rng, n_dst, fanout, n_src)
+        nbr.reshape(n_dst, fanout)[5] = -1                       # a destination without neighbours
+        bf16 = case % 3 == 2
+        ft = rng.standard_normal((n_src, heads, dim)).astype(np.float32)
+        ft_t = dev(ft).to(torch.bfloat16) if bf16 else dev(ft)
+        ft_ref = ft_t.float().cpu().numpy()
+        el = rng.standard_normal((n_src, heads)).astype(np.float32)
+        er = rng.standard_normal((n_dst, heads)).astype(np.float32)
+        want, want_a = orc.gat_block(nbr, n_dst, fanout, ft_ref, el, er, 0.2, want_attn=True)
+        got, got_a = capi.gat_block(dev(nbr), n_dst, fanout, ft_t, dev(el), dev(er), 0.2, want_attn=True)
+        tol = 1e-2 if bf16 else 1e-5
+        assert _close(got.cpu().numpy(), want, tol), (case, heads, dim, fanout, bf16)
+        assert np.max(np.abs(got_a.cpu().numpy() - want_a)) <= 1e-5, (case, heads, dim, fanout)
+        assert not got[5].any()
+
+
+def test_gat_backward_random_shapes(capi):
+    """apt_gat_block_backward against the same arithmetic written with dense torch ops on the
+    fixed-stride layout (float64), for shapes on both sides of the wavefront-per-destination
+    kernel's limits; fp32 and bf16 features."""
+    rng = np.random.default_rng(123)
+    for case in range(30):
+        heads = int(rng.choice([1, 2, 3, 4, 8]))
+        dim = int(rng.choice([4, 8, 16, 64, 20, 128]))
+        fanout = int(rng.choice([1, 3, 8, 15, 16, 17, 33]))
+        n_dst, n_src = 500, 2000
+        nbr = _ell(rng, n_dst, fanout, n_src).reshape(n_dst, fanout)
+        nbr[7] = -1
+        bf16 = case % 3 == 2
+        ft = dev(rng.standard_normal((n_src, heads, dim)).astype(np.float32))
+        if bf16:
+            ft = ft.to(torch.bfloat16)
+        el = dev(rng.standard_normal((n_src, heads)).astype(np.float32))
+        er = dev(rng.standard_normal((n_dst, heads)).astype(np.float32))
+        d_out = dev(rng.standard_normal((n_dst, heads, dim)).astype(np.float32))
+        nb = dev(nbr.reshape(-1))
+        _, attn = capi.gat_block(nb, n_dst, fanout, ft, el, er, 0.2, want_attn=True)
+        fmt = capi.block_formats(nb, n_dst, fanout, n_src, want_csr=False)
+        a_edge, dz_edge, d_er = capi.gat_block_backward(nb, n_dst, fanout, ft, el, er, 0.2, attn, d_out,
+                                                        fmt["csc_indptr"], fmt["num_edges"])
+        # dense statement
+        nbt = dev(nbr)
+        valid = nbt >= 0
+        idx = nbt.clamp(min=0)
+        ftn = ft.double()[idx]                                                    # [n_dst, fanout, H, D]
+        part = (d_out.double()[:, None] * ftn).sum(-1) * valid[..., None]         # [n_dst, fanout, H]
+        a = attn.double().view(n_dst, fanout, heads)
+        s = (a * part).sum(1, keepdim=True)
+        z = el.double()[idx] + er.double()[:, None]
+        dz = a * (part - s) * torch.where(z > 0, 1.0, 0.2) * valid[..., None]
+        tol = dict(rtol=1e-4, atol=1e-4)
+        assert torch.allclose(d_er.double(), dz.sum(1), **tol), (case, heads, dim, fanout, bf16)
+        assert torch.allclose(a_edge.double(), a[valid], **tol), (case, heads, dim, fanout, bf16)
+        assert torch.allclose(dz_edge.double(), dz[valid], **tol), (case, heads, dim, fanout, bf16)
