@@ -18,6 +18,14 @@
  *   "not present".  In id arrays a negative id is padding: it has no
  *   neighbours, is not relabelled and stays negative in outputs.
  *
+ * What the host can check (null pointers, sizes, alignment, workspace) is
+ * checked before anything is launched.  Values that live in device memory are
+ * checked by the kernels where an entry point's comment says what happens to a
+ * value out of range (ids and positions: treated as padding, counted as misses
+ * or skipped); the CSR arrays of a graph (indptr non-decreasing and within
+ * indices) and index arrays that address a caller's side table (weight_row,
+ * eids) are taken on trust, as the reference takes all of its inputs.
+ *
  * Each entry point cites the reference interface it replaces.
  */
 #ifndef APT_AMD_H_
