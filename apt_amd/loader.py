@@ -15,7 +15,7 @@ from .pipeline import MiniBatchPipeline
 
 class MiniBatchLoader:
     def __init__(self, graph, feat, indices, batch_size, hop_fanouts, in_flight=4, shuffle=True, drop_last=True,
-                 replace=False, seed=0, formats=False, requests=None, use_graph=False):
+                 replace=False, seed=0, formats=False, requests=None, use_graph=False, as_blocks=False):
         """indices: node ids to draw seeds from (the training ids).  hop_fanouts
         start from the seeds.  Yields MiniBatchPipeline.result() dicts with
         `output_nodes` (the batch's seeds) added.  A yielded batch lives in its
@@ -23,7 +23,8 @@ class MiniBatchLoader:
         one, and work the consumer has enqueued on its current stream by then is
         waited for before the buffers are reused.  use_graph: every pipeline
         replays a captured HIP graph, which costs the host less per batch (worth it
-        for small batches, where the host's launch calls are the limit)."""
+        for small batches, where the host's launch calls are the limit).  as_blocks:
+        batch["blocks"] are sampler.Block objects, ready for apt_amd.layers."""
         if in_flight < 1:
             raise ValueError("in_flight must be >= 1")
         dev = graph.device
@@ -43,6 +44,7 @@ class MiniBatchLoader:
         self.done = [torch.cuda.Event() for _ in self.pipes]
         self.released = [torch.cuda.Event() for _ in self.pipes]
         self.tail_pipe = self._make(self.tail) if self.tail else None     # the short last batch has buffers of its own
+        self.as_blocks = bool(as_blocks)
         self.epoch = 0
 
     def __len__(self):
@@ -87,7 +89,7 @@ class MiniBatchLoader:
             cur = torch.cuda.current_stream(self.device)
             cur.wait_event(self.done[k])
             self.done[k].synchronize()                     # the sizes are in pinned host memory now
-            out = owner.pop(i).result(staged=True)
+            out = owner.pop(i).result(staged=True, as_blocks=self.as_blocks)
             out["output_nodes"] = batches[i]
             yield out
             if i + F < len(batches):

@@ -213,10 +213,14 @@ class MiniBatchPipeline:
         if self.requests is not None:
             self.request_sizes_host.copy_(self.request_sizes, non_blocking=True)
 
-    def result(self, staged=False):
+    def result(self, staged=False, as_blocks=False):
         """Waits for the batch and narrows the buffers to their real sizes ->
         dict(input_nodes, blocks (outermost first), features, num_edges).
-        staged: the sizes were copied by stage_sizes() and that copy has finished."""
+        staged: the sizes were copied by stage_sizes() and that copy has finished.
+        as_blocks: the blocks come as sampler.Block objects (what the layers of
+        apt_amd.layers take) instead of dicts; they live in this pipeline's buffers
+        like everything else, so a training step must finish with them before the
+        pipeline runs its next batch."""
         sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
         H = len(self.fanouts)
         blocks = []
@@ -232,6 +236,10 @@ class MiniBatchPipeline:
                                   unique=uniq, fanout=f))
             if self.formats is not None:
                 blocks[0]["formats"] = self.formats[h].narrow(num_dst=n, num_src=sizes[h + 1])
+            if as_blocks:
+                from .sampler import Block
+                b = blocks[0]
+                blocks[0] = Block(sizes[h + 1], n, uniq, b["relabeled"], f, b.get("formats"))
         feats = None if self.features is None else self.features[:sizes[H]]
         inp = self.nodes[:sizes[H]] if self.fused else self.frontier[H][:sizes[H]]
         out = dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],

@@ -81,3 +81,45 @@ def test_loader_without_shuffle_and_early_exit(capi):
     assert torch.equal(torch.cat(out), ids)
     with pytest.raises(ValueError):
         MiniBatchLoader(g, store, ids[:10], 128, [5])
+
+
+@pytest.mark.parametrize("formats", [False, True])
+def test_training_loop_on_the_loader(capi, formats):
+    """The loader's batches as Block objects feed apt_amd.layers directly: two SAGE
+    layers trained on them learn a label that needs the neighbourhood; with formats=True
+    the blocks arrive with COO / CSC / CSR already emitted beside the gather."""
+    import torch
+
+    from apt_amd import synth
+    from apt_amd.layers import SAGEConv
+    from apt_amd.loader import MiniBatchLoader
+    from apt_amd.sampler import Block
+    n = 4000
+    indptr, indices = synth.rmat_csr_numpy(n, n * 10, seed=2)
+    g = capi.Graph(torch.from_numpy(indptr).cuda(), torch.from_numpy(indices).cuda())
+    gen = torch.Generator().manual_seed(0)
+    feats = torch.randn(n, 16, generator=gen)
+    deg = np.diff(indptr)
+    sums = np.add.reduceat(np.concatenate([feats[:, 0].numpy()[indices], [0.0]]), indptr[:-1]) * (deg > 0)
+    labels = torch.from_numpy((sums / np.maximum(deg, 1) > 0).astype(np.int64)).cuda()
+    store = capi.FeatStore(feats.cuda())
+    torch.manual_seed(0)
+    l1, l2 = SAGEConv(16, 32, activation=torch.relu).cuda(), SAGEConv(32, 2).cuda()
+    opt = torch.optim.Adam(list(l1.parameters()) + list(l2.parameters()), lr=0.01)
+    loader = MiniBatchLoader(g, store, torch.arange(n), 256, [10, 10], in_flight=3, seed=1, formats=formats,
+                             as_blocks=True)
+    losses = []
+    for epoch in range(4):
+        for batch in loader:
+            blocks = batch["blocks"]
+            assert all(isinstance(b, Block) for b in blocks) and blocks[-1].num_dst == 256
+            if formats:
+                assert blocks[0].formats is not None and "csr_indptr" in blocks[0].formats
+            h = l2(blocks[1], l1(blocks[0], batch["features"]))
+            loss = torch.nn.functional.cross_entropy(h, labels[batch["output_nodes"]])
+            opt.zero_grad()
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+    assert len(losses) == 4 * 15
+    assert np.mean(losses[-10:]) < 0.6 * np.mean(losses[:5]), (losses[:5], losses[-10:])
