@@ -541,13 +541,14 @@ class BlockFormats:
     Buffers are sized for the upper bounds and reused by every emit(); the edge
     count stays on the device (num_edges).  narrow() waits and cuts to size."""
 
-    def __init__(self, num_dst, fanout, num_src, want_csr=True, device="cuda:0"):
+    def __init__(self, num_dst, fanout, num_src, want_csr=True, device="cuda:0", num_edges=None):
         self.num_dst, self.fanout, self.num_src, self.want_csr = int(num_dst), int(fanout), int(num_src), want_csr
         i64 = dict(dtype=torch.int64, device=device)
         slots = max(self.num_dst * self.fanout, 1)
         self.coo_row, self.coo_col = torch.empty(slots, **i64), torch.empty(slots, **i64)
         self.csc_indptr = torch.empty(self.num_dst + 1, **i64)
-        self.num_edges = torch.zeros(1, **i64)
+        # the edge count stays on the device; a caller that reads several at once passes its own int64[1] view
+        self.num_edges = torch.zeros(1, **i64) if num_edges is None else _dev_i64(num_edges, "num_edges")
         self.csr_indptr = torch.empty(self.num_src + 1, **i64) if want_csr else None
         self.csr_indices = torch.empty(slots, **i64) if want_csr else None
         self.csr_eids = torch.empty(slots, **i64) if want_csr else None
@@ -567,9 +568,10 @@ class BlockFormats:
                                       _ptr(self.csr_eids), _ptr(self.workspace), self.workspace.numel(), _stream()))
         return self
 
-    def narrow(self, num_dst=None, num_src=None):
-        """-> dict of the formats cut to the real sizes (waits for the stream)."""
-        e = int(self.num_edges.item())
+    def narrow(self, num_dst=None, num_src=None, num_edges=None):
+        """-> dict of the formats cut to the real sizes (waits for the stream unless
+        the edge count is given)."""
+        e = int(self.num_edges.item()) if num_edges is None else int(num_edges)
         nd = self.num_dst if num_dst is None else int(num_dst)
         ns = self.num_src if num_src is None else int(num_src)
         out = dict(num_edges=e, coo_row=self.coo_row[:e], coo_col=self.coo_col[:e], csc_indptr=self.csc_indptr[:nd + 1])

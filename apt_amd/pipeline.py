@@ -79,7 +79,9 @@ class MiniBatchPipeline:
             self.request_ws = torch.empty(need, dtype=torch.uint8, device=dev)
         self.formats = None
         if formats:
-            self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=formats != "csc", device=dev)
+            self.format_edges = torch.zeros(H, **i64)             # edge count of every hop's block, read in one go
+            self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=formats != "csc", device=dev,
+                                              num_edges=self.format_edges[h:h + 1])
                             for h, f in enumerate(self.fanouts)]
             # with CSR a hop's formats are a string of ~10 small dependent launches: the hops then run beside
             # each other (and beside the gather) on streams of their own; COO + CSC alone are 2 launches per
@@ -90,6 +92,7 @@ class MiniBatchPipeline:
             self.format_done = [torch.cuda.Event() for _ in self.fanouts]
         self.seeds = None
         self.sizes_host = None
+        self.format_edges_host = None
         self.graph_exec = None
         if use_graph:
             if not self.fused:
@@ -212,6 +215,10 @@ class MiniBatchPipeline:
         self.sizes_host.copy_(self.sizes, non_blocking=True)
         if self.requests is not None:
             self.request_sizes_host.copy_(self.request_sizes, non_blocking=True)
+        if self.formats is not None:
+            if self.format_edges_host is None:
+                self.format_edges_host = torch.empty(len(self.fanouts), dtype=torch.int64, pin_memory=True)
+            self.format_edges_host.copy_(self.format_edges, non_blocking=True)
 
     def result(self, staged=False, as_blocks=False):
         """Waits for the batch and narrows the buffers to their real sizes ->
@@ -222,6 +229,9 @@ class MiniBatchPipeline:
         like everything else, so a training step must finish with them before the
         pipeline runs its next batch."""
         sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
+        fmt_edges = None
+        if self.formats is not None:
+            fmt_edges = self.format_edges_host.tolist() if staged else self.format_edges.cpu().tolist()
         H = len(self.fanouts)
         blocks = []
         for h, f in enumerate(self.fanouts):
@@ -235,7 +245,7 @@ class MiniBatchPipeline:
                                   relabeled=self.relabeled[h][:n * f], counts=self.counts[h][:n],
                                   unique=uniq, fanout=f))
             if self.formats is not None:
-                blocks[0]["formats"] = self.formats[h].narrow(num_dst=n, num_src=sizes[h + 1])
+                blocks[0]["formats"] = self.formats[h].narrow(num_dst=n, num_src=sizes[h + 1], num_edges=fmt_edges[h])
             if as_blocks:
                 from .sampler import Block
                 b = blocks[0]
