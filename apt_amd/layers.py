@@ -21,7 +21,8 @@ class BlockAggregate(torch.autograd.Function):
     @staticmethod
     def forward(ctx, block, X, mean):
         ctx.block, ctx.mean = block, mean
-        return capi.spmm_block(block.relabeled, block.num_dst, block.fanout, X.contiguous(), mean=mean)
+        out = capi.spmm_block(block.relabeled, block.num_dst, block.fanout, X.contiguous(), mean=mean)
+        return out if X.dtype == torch.float32 else out.to(X.dtype)      # sums are fp32 inside the kernel
 
     @staticmethod
     def backward(ctx, dZ):
