@@ -452,21 +452,27 @@ int apt_gat_block(const int64_t* neighbors, int64_t num_dst, const int64_t* num_
                   float* attn_out, void* stream);
 
 /* Backward pass of apt_gat_block (no counterpart in the reference, whose GAT layer
- * gets its gradients from DGL's autograd).  Edge half, one wavefront per
- * (destination, head), fanout <= 64: from dOut [num_dst, heads, dim] and the
+ * gets its gradients from DGL's autograd).  Edge half, fanout <= 64 (a wavefront
+ * per destination when heads is a power of two and heads * fanout <= 64, lane
+ * groups or a wavefront per (destination, head) otherwise): from dOut
+ * [num_dst, heads, dim] and the
  * forward's attention weights attn [num_dst * fanout, heads] it writes, in the
  * block's COO order (edge id = csc_indptr[d] + rank of the slot among d's edges,
  * see apt_block_formats), a_edge and dz_edge [E, heads] (attention weight;
  * gradient of the logit before LeakyReLU) and d_er [num_dst, heads] = sum of dz
  * over a destination's edges.  The source half is two sums over the edges of a
- * source: d el = segment sum of dz_edge, d ft = apt_spmm_heads below.
+ * source, both by one apt_spmm_heads call over the block's CSR order: d ft with
+ * head_weights = a_edge, d el as the second sum with head_weights2 = dz_edge.
+ * apt_spmm_heads is also the backward of the plain block sum / mean
+ * (head_weights NULL, heads 1).
  *   apt_spmm_heads  out[col[e], h, :] += head_weights[w(e), h] * input[row[e], h, :],
  *                   w(e) = weight_row[e] or e when weight_row is NULL (dim = heads *
  *                   head_dim features per row; out fp32, zero-filled by the caller;
  *                   one segment).  grouped != 0: the caller guarantees that edges
  *                   with equal col are consecutive (the block's CSR order); rows that
  *                   lie inside a wavefront's 64 edges are then stored without
- *                   atomics and the result is deterministic.  head_weights2 / out2
+ *                   atomics (deterministic but for rows that span more than two
+ *                   ranges).  head_weights2 / out2
  *                   (both or neither): out2[col[e], h] += head_weights2[w(e), h], a
  *                   second, scalar sum per row and head in the same pass (d el of
  *                   the GAT backward); out2 fp32 [num_out_rows, heads], zero-filled.
