@@ -82,6 +82,269 @@ def parse_args():
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     return ap.parse_args()
 
+def seconds_per_call(torch, fn, reps=10, warm=3):
+    """Mean duration of fn() on the current stream: `reps` back-to-back calls between two events."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e-3
+
+
+def stage_aggregation(args, capi, dev, K, seed_sets, stage_pipe, synth, torch, W):
+    """Optional aggregation stage on the outermost block of the last batch."""
+    stage_pipe.run(seed_sets[W + K - 1], args.seed + 100 + W + K - 1)
+    res = stage_pipe.result()
+    blk = res["blocks"][0]
+    rel = blk["relabeled"]
+    f = blk["fanout"]
+    col_all = torch.arange(blk["seeds"].numel(), device=dev).repeat_interleave(f)
+    keep = rel >= 0
+    row_e, col_e = rel[keep].contiguous(), col_all[keep].contiguous()
+    n_src, n_dst, E, hid = blk["unique"].numel(), blk["seeds"].numel(), int(keep.sum()), 256
+    agg = {"edges": E, "num_src": n_src, "num_dst": n_dst, "hidden": hid}
+    for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+        h = synth.random_features(n_src, hid, dt, args.seed + 7, dev)
+        fn = lambda: capi.spmm_sum(0, row_e, col_e, h, n_dst)
+        t = seconds_per_call(torch, fn)
+        nbytes = E * hid * es + 2 * n_dst * hid * 4 + 16 * E   # rows read, zero-fill + sums written, ids
+        agg[f"spmm_copy_u_sum_{name}_us"] = t * 1e6
+        agg[f"spmm_copy_u_sum_{name}_GBps"] = nbytes / t / 1e9
+        # the same sum (as a mean) straight from the sampler's fixed-stride block layout
+        fn = lambda: capi.spmm_block(rel, n_dst, f, h, mean=True)
+        t = seconds_per_call(torch, fn)
+        nbytes = E * hid * es + n_dst * hid * 4 + 8 * n_dst * f
+        agg[f"spmm_block_mean_{name}_us"] = t * 1e6
+        agg[f"spmm_block_mean_{name}_GBps"] = nbytes / t / 1e9
+    # GAT layer of the same block: 4 heads x 64, logits then fused LeakyReLU + edge softmax + weighted sum
+    heads, hdim = 4, 64
+    for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+        ft = synth.random_features(n_src, heads * hdim, dt, args.seed + 9, dev).view(n_src, heads, hdim)
+        al = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
+        ar = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
+        el, er = capi.gat_scores(ft, al), capi.gat_scores(ft[:n_dst], ar)
+        for tag, fn, nbytes in (
+                ("gat_scores", lambda: capi.gat_scores(ft, al), n_src * heads * (hdim * es + 4)),
+                ("gat_block", lambda: capi.gat_block(rel, n_dst, f, ft, el, er, 0.2),
+                 E * heads * (hdim * es + 4) + n_dst * heads * (hdim * 4 + 4) + 8 * n_dst * f)):
+            t = seconds_per_call(torch, fn)
+            agg[f"{tag}_{name}_us"] = t * 1e6
+            agg[f"{tag}_{name}_GBps"] = nbytes / t / 1e9
+        # backward of the aggregation: logit gradients per (destination, head), then the sums over the
+        # edges of a source on the block's CSR order
+        fmt_b = capi.block_formats(rel, n_dst, f, n_src)
+        _, attn_w = capi.gat_block(rel, n_dst, f, ft, el, er, 0.2, want_attn=True)
+        d_out = torch.randn(n_dst, heads, hdim, device=dev)
+        csr_ip = fmt_b["csr_indptr"][:n_src + 1].contiguous()
+        src_csr = fmt_b["coo_row"][fmt_b["csr_eids"]].contiguous()
+        d2 = d_out.view(n_dst, heads * hdim)
+
+        def gat_bwd():
+            a_e, dz_e, d_er = capi.gat_block_backward(rel, n_dst, f, ft, el, er, 0.2, attn_w, d_out,
+                                                      fmt_b["csc_indptr"], fmt_b["num_edges"])
+            capi.spmm_heads(fmt_b["csr_indices"], src_csr, d_out, a_e, n_src, weight_row=fmt_b["csr_eids"],
+                            grouped=True, head_weights2=dz_e, out_indptr=csr_ip)
+
+        # backward of the plain sum / mean (SAGE, GCN): the same sum over the CSR order, no weights
+        for tag, fn in (("gat_block_backward", gat_bwd),
+                        ("spmm_block_backward", lambda: capi.spmm_heads(
+                            fmt_b["csr_indices"], src_csr, d2, None, n_src, grouped=True, out_indptr=csr_ip))):
+            if tag.startswith("spmm_block_backward") and name != "fp32":
+                continue
+            agg[f"{tag}_{name}_us"] = seconds_per_call(torch, fn) * 1e6
+        del ft, el, er, fmt_b, attn_w, d_out
+    hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
+    h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)
+    fn = lambda: capi.sddmm(0, row_e, col_e, h, hd)
+    t = seconds_per_call(torch, fn)
+    agg["sddmm_u_add_v_fp32_us"] = t * 1e6
+    agg["sddmm_u_add_v_fp32_GBps"] = (3 * E * hid * 4 + 16 * E) / t / 1e9
+    del h, hd
+    return agg
+
+
+def stage_formats(args, B, ev, graph, hops, K, MiniBatchPipeline, requests, seed_sets, store, torch, W):
+    """Optional: every hop's block as COO + CSC (+ CSR), device-side sizes, after sampling."""
+    fmt = {}
+    for name, what in (("coo_csc", "csc"), ("coo_csc_csr", True)):
+        fp = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, formats=what, requests=requests)
+        t = 0.0
+        for i in range(W + K):
+            m = (ev(), ev())
+            fp.sample(seed_sets[i], args.seed + 100 + i)
+            m[0].record()
+            fp.emit_formats()
+            m[1].record()
+            torch.cuda.synchronize()
+            if i >= W:
+                t += m[0].elapsed_time(m[1])
+        fmt[name + "_ms"] = t / K                       # the hops beside each other, nothing else running
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            fp.run(seed_sets[W + i], args.seed + 100 + W + i)
+        torch.cuda.synchronize()
+        fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
+        del fp
+    return fmt
+
+
+def stage_shuffle(args, capi, dev, hops, N, seed_sets, stage_pipe, torch, W):
+    """Optional: bucketing by owner and pack / unpack of hidden rows (the local halves of feat_shuffle)."""
+    ms_of = lambda fn: seconds_per_call(torch, fn) * 1e3
+
+    stage_pipe.run(seed_sets[W], args.seed + 100 + W)
+    torch.cuda.synchronize()
+    H = len(hops)
+    n_in = int(stage_pipe.sizes[H].item())
+    ids = stage_pipe.nodes[:n_in].contiguous()
+    world, hid = 8, 256
+    mv = torch.linspace(0, N, world + 1).to(torch.int64).to(dev)
+    t_bucket = ms_of(lambda: capi.cluster_permute(ids, mv, world))
+    _, _, _, perm = capi.cluster_permute(ids, mv, world)
+    hrows = torch.randn(n_in, hid, device=dev)
+    t_unpack = ms_of(lambda: capi.permute_rows(hrows, perm))
+    t_pack = ms_of(lambda: capi.scatter_rows(hrows, perm))
+    row_bytes = 2 * hid * 4 + 8
+    shuffle = {"ids": n_in, "owners": world, "hidden": hid,
+               "cluster_permute_us": t_bucket * 1e3, "cluster_permute_GBps": 24.0 * n_in / (t_bucket * 1e-3) / 1e9,
+               "unpack_us": t_unpack * 1e3, "unpack_GBps": n_in * row_bytes / (t_unpack * 1e-3) / 1e9,
+               "pack_us": t_pack * 1e3, "pack_GBps": n_in * row_bytes / (t_pack * 1e-3) / 1e9}
+    del hrows, perm, ids
+    return shuffle
+
+
+def stage_cache_build(args, B, bytes_per_row, capi, dev, graph, hops, indptr, N, seed_sets, stage_pipe, store, torch,
+                      W):
+    """Optional: cache construction and the strategy dry run (the callers of the registries)."""
+    from apt_amd import cache as cache_mod
+    from apt_amd import cost_model as cm
+
+    time_ms = lambda fn, reps=5: seconds_per_call(torch, fn, reps=reps, warm=1) * 1e3
+
+    stage_pipe.run(seed_sets[W], args.seed + 100 + W)
+    torch.cuda.synchronize()
+    H = len(hops)
+    n_in = int(stage_pipe.sizes[H].item())
+    counter = cache_mod.HotnessCounter(N, dev)
+    t_count = time_ms(lambda: counter.add(stage_pipe.nodes, n_dev=stage_pipe.sizes[H:H + 1], output_nodes=seed_sets[W]))
+    deg = indptr[1:] - indptr[:-1]
+    hot = torch.topk(deg, min(1_000_000, N // 4)).indices.contiguous()
+    t_csr = time_ms(lambda: cache_mod.build_graph_cache(graph, hot), reps=3)
+    c_edges = int(deg[hot].sum().item())
+    t_feat = time_ms(lambda: capi.gather_rows(store, hot), reps=3)
+    world = 8
+    mv = torch.linspace(0, N, world + 1).to(torch.int64)
+    run = cm.AllPSDryRun(graph, world, list(reversed(hops)), mv, rng_seed=args.seed)
+    per_rank = [seed_sets[i % len(seed_sets)] for i in range(world)]
+    run.sample(per_rank)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    res = run.sample(per_rank)
+    torch.cuda.synchronize()
+    t_dry = time.perf_counter() - t0
+    cache_build = {
+        "count_ids_us": t_count * 1e3, "count_ids_nodes": n_in + B,
+        "cached_csr_rows": int(hot.numel()), "cached_csr_edges": c_edges, "cached_csr_ms": t_csr,
+        "cached_csr_GBps": 16.0 * c_edges / (t_csr * 1e-3) / 1e9,          # every edge read and written once
+        "cached_features_ms": t_feat, "cached_features_GBps": hot.numel() * bytes_per_row / (t_feat * 1e-3) / 1e9,
+        "dry_run_all_strategies_ms_per_step": t_dry * 1e3, "dry_run_world_size": world,
+        "dry_run_input_nodes_rank0": {"DP": int(res[0].dp_seeds.numel()), "NP": int(res[0].np_seeds.numel()),
+                                      "SP": int(res[0].sp_seeds.numel()), "MP": int(res[0].mp_seeds.numel())},
+    }
+    del counter, hot, deg, run, res
+    return cache_build
+
+
+def stage_cpu_baseline(args, bytes_per_row, cache, dtype, feats, hops, indices, indptr, K, lo, min_vids, N, P, pos_map,
+                       requests, seed_sets, torch, W):
+    """CPU baseline: the oracle on this machine's host cores, bounded sample."""
+    budget = args.cpu_seconds
+    import numpy as np
+
+    import oracle as orc
+    threads = args.cpu_threads or min(16, orc.max_threads())
+    orc.set_threads(threads)
+    h_indptr = indptr.cpu().numpy()
+    h_indices = indices.cpu().numpy()
+    if dtype == torch.bfloat16:
+        h_feats = feats.view(torch.int16).cpu().numpy().view(np.uint16)
+    else:
+        h_feats = feats.cpu().numpy()
+    to_np = lambda t: (t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype == torch.bfloat16
+                       else t.cpu().numpy())
+    if requests is None:
+        og = orc.Graph(h_indptr, h_indices)
+        ofs = orc.FeatStore(h_feats)
+    else:
+        h_pos = pos_map.cpu().numpy()
+        og = orc.Graph(h_indptr, h_indices, row_begin=lo, num_total_nodes=N)
+        ofs = orc.FeatStore(h_feats, to_np(cache), h_pos)
+        h_mv, h_rw = min_vids.cpu().numpy(), requests["remote_worker_map"].cpu().numpy()
+    h_seeds = [s.cpu().numpy() for s in seed_sets[W:]]
+    def cpu_leg(seconds, first):
+        """Batches of the timed seed sets (cycled with fresh rng keys) until `seconds` are used."""
+        edges_done = batches = 0
+        tc = 0.0
+        while tc < seconds:
+            s = h_seeds[(first + batches) % K]
+            key = args.seed + 100 + W + first + batches
+            t1 = time.perf_counter()
+            inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
+            if requests is None:
+                orc.gather_rows(ofs, inp)
+            else:
+                bs, _, so, _ = orc.cluster_reqs(inp, h_pos, h_rw, h_mv, P, P)
+                orc.gather_rows(ofs, so[:bs[0]])
+            tc += time.perf_counter() - t1
+            edges_done += sum(int(b["counts"].sum()) for b in blocks)
+            batches += 1
+        return edges_done, batches, tc
+
+    # most of the budget on all threads (the reported value), the rest on one thread for reference
+    cpu_edges, cpu_batches, tc = cpu_leg(budget * 0.75, 0)
+    one = None
+    if threads > 1:
+        orc.set_threads(1)
+        e1, b1, t1s = cpu_leg(budget * 0.25, cpu_batches)
+        one = dict(value=e1 / t1s, batches=b1, seconds=t1s)
+        orc.set_threads(threads)
+    # the gather stage alone, as the reference states it on the CPU (src/load_subtensor.cc:10-17: torch's
+    # index_select over the host table), on the input nodes of one batch
+    gather_cpu = None
+    if requests is None:
+        inp, _ = orc.sample_blocks(og, h_seeds[0], hops, args.replace, args.seed + 100 + W)
+        table = torch.from_numpy(h_feats.view(np.int16) if dtype == torch.bfloat16 else h_feats)
+        ids_t = torch.from_numpy(inp)
+        torch.set_num_threads(threads)
+        table.index_select(0, ids_t[:1000])
+        t1 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t1 < 1.0:
+            table.index_select(0, ids_t)
+            reps += 1
+        tg = (time.perf_counter() - t1) / reps
+        gather_cpu = dict(GBps=len(inp) * bytes_per_row / tg / 1e9, ms=tg * 1e3, rows=int(len(inp)),
+                          what="torch.index_select on the host table (the reference's CPU gather), "
+                               f"{threads} threads")
+        del table, ids_t
+    model = ""
+    try:
+        model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
+    except (OSError, StopIteration):
+        pass
+    cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
+               sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
+                      f"with fresh rng keys) in {tc:.1f} s: sampling, relabel and gather on {threads} "
+                      f"OpenMP threads",
+               one_thread=one, gather_stage=gather_cpu, host_cpu=model, host_logical_cpus=os.cpu_count())
+    del h_indices, h_feats, og, ofs
+    return cpu
+
 
 def main():
     args = parse_args()
@@ -120,6 +383,7 @@ def main():
     N = w["nodes"]
     requests = None
     part_note = ""
+    P = lo = cache = pos_map = min_vids = None      # only partitioned workloads have them
     if "parts" in w:
         P = w["parts"]
         lo, hi = N * w["part"] // P, N * (w["part"] + 1) // P
@@ -318,303 +582,35 @@ def main():
     # ---- optional aggregation stage on the outermost block of the last batch
     agg = None
     if args.aggregation:
-        stage_pipe.run(seed_sets[W + K - 1], args.seed + 100 + W + K - 1)
-        res = stage_pipe.result()
-        blk = res["blocks"][0]
-        rel = blk["relabeled"]
-        f = blk["fanout"]
-        col_all = torch.arange(blk["seeds"].numel(), device=dev).repeat_interleave(f)
-        keep = rel >= 0
-        row_e, col_e = rel[keep].contiguous(), col_all[keep].contiguous()
-        n_src, n_dst, E, hid = blk["unique"].numel(), blk["seeds"].numel(), int(keep.sum()), 256
-        agg = {"edges": E, "num_src": n_src, "num_dst": n_dst, "hidden": hid}
-        for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
-            h = synth.random_features(n_src, hid, dt, args.seed + 7, dev)
-            fn = lambda: capi.spmm_sum(0, row_e, col_e, h, n_dst)
-            for _ in range(3):
-                fn()
-            e0, e1 = ev(), ev()
-            e0.record()
-            for _ in range(10):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            t = e0.elapsed_time(e1) / 10 * 1e-3
-            nbytes = E * hid * es + 2 * n_dst * hid * 4 + 16 * E   # rows read, zero-fill + sums written, ids
-            agg[f"spmm_copy_u_sum_{name}_us"] = t * 1e6
-            agg[f"spmm_copy_u_sum_{name}_GBps"] = nbytes / t / 1e9
-            # the same sum (as a mean) straight from the sampler's fixed-stride block layout
-            fn = lambda: capi.spmm_block(rel, n_dst, f, h, mean=True)
-            for _ in range(3):
-                fn()
-            e0, e1 = ev(), ev()
-            e0.record()
-            for _ in range(10):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            t = e0.elapsed_time(e1) / 10 * 1e-3
-            nbytes = E * hid * es + n_dst * hid * 4 + 8 * n_dst * f
-            agg[f"spmm_block_mean_{name}_us"] = t * 1e6
-            agg[f"spmm_block_mean_{name}_GBps"] = nbytes / t / 1e9
-        # GAT layer of the same block: 4 heads x 64, logits then fused LeakyReLU + edge softmax + weighted sum
-        heads, hdim = 4, 64
-        for name, dt, es in (("fp32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
-            ft = synth.random_features(n_src, heads * hdim, dt, args.seed + 9, dev).view(n_src, heads, hdim)
-            al = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
-            ar = (torch.randn(heads, hdim, device=dev) * 0.02).contiguous()
-            el, er = capi.gat_scores(ft, al), capi.gat_scores(ft[:n_dst], ar)
-            for tag, fn, nbytes in (
-                    ("gat_scores", lambda: capi.gat_scores(ft, al), n_src * heads * (hdim * es + 4)),
-                    ("gat_block", lambda: capi.gat_block(rel, n_dst, f, ft, el, er, 0.2),
-                     E * heads * (hdim * es + 4) + n_dst * heads * (hdim * 4 + 4) + 8 * n_dst * f)):
-                for _ in range(3):
-                    fn()
-                e0, e1 = ev(), ev()
-                e0.record()
-                for _ in range(10):
-                    fn()
-                e1.record()
-                torch.cuda.synchronize()
-                t = e0.elapsed_time(e1) / 10 * 1e-3
-                agg[f"{tag}_{name}_us"] = t * 1e6
-                agg[f"{tag}_{name}_GBps"] = nbytes / t / 1e9
-            # backward of the aggregation: logit gradients per (destination, head), then the sums over the
-            # edges of a source on the block's CSR order
-            fmt_b = capi.block_formats(rel, n_dst, f, n_src)
-            _, attn_w = capi.gat_block(rel, n_dst, f, ft, el, er, 0.2, want_attn=True)
-            d_out = torch.randn(n_dst, heads, hdim, device=dev)
-            csr_ip = fmt_b["csr_indptr"][:n_src + 1].contiguous()
-            src_csr = fmt_b["coo_row"][fmt_b["csr_eids"]].contiguous()
-            d2 = d_out.view(n_dst, heads * hdim)
-
-            def gat_bwd():
-                a_e, dz_e, d_er = capi.gat_block_backward(rel, n_dst, f, ft, el, er, 0.2, attn_w, d_out,
-                                                          fmt_b["csc_indptr"], fmt_b["num_edges"])
-                capi.spmm_heads(fmt_b["csr_indices"], src_csr, d_out, a_e, n_src, weight_row=fmt_b["csr_eids"],
-                                grouped=True, head_weights2=dz_e, out_indptr=csr_ip)
-
-            # backward of the plain sum / mean (SAGE, GCN): the same sum over the CSR order, no weights
-            for tag, fn in (("gat_block_backward", gat_bwd),
-                            ("spmm_block_backward", lambda: capi.spmm_heads(
-                                fmt_b["csr_indices"], src_csr, d2, None, n_src, grouped=True, out_indptr=csr_ip))):
-                if tag.startswith("spmm_block_backward") and name != "fp32":
-                    continue
-                for _ in range(3):
-                    fn()
-                e0, e1 = ev(), ev()
-                e0.record()
-                for _ in range(10):
-                    fn()
-                e1.record()
-                torch.cuda.synchronize()
-                agg[f"{tag}_{name}_us"] = e0.elapsed_time(e1) / 10 * 1e3
-            del ft, el, er, fmt_b, attn_w, d_out
-        hd = synth.random_features(n_dst, hid, torch.float32, args.seed + 8, dev)
-        h = synth.random_features(n_src, hid, torch.float32, args.seed + 7, dev)
-        fn = lambda: capi.sddmm(0, row_e, col_e, h, hd)
-        for _ in range(3):
-            fn()
-        e0, e1 = ev(), ev()
-        e0.record()
-        for _ in range(10):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) / 10 * 1e-3
-        agg["sddmm_u_add_v_fp32_us"] = t * 1e6
-        agg["sddmm_u_add_v_fp32_GBps"] = (3 * E * hid * 4 + 16 * E) / t / 1e9
-        del h, hd
+        agg = stage_aggregation(args=args, capi=capi, dev=dev, K=K, seed_sets=seed_sets,
+                                stage_pipe=stage_pipe, synth=synth, torch=torch, W=W)
 
     # ---- optional: every hop's block as COO + CSC (+ CSR), device-side sizes, after sampling
     fmt = None
     if args.formats:
-        fmt = {}
-        for name, what in (("coo_csc", "csc"), ("coo_csc_csr", True)):
-            fp = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, formats=what, requests=requests)
-            t = 0.0
-            for i in range(W + K):
-                m = (ev(), ev())
-                fp.sample(seed_sets[i], args.seed + 100 + i)
-                m[0].record()
-                fp.emit_formats()
-                m[1].record()
-                torch.cuda.synchronize()
-                if i >= W:
-                    t += m[0].elapsed_time(m[1])
-            fmt[name + "_ms"] = t / K                       # the hops beside each other, nothing else running
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for i in range(K):
-                fp.run(seed_sets[W + i], args.seed + 100 + W + i)
-            torch.cuda.synchronize()
-            fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
-            del fp
+        fmt = stage_formats(args=args, B=B, ev=ev, graph=graph, hops=hops, K=K,
+                            MiniBatchPipeline=MiniBatchPipeline, requests=requests, seed_sets=seed_sets,
+                            store=store, torch=torch, W=W)
 
     # ---- optional: bucketing by owner and pack / unpack of hidden rows (the local halves of feat_shuffle)
     shuffle = None
     if args.shuffle:
-        def ms_of(fn, reps=10):
-            for _ in range(3):
-                fn()
-            e0, e1 = ev(), ev()
-            e0.record()
-            for _ in range(reps):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) / reps
-
-        stage_pipe.run(seed_sets[W], args.seed + 100 + W)
-        torch.cuda.synchronize()
-        H = len(hops)
-        n_in = int(stage_pipe.sizes[H].item())
-        ids = stage_pipe.nodes[:n_in].contiguous()
-        world, hid = 8, 256
-        mv = torch.linspace(0, N, world + 1).to(torch.int64).to(dev)
-        t_bucket = ms_of(lambda: capi.cluster_permute(ids, mv, world))
-        _, _, _, perm = capi.cluster_permute(ids, mv, world)
-        hrows = torch.randn(n_in, hid, device=dev)
-        t_unpack = ms_of(lambda: capi.permute_rows(hrows, perm))
-        t_pack = ms_of(lambda: capi.scatter_rows(hrows, perm))
-        row_bytes = 2 * hid * 4 + 8
-        shuffle = {"ids": n_in, "owners": world, "hidden": hid,
-                   "cluster_permute_us": t_bucket * 1e3, "cluster_permute_GBps": 24.0 * n_in / (t_bucket * 1e-3) / 1e9,
-                   "unpack_us": t_unpack * 1e3, "unpack_GBps": n_in * row_bytes / (t_unpack * 1e-3) / 1e9,
-                   "pack_us": t_pack * 1e3, "pack_GBps": n_in * row_bytes / (t_pack * 1e-3) / 1e9}
-        del hrows, perm, ids
+        shuffle = stage_shuffle(args=args, capi=capi, dev=dev, hops=hops, N=N, seed_sets=seed_sets,
+                                stage_pipe=stage_pipe, torch=torch, W=W)
 
     # ---- optional: cache construction and the strategy dry run (the callers of the registries)
     cache_build = None
     if args.cache_build and requests is None:
-        from apt_amd import cache as cache_mod
-        from apt_amd import cost_model as cm
-
-        def time_ms(fn, reps=5):
-            fn()
-            e0, e1 = ev(), ev()
-            e0.record()
-            for _ in range(reps):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) / reps
-
-        stage_pipe.run(seed_sets[W], args.seed + 100 + W)
-        torch.cuda.synchronize()
-        H = len(hops)
-        n_in = int(stage_pipe.sizes[H].item())
-        counter = cache_mod.HotnessCounter(N, dev)
-        t_count = time_ms(lambda: counter.add(stage_pipe.nodes, n_dev=stage_pipe.sizes[H:H + 1], output_nodes=seed_sets[W]))
-        deg = indptr[1:] - indptr[:-1]
-        hot = torch.topk(deg, min(1_000_000, N // 4)).indices.contiguous()
-        t_csr = time_ms(lambda: cache_mod.build_graph_cache(graph, hot), reps=3)
-        c_edges = int(deg[hot].sum().item())
-        t_feat = time_ms(lambda: capi.gather_rows(store, hot), reps=3)
-        world = 8
-        mv = torch.linspace(0, N, world + 1).to(torch.int64)
-        run = cm.AllPSDryRun(graph, world, list(reversed(hops)), mv, rng_seed=args.seed)
-        per_rank = [seed_sets[i % len(seed_sets)] for i in range(world)]
-        run.sample(per_rank)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        res = run.sample(per_rank)
-        torch.cuda.synchronize()
-        t_dry = time.perf_counter() - t0
-        cache_build = {
-            "count_ids_us": t_count * 1e3, "count_ids_nodes": n_in + B,
-            "cached_csr_rows": int(hot.numel()), "cached_csr_edges": c_edges, "cached_csr_ms": t_csr,
-            "cached_csr_GBps": 16.0 * c_edges / (t_csr * 1e-3) / 1e9,          # every edge read and written once
-            "cached_features_ms": t_feat, "cached_features_GBps": hot.numel() * bytes_per_row / (t_feat * 1e-3) / 1e9,
-            "dry_run_all_strategies_ms_per_step": t_dry * 1e3, "dry_run_world_size": world,
-            "dry_run_input_nodes_rank0": {"DP": int(res[0].dp_seeds.numel()), "NP": int(res[0].np_seeds.numel()),
-                                          "SP": int(res[0].sp_seeds.numel()), "MP": int(res[0].mp_seeds.numel())},
-        }
-        del counter, hot, deg, run, res
+        cache_build = stage_cache_build(args=args, B=B, bytes_per_row=bytes_per_row, capi=capi, dev=dev,
+                                        graph=graph, hops=hops, indptr=indptr, N=N, seed_sets=seed_sets,
+                                        stage_pipe=stage_pipe, store=store, torch=torch, W=W)
 
     # ---- CPU baseline: the oracle on this machine's host cores, bounded sample
     cpu = None
-    budget = args.cpu_seconds
-    if budget > 0:
-        import numpy as np
-
-        import oracle as orc
-        threads = args.cpu_threads or min(16, orc.max_threads())
-        orc.set_threads(threads)
-        h_indptr = indptr.cpu().numpy()
-        h_indices = indices.cpu().numpy()
-        if dtype == torch.bfloat16:
-            h_feats = feats.view(torch.int16).cpu().numpy().view(np.uint16)
-        else:
-            h_feats = feats.cpu().numpy()
-        to_np = lambda t: (t.view(torch.int16).cpu().numpy().view(np.uint16) if t.dtype == torch.bfloat16
-                           else t.cpu().numpy())
-        if requests is None:
-            og = orc.Graph(h_indptr, h_indices)
-            ofs = orc.FeatStore(h_feats)
-        else:
-            h_pos = pos_map.cpu().numpy()
-            og = orc.Graph(h_indptr, h_indices, row_begin=lo, num_total_nodes=N)
-            ofs = orc.FeatStore(h_feats, to_np(cache), h_pos)
-            h_mv, h_rw = min_vids.cpu().numpy(), requests["remote_worker_map"].cpu().numpy()
-        h_seeds = [s.cpu().numpy() for s in seed_sets[W:]]
-        def cpu_leg(seconds, first):
-            """Batches of the timed seed sets (cycled with fresh rng keys) until `seconds` are used."""
-            edges_done = batches = 0
-            tc = 0.0
-            while tc < seconds:
-                s = h_seeds[(first + batches) % K]
-                key = args.seed + 100 + W + first + batches
-                t1 = time.perf_counter()
-                inp, blocks = orc.sample_blocks(og, s, hops, args.replace, key)
-                if requests is None:
-                    orc.gather_rows(ofs, inp)
-                else:
-                    bs, _, so, _ = orc.cluster_reqs(inp, h_pos, h_rw, h_mv, P, P)
-                    orc.gather_rows(ofs, so[:bs[0]])
-                tc += time.perf_counter() - t1
-                edges_done += sum(int(b["counts"].sum()) for b in blocks)
-                batches += 1
-            return edges_done, batches, tc
-
-        # most of the budget on all threads (the reported value), the rest on one thread for reference
-        cpu_edges, cpu_batches, tc = cpu_leg(budget * 0.75, 0)
-        one = None
-        if threads > 1:
-            orc.set_threads(1)
-            e1, b1, t1s = cpu_leg(budget * 0.25, cpu_batches)
-            one = dict(value=e1 / t1s, batches=b1, seconds=t1s)
-            orc.set_threads(threads)
-        # the gather stage alone, as the reference states it on the CPU (src/load_subtensor.cc:10-17: torch's
-        # index_select over the host table), on the input nodes of one batch
-        gather_cpu = None
-        if requests is None:
-            inp, _ = orc.sample_blocks(og, h_seeds[0], hops, args.replace, args.seed + 100 + W)
-            table = torch.from_numpy(h_feats.view(np.int16) if dtype == torch.bfloat16 else h_feats)
-            ids_t = torch.from_numpy(inp)
-            torch.set_num_threads(threads)
-            table.index_select(0, ids_t[:1000])
-            t1 = time.perf_counter()
-            reps = 0
-            while time.perf_counter() - t1 < 1.0:
-                table.index_select(0, ids_t)
-                reps += 1
-            tg = (time.perf_counter() - t1) / reps
-            gather_cpu = dict(GBps=len(inp) * bytes_per_row / tg / 1e9, ms=tg * 1e3, rows=int(len(inp)),
-                              what="torch.index_select on the host table (the reference's CPU gather), "
-                                   f"{threads} threads")
-            del table, ids_t
-        model = ""
-        try:
-            model = next(l.split(":", 1)[1].strip() for l in open("/proc/cpuinfo") if l.startswith("model name"))
-        except (OSError, StopIteration):
-            pass
-        cpu = dict(value=cpu_edges / tc, unit="edges/s", cores=threads, kind="port",
-                   sample=f"{cpu_batches} batches of the same workload (the timed seed sets, cycled "
-                          f"with fresh rng keys) in {tc:.1f} s: sampling, relabel and gather on {threads} "
-                          f"OpenMP threads",
-                   one_thread=one, gather_stage=gather_cpu, host_cpu=model, host_logical_cpus=os.cpu_count())
-        del h_indices, h_feats, og, ofs
+    if args.cpu_seconds > 0:
+        cpu = stage_cpu_baseline(args=args, bytes_per_row=bytes_per_row, cache=cache, dtype=dtype, feats=feats,
+                                 hops=hops, indices=indices, indptr=indptr, K=K, lo=lo, min_vids=min_vids, N=N,
+                                 P=P, pos_map=pos_map, requests=requests, seed_sets=seed_sets, torch=torch, W=W)
 
     out = {
         "metric": "sampled edges/s (3-hop 15,10,5) + feature-gather GB/s as % of HBM peak",
