@@ -212,18 +212,28 @@ __global__ __launch_bounds__(kAggBlock) void spmm_kernel(AggParams p) {
 
 // Companion of spmm_kernel with out_indptr: zeroes the output rows that the main kernel does not store whole,
 // i.e. rows without edges and rows whose edges lie in more than one wavefront range (those are added
-// atomically).  A lane group of 16 per row.
+// atomically).  A wavefront checks 64 rows with one coalesced pair of loads, then zeroes the flagged ones
+// together, a row at a time.
 __global__ __launch_bounds__(kAggBlock) void spmm_zero_rows_kernel(const int64_t* __restrict__ out_indptr,
                                                                    int64_t num_rows, int64_t dim, float* out,
                                                                    float* out2, int heads) {
-  constexpr int kLanes = 16;
-  const int l = threadIdx.x % kLanes;
-  for (int64_t r = (static_cast<int64_t>(blockIdx.x) * kAggBlock + threadIdx.x) / kLanes; r < num_rows;
-       r += static_cast<int64_t>(gridDim.x) * (kAggBlock / kLanes)) {
-    const int64_t lo = out_indptr[r], hi = out_indptr[r + 1];
-    if (hi > lo && lo / kEdgesPerWave == (hi - 1) / kEdgesPerWave) continue;   // stored whole by one wavefront
-    for (int64_t d = l; d < dim; d += kLanes) out[r * dim + d] = 0.f;
-    if (out2 != nullptr && l < heads) out2[r * heads + l] = 0.f;
+  const int lane = threadIdx.x % kWave;
+  for (int64_t base = (static_cast<int64_t>(blockIdx.x) * kAggWaves + threadIdx.x / kWave) * kWave; base < num_rows;
+       base += static_cast<int64_t>(gridDim.x) * kAggWaves * kWave) {
+    const int64_t r = base + lane;
+    bool need = false;
+    if (r < num_rows) {
+      const int64_t lo = out_indptr[r], hi = out_indptr[r + 1];
+      need = !(hi > lo && lo / kEdgesPerWave == (hi - 1) / kEdgesPerWave);   // else stored whole by one wavefront
+    }
+    uint64_t todo = ballot(need);
+    while (todo != 0) {
+      const int j = __ffsll(static_cast<long long>(todo)) - 1;
+      todo &= todo - 1;
+      float* row = out + (base + j) * dim;
+      for (int64_t d = lane; d < dim; d += kWave) row[d] = 0.f;
+      if (out2 != nullptr && lane < heads) out2[(base + j) * heads + lane] = 0.f;
+    }
   }
 }
 
@@ -1073,12 +1083,12 @@ extern "C" int apt_spmm_heads(const int64_t* coo_row, const int64_t* coo_col, in
               elem_size);
   APT_REQUIRE(num_out_rows >= 0 && num_in_rows >= 0, APT_EINVAL, "apt_spmm_heads: negative row count");
   APT_REQUIRE(out_indptr == nullptr || grouped != 0, APT_EINVAL, "apt_spmm_heads: out_indptr needs grouped edges");
-  APT_REQUIRE(heads <= 16 || out2 == nullptr || out_indptr == nullptr, APT_ELIMIT,
-              "apt_spmm_heads: out_indptr with a second sum supports at most 16 heads");
+  APT_REQUIRE(heads <= kWave || out2 == nullptr || out_indptr == nullptr, APT_ELIMIT,
+              "apt_spmm_heads: out_indptr with a second sum supports at most 64 heads");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (out_indptr != nullptr && num_out_rows > 0) {
     APT_REQUIRE(out != nullptr, APT_EINVAL, "apt_spmm_heads: out is NULL");
-    const unsigned zb = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_out_rows, kAggBlock / 16), 1 << 20));
+    const unsigned zb = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_out_rows, kAggBlock), 1 << 20));
     hipLaunchKernelGGL(spmm_zero_rows_kernel, dim3(zb), dim3(kAggBlock), 0, st, out_indptr, num_out_rows, dim, out,
                        out2, heads);
     APT_LAUNCH_CHECK("spmm_zero_rows_kernel");
