@@ -16,7 +16,7 @@ capi.lib()  # fail loudly when the HIP library is missing
 
 _NPC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libnpc.so")
 if not os.path.exists(_NPC):
-    raise ImportError(f"{_NPC} is missing: build it with `python -m apt_amd.build`")
+    raise ImportError(f"{_NPC} is missing: build it with `python apt_amd/build.py`")
 try:
     torch.ops.load_library(_NPC)  # reference python/npc/__init__.py:6-12
 except Exception as e:  # pragma: no cover

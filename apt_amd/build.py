@@ -1,4 +1,7 @@
-"""Builds libapt_hip.so (the C-ABI HIP library) for gfx950 with hipcc.
+"""Builds libapt_hip.so (the C-ABI HIP library) for gfx950 with hipcc, and libnpc.so.
+
+Run it as a script (`python apt_amd/build.py`): importing it as `apt_amd.build`
+would first import the package, which needs the libraries this file produces.
 
 The library has no dependency on torch or Python: it is plain HIP.  hipcc
 cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is
@@ -29,8 +32,8 @@ def _obj(src):
 def build(force=True, verbose=False):
     """Compile every source and link libapt_hip.so.  Returns its path."""
     procs = []
-    headers = [os.path.join(CSRC, "common.hpp"), os.path.join(HERE, "..", "include", "apt_amd.h"),
-               os.path.join(HERE, "..", "include", "apt_synth.h")]
+    headers = [os.path.join(CSRC, h) for h in sorted(os.listdir(CSRC)) if h.endswith(".hpp")]
+    headers += [os.path.join(HERE, "..", "include", "apt_amd.h"), os.path.join(HERE, "..", "include", "apt_synth.h")]
     newest_hdr = max(os.path.getmtime(h) for h in headers)
     objs = []
     for s in SOURCES:

@@ -88,7 +88,7 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError(
-                f"{LIB_PATH} is missing: build it with `python -m apt_amd.build` "
+                f"{LIB_PATH} is missing: build it with `python apt_amd/build.py` "
                 "(hipcc, gfx950).  There is no CPU fallback.")
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SYMBOLS.items():
