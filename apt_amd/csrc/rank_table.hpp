@@ -6,9 +6,12 @@
 
 namespace apt {
 
-// States of a relabeled[] slot before its compact id is known.
-constexpr int64_t kSlotOwner = -2;  // bid placed and, so far, the smallest for its node
-constexpr int64_t kSlotLoser = -3;  // another slot holds a smaller bid for the same node
+// States of a relabeled[] slot before its compact id is known.  They are the two
+// most negative values, so that no id a graph can hold, valid or corrupt, is
+// mistaken for one: a negative id is padding and passes through unchanged, as in
+// the hash-table relabel.
+constexpr int64_t kSlotLoser = INT64_MIN;      // another slot holds a smaller bid for the same node
+constexpr int64_t kSlotOwner = INT64_MIN + 1;  // bid placed and, so far, the smallest for its node
 
 struct RankTable {
   uint32_t* entries;        // one per node: (epoch << payload bits) | id or bid
@@ -33,7 +36,7 @@ __device__ __forceinline__ uint32_t table_base(const uint32_t* state) { return s
 // yet and ownership is decided by re-reading the table; no flags are kept.
 __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, uint32_t tb, bool first_hop,
                                                   int64_t v, int64_t ns, int64_t j) {
-  if (v < 0) return v;
+  if (v < 0) return v <= kSlotOwner ? -1 : v;  // padding; never one of the two states above
   if (v >= t.len) return -1;  // an id the table cannot hold: treated as padding
   const uint32_t first_bid = tb + static_cast<uint32_t>(ns);
   const uint32_t bid = first_bid + static_cast<uint32_t>(j);

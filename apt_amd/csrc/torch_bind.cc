@@ -410,12 +410,32 @@ Tensor LoadSubtensor(Tensor node_id) {
   return out;
 }
 
-// reference src/load_subtensor.cc:10-17
+// reference src/load_subtensor.cc:10-17: two index_selects, the result on the host
+// as there.  The local table lives in HBM here, so the rows come from the GPU; the
+// ids are checked on the host first (the map copy is a host tensor), where the
+// reference's host index_select would raise: an id outside the map or without a
+// local row never reaches a kernel.
 Tensor CPULoadSubtensor(Tensor node_id) {
   auto& s = S();
   TORCH_CHECK(s.has_feat, "npc: no features registered (cache_feats_shared)");
-  auto pos = -s.cpu_feat_pos_map.index_select(0, node_id.cpu()) - 2;
-  return s.local_feats.index_select(0, pos.to(s.local_feats.device()));
+  TORCH_CHECK(node_id.scalar_type() == torch::kInt64, "npc: node_id must be int64");
+  auto ids = node_id.cpu().contiguous().view({-1});
+  const int64_t total = s.cpu_feat_pos_map.numel();
+  const int64_t* idp = ids.data_ptr<int64_t>();
+  const int64_t* map = s.cpu_feat_pos_map.data_ptr<int64_t>();
+  auto pos = torch::empty({ids.numel()}, torch::TensorOptions().dtype(torch::kInt64));
+  int64_t* pp = pos.data_ptr<int64_t>();
+  const int64_t n_local = s.local_feats.size(0);
+  for (int64_t i = 0; i < ids.numel(); ++i) {
+    const int64_t v = idp[i];
+    TORCH_CHECK_INDEX(v >= 0 && v < total, "npc: cpu_load_subtensor: node id ", v, " at position ", i,
+                      " is outside [0, ", total, ")");
+    const int64_t row = -map[v] - 2;  // ENCODE_ID, src/utils.h:17
+    TORCH_CHECK_INDEX(row >= 0 && row < n_local, "npc: cpu_load_subtensor: node ", v, " at position ", i,
+                      " has no local feature row");
+    pp[i] = row;
+  }
+  return s.local_feats.index_select(0, pos.to(s.local_feats.device())).cpu();
 }
 
 std::tuple<Tensor, Tensor, Tensor, Tensor> ClusterAndPermuteLocal(Tensor seeds) {

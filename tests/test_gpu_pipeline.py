@@ -97,7 +97,9 @@ def test_operator_layer_dp_sampler(orc, capi):
     assert np.array_equal(output_nodes.cpu().numpy(), seeds)
     _, x = npc.load_batch(type("A", (), {"system": "DP"})(), (input_nodes, output_nodes, blocks))
     assert np.array_equal(x.cpu().numpy(), feats[frontier])
-    assert np.array_equal(npc.cpu_load_subtensor(input_nodes.cpu()).cpu().numpy(), feats[frontier])
+    host_rows = npc.cpu_load_subtensor(input_nodes.cpu())
+    assert host_rows.device.type == "cpu"                      # as the reference's CPU statement returns
+    assert np.array_equal(host_rows.numpy(), feats[frontier])
     with pytest.raises(IndexError):
         npc.load_subtensor(torch.tensor([0, n + 5]))
     with pytest.raises(RuntimeError):
@@ -105,6 +107,53 @@ def test_operator_layer_dp_sampler(orc, capi):
     # the operators are reachable under the reference's names
     u, r = torch.ops.npc.relabel_csc(dev(seeds), dev(seeds[::-1].copy()))
     assert np.array_equal(u.cpu().numpy(), seeds)
+
+
+def test_cpu_load_subtensor_rejects_ids_without_a_local_row(orc, capi):
+    """Ids are checked on the host before anything is enqueued: a node outside the map, or one
+    that has no local row (map entry -1, or a cache-only node), raises IndexError."""
+    import apt_amd as npc
+    n, dim = 1000, 16
+    feats = np.random.default_rng(0).standard_normal((600, dim)).astype(np.float32)
+    local_idx = torch.arange(0, 600)
+    cache = torch.from_numpy(np.random.default_rng(1).standard_normal((50, dim)).astype(np.float32))
+    cache_idx = torch.arange(700, 750)
+    npc.set_topology(0, 1)
+    npc.cache_feats_shared(n, torch.from_numpy(feats), cache, cache_idx, local_idx, 0)
+    ok = npc.cpu_load_subtensor(torch.tensor([5, 599, 0, 5]))
+    assert np.array_equal(ok.numpy(), feats[[5, 599, 0, 5]])
+    assert npc.cpu_load_subtensor(torch.empty(0, dtype=torch.int64)).shape == (0, dim)
+    for bad in ([5, 650], [720], [n], [-1], [3, -7, 2]):
+        with pytest.raises(IndexError):
+            npc.cpu_load_subtensor(torch.tensor(bad))
+    torch.cuda.synchronize()                                   # nothing faulted on the device
+
+
+def test_fused_driver_passes_corrupt_negative_ids_through(orc, capi):
+    """An adjacency list that holds negative entries (-2, -3, ... a corrupt file): every negative id
+    is padding for the relabel, in the fused driver as in the per-hop one and in the oracle."""
+    from apt_amd.pipeline import MiniBatchPipeline
+    indptr, indices = small_graph(3000, 12, seed=9)
+    indices = indices.copy()
+    rng = np.random.default_rng(2)
+    hit = rng.permutation(len(indices))[: len(indices) // 10]
+    indices[hit] = rng.choice(np.array([-1, -2, -3, -4, -(2 ** 40), np.iinfo(np.int64).min + 2]), size=len(hit))
+    og = orc.Graph(indptr, indices)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    hops = [5, 10, 15]
+    seeds = rng.permutation(3000)[:256]
+    want_in, want_blocks = orc.sample_blocks(og, seeds, hops, False, 31)
+    assert any((b["relabeled"] < -1).any() for b in want_blocks)
+    for fused in (True, False):
+        pipe = MiniBatchPipeline(dg, None, 256, hops, replace=False, fused=fused, gather=False)
+        for _ in range(2):
+            pipe.run(dev(seeds), 31)
+            res = pipe.result()
+            assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+            assert (res["input_nodes"] >= 0).all()
+            for got, want in zip(res["blocks"], want_blocks):
+                for k in ("neighbors", "relabeled", "counts", "unique"):
+                    assert np.array_equal(got[k].cpu().numpy(), want[k]), (fused, k)
 
 
 def test_operator_layer_caches_and_buckets(orc, capi):
