@@ -152,3 +152,35 @@ def random_features(num_rows, dim, dtype, seed, device="cuda:0"):
         e = min(s + step, num_rows)
         out[s:e] = torch.randn((e - s, dim), generator=gen, device=device, dtype=torch.float32).to(dtype)
     return out
+
+
+def partition_share(num_nodes, num_edges, parts, part, dim, dtype, cache_ratio, seed, device="cuda:0"):
+    """One GPU's share of a graph split into `parts` contiguous id ranges (the reference's partitioned
+    layout: python/npc/utils/utils.py load_partition, src/cache_feats.cc:14-61, src/core.cc:102-125):
+    the CSR rows of range `part` (neighbour ids stay global), the feature rows of that range, a cache
+    of the `cache_ratio` hottest remote rows (largest expected degree; ties by id), the position map
+    over all ids (-(i)-2 local row i, >= 0 cache row, -1 absent), the range bounds `min_vids` and the
+    owner -> request-bucket map (bucket 0 = this GPU, the other owners 1.. in id order).
+    -> dict(lo, hi, indptr, indices, feats, cache, hot, pos_map, min_vids, remote_worker_map)"""
+    import torch
+
+    lo, hi = num_nodes * part // parts, num_nodes * (part + 1) // parts
+    indptr, indices = rmat_csr_gpu(num_nodes, num_edges, seed, device, row_begin=lo, num_rows=hi - lo)
+    feats = random_features(hi - lo, dim, dtype, seed + 1, device)
+    exp_deg = rmat_expected_degree(num_nodes, num_edges, device)
+    exp_deg[lo:hi] = -1.0
+    n_cache = int((num_nodes - (hi - lo)) * cache_ratio)
+    hot = torch.sort(exp_deg, descending=True, stable=True).indices[:n_cache].contiguous()
+    del exp_deg
+    cache = random_features(n_cache, dim, dtype, seed + 3, device)
+    pos_map = torch.full((num_nodes,), -1, dtype=torch.int64, device=device)
+    pos_map[lo:hi] = -torch.arange(hi - lo, dtype=torch.int64, device=device) - 2
+    pos_map[hot] = torch.arange(n_cache, dtype=torch.int64, device=device)
+    min_vids = torch.tensor([num_nodes * k // parts for k in range(parts + 1)], dtype=torch.int64, device=device)
+    rwm, nxt = [0] * parts, 1
+    for k in range(parts):
+        if k != part:
+            rwm[k] = nxt
+            nxt += 1
+    return dict(lo=lo, hi=hi, indptr=indptr, indices=indices, feats=feats, cache=cache, hot=hot, pos_map=pos_map,
+                min_vids=min_vids, remote_worker_map=torch.tensor(rwm, dtype=torch.int64, device=device))

@@ -386,32 +386,15 @@ def main():
     P = lo = cache = pos_map = min_vids = None      # only partitioned workloads have them
     if "parts" in w:
         P = w["parts"]
-        lo, hi = N * w["part"] // P, N * (w["part"] + 1) // P
-        indptr, indices = synth.rmat_csr_gpu(N, w["edges"], args.seed, dev, row_begin=lo, num_rows=hi - lo)
+        share = synth.partition_share(N, w["edges"], P, w["part"], w["dim"], dtype, w["cache_ratio"], args.seed, dev)
+        lo, hi, indptr, indices, feats = share["lo"], share["hi"], share["indptr"], share["indices"], share["feats"]
+        cache, pos_map, min_vids, n_cache = share["cache"], share["pos_map"], share["min_vids"], share["hot"].numel()
         graph = capi.Graph(indptr, indices, row_begin=lo, num_total_nodes=N)
-        feats = synth.random_features(hi - lo, w["dim"], dtype, args.seed + 1, dev)
-        # hot-node cache: the remote nodes with the largest expected degree
-        exp_deg = synth.rmat_expected_degree(N, w["edges"], dev)
-        exp_deg[lo:hi] = -1.0
-        n_cache = int((N - (hi - lo)) * w["cache_ratio"])
-        hot = torch.sort(exp_deg, descending=True, stable=True).indices[:n_cache].contiguous()
-        del exp_deg
-        cache = synth.random_features(n_cache, w["dim"], dtype, args.seed + 3, dev)
-        pos_map = torch.full((N,), -1, dtype=torch.int64, device=dev)
-        pos_map[lo:hi] = -torch.arange(hi - lo, dtype=torch.int64, device=dev) - 2
-        pos_map[hot] = torch.arange(n_cache, dtype=torch.int64, device=dev)
         store = capi.FeatStore(feats, cache, pos_map)
-        min_vids = torch.tensor([N * k // P for k in range(P + 1)], dtype=torch.int64, device=dev)
-        # bucket 0 is this GPU (reference src/cuda/npc_kernel.cu:398-408): the own part maps to 0,
-        # the other owners to 1..P-1
-        rwm = [0] * P
-        nxt = 1
-        for k in range(P):
-            if k != w["part"]:
-                rwm[k] = nxt
-                nxt += 1
-        requests = dict(feat_pos_map=pos_map, remote_worker_map=torch.tensor(rwm, dtype=torch.int64, device=dev),
+        # bucket 0 is this GPU (reference src/cuda/npc_kernel.cu:398-408), the other owners 1..P-1
+        requests = dict(feat_pos_map=pos_map, remote_worker_map=share["remote_worker_map"],
                         min_vids=min_vids, world_size=P, num_remote_workers=P)
+        del share
         seed_lo, seed_n = lo, hi - lo
         part_note = (f", rows [{lo}, {hi}) of {P} contiguous parts held here, cache of the {n_cache} "
                      f"hottest remote rows, misses bucketed into {P} owner lists")
