@@ -45,6 +45,8 @@ SYMBOLS = {
     "apt_sample_neighbors": (_I, [C.POINTER(CGraph), _P, _I64, _P, _I, _I, _U64, _I, _P, _P, _P, _P]),
     "apt_relabel_workspace_bytes": (_SZ, [_I64]),
     "apt_relabel": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_relabel_static_max_items": (_I64, []),
+    "apt_relabel_static": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P]),
     "apt_gather_rows": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P]),
     "apt_time_next_gather": (_I, [_P, _P]),
     "apt_permute_rows": (_I, [_P, _I64, _P, _I64, _I64, _I, _P, _P]),

@@ -24,6 +24,8 @@
 //     the output and into their slot, so only repeated keys go back to the table;
 //   * the count stays on the device unless the caller asks for it.
 // Passes: fill -> insert -> count owners per block -> place owners -> relabel.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace apt {
@@ -291,34 +293,39 @@ extern "C" size_t apt_relabel_workspace_bytes(int64_t num_items) {
   return apt::relabel_layout(num_items).total;
 }
 
-extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
-                           const int64_t* num_seeds_dev, const int64_t* neighbors,
-                           int64_t num_neighbors, int64_t neighbor_stride,
-                           int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev,
-                           int64_t* num_unique_host, void* workspace,
-                           size_t workspace_bytes, void* stream) {
-  using namespace apt;
-  APT_REQUIRE(num_seeds >= 0 && num_neighbors >= 0, APT_EINVAL,
-              "apt_relabel: negative size (%lld seeds, %lld neighbors)",
-              (long long)num_seeds, (long long)num_neighbors);
-  const int64_t items = num_seeds + num_neighbors;
-  APT_REQUIRE(items <= kRelMaxItems, APT_ELIMIT,
-              "apt_relabel: %lld items exceed the supported maximum %lld per call",
-              (long long)items, (long long)kRelMaxItems);
-  APT_REQUIRE(num_unique_dev != nullptr, APT_EINVAL, "apt_relabel: num_unique_dev is NULL");
-  APT_REQUIRE(num_seeds == 0 || seeds != nullptr, APT_EINVAL, "apt_relabel: seeds is NULL");
-  APT_REQUIRE(num_neighbors == 0 || (neighbors != nullptr && relabeled != nullptr), APT_EINVAL,
-              "apt_relabel: neighbors/relabeled is NULL");
-  APT_REQUIRE(items == 0 || unique != nullptr, APT_EINVAL, "apt_relabel: unique is NULL");
-  APT_REQUIRE(num_seeds_dev == nullptr || neighbor_stride >= 0, APT_EINVAL,
-              "apt_relabel: neighbor_stride %lld < 0", (long long)neighbor_stride);
-  const RelabelLayout L = relabel_layout(items);
-  APT_REQUIRE(workspace != nullptr && workspace_bytes >= L.total, APT_EWORKSPACE,
-              "apt_relabel: workspace of %zu bytes, %zu needed", workspace_bytes, L.total);
-  APT_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, APT_EINVAL,
-              "apt_relabel: workspace must be 16-byte aligned");
+namespace apt {
 
-  char* ws = static_cast<char*>(workspace);
+// Validation shared by the two entry points.
+static int relabel_check_args(const char* who, const int64_t* seeds, int64_t num_seeds,
+                              const int64_t* num_seeds_dev, const int64_t* neighbors,
+                              int64_t num_neighbors, int64_t neighbor_stride, const int64_t* unique,
+                              const int64_t* relabeled, const int64_t* num_unique_dev, int64_t max_items) {
+  APT_REQUIRE(num_seeds >= 0 && num_neighbors >= 0, APT_EINVAL,
+              "%s: negative size (%lld seeds, %lld neighbors)", who,
+              (long long)num_seeds, (long long)num_neighbors);
+  // each size on its own first: their sum must not wrap
+  APT_REQUIRE(num_seeds <= max_items && num_neighbors <= max_items && num_seeds + num_neighbors <= max_items,
+              APT_ELIMIT, "%s: %lld seeds + %lld neighbors exceed the supported maximum of %lld items per call",
+              who, (long long)num_seeds, (long long)num_neighbors, (long long)max_items);
+  const int64_t items = num_seeds + num_neighbors;
+  APT_REQUIRE(num_unique_dev != nullptr, APT_EINVAL, "%s: num_unique_dev is NULL", who);
+  APT_REQUIRE(num_seeds == 0 || seeds != nullptr, APT_EINVAL, "%s: seeds is NULL", who);
+  APT_REQUIRE(num_neighbors == 0 || (neighbors != nullptr && relabeled != nullptr), APT_EINVAL,
+              "%s: neighbors/relabeled is NULL", who);
+  APT_REQUIRE(items == 0 || unique != nullptr, APT_EINVAL, "%s: unique is NULL", who);
+  APT_REQUIRE(num_seeds_dev == nullptr || neighbor_stride >= 0, APT_EINVAL,
+              "%s: neighbor_stride %lld < 0", who, (long long)neighbor_stride);
+  return APT_OK;
+}
+
+// The five passes on `st`; `ws` holds relabel_layout(num_seeds + num_neighbors).total bytes
+// whose contents do not matter on entry (the fill pass sets what must start clean).
+static int relabel_enqueue(const int64_t* seeds, int64_t num_seeds, const int64_t* num_seeds_dev,
+                           const int64_t* neighbors, int64_t num_neighbors, int64_t neighbor_stride,
+                           int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev, char* ws,
+                           hipStream_t st) {
+  const int64_t items = num_seeds + num_neighbors;
+  const RelabelLayout L = relabel_layout(items);
   RelabelParams p;
   p.seeds = seeds;
   p.ns = num_seeds;
@@ -335,7 +342,6 @@ extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
   p.relabeled = relabeled;
   p.num_unique = num_unique_dev;
 
-  hipStream_t st = static_cast<hipStream_t>(stream);
   const unsigned fill_blocks =
       static_cast<unsigned>(std::min<int64_t>(ceil_div((int64_t)(L.cap_max / 2 + (items + 15) / 16), kRelBlock), 8192));
   const unsigned item_blocks =
@@ -358,10 +364,94 @@ extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
     hipLaunchKernelGGL(relabel_lookup_kernel, dim3(nb), dim3(kRelBlock), 0, st, p);
     APT_LAUNCH_CHECK("relabel_lookup_kernel");
   }
+  return APT_OK;
+}
+
+}  // namespace apt
+
+extern "C" int apt_relabel(const int64_t* seeds, int64_t num_seeds,
+                           const int64_t* num_seeds_dev, const int64_t* neighbors,
+                           int64_t num_neighbors, int64_t neighbor_stride,
+                           int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev,
+                           int64_t* num_unique_host, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  using namespace apt;
+  int rc = relabel_check_args("apt_relabel", seeds, num_seeds, num_seeds_dev, neighbors, num_neighbors,
+                              neighbor_stride, unique, relabeled, num_unique_dev, kRelMaxItems);
+  if (rc != APT_OK) return rc;
+  const RelabelLayout L = relabel_layout(num_seeds + num_neighbors);
+  APT_REQUIRE(workspace != nullptr && workspace_bytes >= L.total, APT_EWORKSPACE,
+              "apt_relabel: workspace of %zu bytes, %zu needed", workspace_bytes, L.total);
+  APT_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, APT_EINVAL,
+              "apt_relabel: workspace must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = relabel_enqueue(seeds, num_seeds, num_seeds_dev, neighbors, num_neighbors, neighbor_stride, unique,
+                       relabeled, num_unique_dev, static_cast<char*>(workspace), st);
+  if (rc != APT_OK) return rc;
   if (num_unique_host != nullptr) {
     APT_HIP(hipMemcpyAsync(num_unique_host, num_unique_dev, sizeof(int64_t),
                            hipMemcpyDeviceToHost, st));
     APT_HIP(hipStreamSynchronize(st));
   }
   return APT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// apt_relabel_static: the same passes with the scratch in a fixed device array
+// of this library, for callers that cannot allocate (code under HIP graph
+// capture, serving loops, harnesses that forbid hipMalloc).  One array per GPU,
+// held until the process ends; every call on a GPU shares it, so calls that
+// overlap on one GPU (two streams, two threads) race.  Its contents after a call
+// are the last call's: nothing needs clearing between calls, because the fill
+// pass of every call resets exactly what its own passes read.
+namespace apt {
+
+constexpr int64_t kRelStaticMaxItems = int64_t{1} << 21;  // seeds + neighbours per call
+// relabel_layout(kRelStaticMaxItems).total: a table of 2^22 words (32 MiB), 6 bytes per item, 8 KiB of tile counts
+constexpr size_t kRelStaticBytes = (size_t{1} << 22) * 8 + (size_t{1} << 21) * 6 + (size_t{1} << 21) / kRelTile * 4;
+
+static __device__ __align__(256) unsigned char scratch[kRelStaticBytes];
+
+constexpr int kRelMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kRelMaxDevices] = {};  // per device: that GPU's copy of the array
+
+// Device address of the current GPU's array (resolved once per device, under the lock).
+static int static_scratch(char** out) {
+  int dev = -1;
+  APT_HIP(hipGetDevice(&dev));
+  APT_REQUIRE(dev >= 0 && dev < kRelMaxDevices, APT_ELIMIT, "apt_relabel_static: device %d outside [0, %d)", dev,
+              kRelMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    APT_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    APT_REQUIRE(ptr != nullptr && (reinterpret_cast<uintptr_t>(ptr) & 255) == 0, APT_EHIP,
+                "apt_relabel_static: the scratch array resolved to %p on device %d", ptr, dev);
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = static_cast<char*>(g_scratch_ptr[dev]);
+  return APT_OK;
+}
+
+}  // namespace apt
+
+extern "C" int64_t apt_relabel_static_max_items(void) { return apt::kRelStaticMaxItems; }
+
+extern "C" int apt_relabel_static(const int64_t* seeds, int64_t num_seeds, const int64_t* num_seeds_dev,
+                                  const int64_t* neighbors, int64_t num_neighbors, int64_t neighbor_stride,
+                                  int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev, void* stream) {
+  using namespace apt;
+  static_assert(kRelStaticBytes % 256 == 0, "scratch size keeps the layout's alignment");
+  int rc = relabel_check_args("apt_relabel_static", seeds, num_seeds, num_seeds_dev, neighbors, num_neighbors,
+                              neighbor_stride, unique, relabeled, num_unique_dev, kRelStaticMaxItems);
+  if (rc != APT_OK) return rc;
+  APT_REQUIRE(relabel_layout(num_seeds + num_neighbors).total <= kRelStaticBytes, APT_ELIMIT,
+              "apt_relabel_static: %lld items need more than the %zu bytes of fixed scratch",
+              (long long)(num_seeds + num_neighbors), kRelStaticBytes);
+  char* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != APT_OK) return rc;
+  return relabel_enqueue(seeds, num_seeds, num_seeds_dev, neighbors, num_neighbors, neighbor_stride, unique,
+                         relabeled, num_unique_dev, ws, static_cast<hipStream_t>(stream));
 }

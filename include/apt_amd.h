@@ -151,6 +151,25 @@ int apt_relabel(const int64_t* seeds, int64_t num_seeds,
                 int64_t* num_unique_host, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* apt_relabel without a workspace argument and without any allocation.
+ * No counterpart in the reference.  It is for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The scratch of the passes lives in a fixed device array inside
+ * the library (about 44 MiB per GPU, held until the process ends), so
+ *   - num_seeds + num_neighbors must not exceed apt_relabel_static_max_items()
+ *     (2^21); larger calls fail with APT_ELIMIT and enqueue nothing;
+ *   - every call on a GPU shares that GPU's array: calls that overlap on one
+ *     GPU (different streams or threads) race; calls on one stream do not;
+ *   - the first call on a device resolves the array's address (no allocation,
+ *     but make it outside a graph capture).
+ * Arguments and results as apt_relabel (no host copy of the count). */
+int64_t apt_relabel_static_max_items(void);
+int apt_relabel_static(const int64_t* seeds, int64_t num_seeds,
+                       const int64_t* num_seeds_dev, const int64_t* neighbors,
+                       int64_t num_neighbors, int64_t neighbor_stride,
+                       int64_t* unique, int64_t* relabeled,
+                       int64_t* num_unique_dev, void* stream);
+
 /* Feature tables as the reference registers them with cache_feats_shared
  * (src/cache_feats.cc:14-61, src/state.h:10-16).
  *   local_table  [num_local_rows, local_dim] elements ("uva_feats")
