@@ -15,10 +15,17 @@
 //     lanes of the group with shuffles);
 //   * unused output slots are written as -1 (the reference leaves garbage for
 //     degree-0 rows, :277).
+#include <hip/hip_ext.h>
+
 #include "common.hpp"
 #include "rank_table.hpp"
 
 namespace apt {
+
+// One-shot measurement hook (apt_time_next_sample): the next sampling launch of
+// this thread whose hop index matches records the two events on its dispatch.
+static thread_local hipEvent_t t_sample_start = nullptr, t_sample_stop = nullptr;
+static thread_local int t_sample_hop = -1;
 
 // Arguments of the fused relabel marking (see SampleParams).
 struct SampleMark {
@@ -290,15 +297,28 @@ static int launch_sample(const SampleParams& p, bool replace, int64_t blocks, si
   const dim3 grid(static_cast<unsigned>(blocks)), block(kSampleBlock);
   // rows of a group in flight at once: as many as it has, up to 4
   const int u = p.rows_per_group >= 4 ? 4 : (p.rows_per_group >= 2 ? 2 : 1);
-  if (replace) {
-    if (u == 4) hipLaunchKernelGGL((sample_kernel<LPS, true, 4>), grid, block, dyn_lds, st, p);
-    else if (u == 2) hipLaunchKernelGGL((sample_kernel<LPS, true, 2>), grid, block, dyn_lds, st, p);
-    else hipLaunchKernelGGL((sample_kernel<LPS, true, 1>), grid, block, dyn_lds, st, p);
-  } else {
-    if (u == 4) hipLaunchKernelGGL((sample_kernel<LPS, false, 4>), grid, block, dyn_lds, st, p);
-    else if (u == 2) hipLaunchKernelGGL((sample_kernel<LPS, false, 2>), grid, block, dyn_lds, st, p);
-    else hipLaunchKernelGGL((sample_kernel<LPS, false, 1>), grid, block, dyn_lds, st, p);
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  if (t_sample_hop == p.hop && (t_sample_start != nullptr || t_sample_stop != nullptr)) {
+    ev0 = t_sample_start;
+    ev1 = t_sample_stop;
+    t_sample_start = t_sample_stop = nullptr;
+    t_sample_hop = -1;
   }
+#define APT_SAMPLE_LAUNCH(RP, UU)                                                                       \
+  if (ev0 != nullptr || ev1 != nullptr)                                                                 \
+    hipExtLaunchKernelGGL((sample_kernel<LPS, RP, UU>), grid, block, dyn_lds, st, ev0, ev1, 0, p);      \
+  else                                                                                                  \
+    hipLaunchKernelGGL((sample_kernel<LPS, RP, UU>), grid, block, dyn_lds, st, p)
+  if (replace) {
+    if (u == 4) { APT_SAMPLE_LAUNCH(true, 4); }
+    else if (u == 2) { APT_SAMPLE_LAUNCH(true, 2); }
+    else { APT_SAMPLE_LAUNCH(true, 1); }
+  } else {
+    if (u == 4) { APT_SAMPLE_LAUNCH(false, 4); }
+    else if (u == 2) { APT_SAMPLE_LAUNCH(false, 2); }
+    else { APT_SAMPLE_LAUNCH(false, 1); }
+  }
+#undef APT_SAMPLE_LAUNCH
   APT_LAUNCH_CHECK("sample_kernel");
   return APT_OK;
 }
@@ -410,4 +430,11 @@ extern "C" int apt_sample_neighbors(const apt_graph* graph, const int64_t* front
   return apt::sample_launch(graph, frontier, num_frontier, num_frontier_dev, fanout, replace,
                             rng_seed, nullptr, hop, out_neighbors, out_counts, out_total,
                             static_cast<hipStream_t>(stream), "apt_sample_neighbors", nullptr);
+}
+
+extern "C" int apt_time_next_sample(int hop, void* start_event, void* stop_event) {
+  apt::t_sample_start = static_cast<hipEvent_t>(start_event);
+  apt::t_sample_stop = static_cast<hipEvent_t>(stop_event);
+  apt::t_sample_hop = (start_event != nullptr || stop_event != nullptr) ? hop : -1;
+  return APT_OK;
 }

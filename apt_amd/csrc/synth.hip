@@ -83,6 +83,66 @@ __global__ __launch_bounds__(kSynBlock) void copy_kernel(const uint4* __restrict
 
 }  // namespace apt
 
+namespace apt {
+
+__device__ __forceinline__ uint64_t probe_mix(uint64_t x) {
+  x *= 0x9E3779B97F4A7C15ull;
+  x ^= x >> 32;
+  x *= 0xD6E8FEB86659FD93ull;
+  x ^= x >> 32;
+  return x;
+}
+
+// One access per item to a pseudo-random word of a table: what bounds the
+// sampling and relabel kernels (one transaction per sampled id), as opposed to
+// bytes.  MODE 0 load, 1 store, 2 atomicMin without use of the result,
+// 3 atomicMin whose result is used, 4 16-byte load.
+template <int MODE>
+__global__ __launch_bounds__(kSynBlock) void random_access_kernel(uint32_t* table, uint64_t words, int64_t n,
+                                                                  uint32_t salt, uint32_t* sink) {
+  uint32_t acc = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * kSynBlock + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * kSynBlock) {
+    const uint64_t w = probe_mix(static_cast<uint64_t>(i) + (static_cast<uint64_t>(salt) << 40)) % words;
+    if (MODE == 0) acc += __builtin_nontemporal_load(&table[w]);
+    else if (MODE == 1) table[w] = static_cast<uint32_t>(i);
+    else if (MODE == 2) atomicMin(&table[w], static_cast<uint32_t>(i) | 0x80000000u);
+    else if (MODE == 3) acc += atomicMin(&table[w], static_cast<uint32_t>(i) | 0x80000000u);
+    else {
+      const uint4 v = *reinterpret_cast<const uint4*>(&table[w & ~uint64_t{3}]);
+      acc += v.x + v.w;
+    }
+  }
+  if (acc == 0x12345679u) sink[0] = acc;  // keeps the loads alive
+}
+
+}  // namespace apt
+
+extern "C" int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
+                                       uint32_t salt, void* sink, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(mode >= 0 && mode <= 4, APT_EINVAL, "apt_synth_random_access: mode %d outside 0..4", mode);
+  APT_REQUIRE(table != nullptr && sink != nullptr && table_bytes >= 16 && table_bytes % 16 == 0 &&
+                  (reinterpret_cast<uintptr_t>(table) & 15) == 0,
+              APT_EINVAL, "apt_synth_random_access: table must be 16-byte aligned, a multiple of 16 bytes long");
+  APT_REQUIRE(num_accesses >= 0, APT_EINVAL, "apt_synth_random_access: num_accesses < 0");
+  if (num_accesses == 0) return APT_OK;
+  const uint64_t words = static_cast<uint64_t>(table_bytes) / 4;
+  const dim3 grid(static_cast<unsigned>(std::min<int64_t>(ceil_div(num_accesses, kSynBlock), 16384))), block(kSynBlock);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* t = static_cast<uint32_t*>(table);
+  uint32_t* sk = static_cast<uint32_t*>(sink);
+  switch (mode) {
+    case 0: hipLaunchKernelGGL(random_access_kernel<0>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+    case 1: hipLaunchKernelGGL(random_access_kernel<1>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+    case 2: hipLaunchKernelGGL(random_access_kernel<2>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+    case 3: hipLaunchKernelGGL(random_access_kernel<3>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+    default: hipLaunchKernelGGL(random_access_kernel<4>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+  }
+  APT_LAUNCH_CHECK("random_access_kernel");
+  return APT_OK;
+}
+
 extern "C" int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream) {
   using namespace apt;
   APT_REQUIRE(bytes >= 0 && bytes % 16 == 0, APT_EINVAL, "apt_synth_copy: bytes must be a multiple of 16");

@@ -21,9 +21,13 @@ import sys
 import time
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes the gather kernel moves per gathered row, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this script (profiles/gather_kernel_full_pmc.txt); None where it has not been measured.
-MEASURED_GATHER_TRAFFIC_PER_ROW = {"full": 520.0}   # (190.5 MB + 184.7 MB) / 721651 rows
+# HBM bytes the gather kernel moves per gathered row, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this script, each scaled by what the same counter reads for the plain copy kernel.  Keyed by everything the
+# figure depends on, (workload, feature dtype, feature dim, batch); a run with any other combination reports
+# traffic null.  Each entry names the profiles/ file that holds the counter readings.
+MEASURED_GATHER_TRAFFIC_PER_ROW = {
+    ("full", "bf16", 128, 4096): (520.0, "profiles/gather_kernel_full_pmc.txt"),   # (190.5 MB + 184.7 MB) / 721651 rows
+}
 
 WORKLOADS = {
     # full-scale single GPU: 111M nodes, 3.2B directed edges, 128 x bf16, batch 4096
@@ -47,8 +51,8 @@ WORKLOADS = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="full", choices=sorted(WORKLOADS))
     ap.add_argument("--batch_size", type=int, default=None)
     ap.add_argument("--feature_dtype", default=None, choices=["fp32", "bf16"])
@@ -80,7 +84,139 @@ def parse_args():
                     help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
                          "cached feature table) and one step of the all-strategies dry run")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
+    ap.add_argument("--target_leg", default="auto", choices=["auto", "on", "off"],
+                    help="after the timed region also run batch 1024 on the same graph with 128 x bf16 and 128 x fp32 "
+                         "features (the shape the 60 %%-of-peak gather target is stated on) and report it under "
+                         "stages.target_shape; auto = only for workload full")
+    ap.add_argument("--target_steps", type=int, default=100)
+    ap.add_argument("--ceilings", default="auto", choices=["auto", "on", "off"],
+                    help="measure the GPU's rate for random 4-byte loads / stores / atomics (what bounds the sampling "
+                         "kernel) and quote the last hop's sampling kernel against it; auto = on")
     return ap.parse_args()
+
+def quantiles(xs):
+    """median / p10 / p90 / min / max of a list (nearest rank)."""
+    v = sorted(xs)
+    at = lambda q: v[min(len(v) - 1, max(0, int(round(q * (len(v) - 1)))))]
+    return {"median": at(0.5), "p10": at(0.1), "p90": at(0.9), "min": v[0], "max": v[-1], "n": len(v)}
+
+
+class KernelEvents:
+    """Pairs of HIP events that ride on a kernel dispatch (kernel begin / kernel end), see
+    apt_time_next_gather / apt_time_next_sample."""
+
+    def __init__(self):
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def pair(self):
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        assert self.hip.hipEventCreate(ctypes.byref(a)) == 0 and self.hip.hipEventCreate(ctypes.byref(b)) == 0
+        return a, b
+
+    def ms(self, pair, destroy=True):
+        ms = ctypes.c_float()
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), pair[0], pair[1])
+        assert rc == 0, f"hipEventElapsedTime -> {rc}"
+        if destroy:
+            self.hip.hipEventDestroy(pair[0])
+            self.hip.hipEventDestroy(pair[1])
+        return ms.value
+
+
+def gather_bytes_per_row(dim, esize, has_pos_map):
+    """-> (bytes the launch moves per row, the per-row figure of the roofline definition).  Row read + row
+    write + 8-byte id (+ the 8-byte position-map entry: the definition always counts it, the launch only reads
+    it when the store has a map; an identity store has none)."""
+    return 2 * dim * esize + 8 + (8 if has_pos_map else 0), 2 * dim * esize + 16
+
+
+def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, seed_n, store_of, synth, torch):
+    """Batch 1024 on the same graph with 128 x bf16 and 128 x fp32 rows: the shape the gather target
+    (>= 60 % of HBM peak) is stated on.  Every gather dispatch carries events; the sizes of every batch are
+    kept on the device and read afterwards, so each launch's rows and duration give its own fraction."""
+    B, Kt, Wt, H = 1024, args.target_steps, 20, len(hops)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed + 77)
+    out = {"batch": B, "batches": Kt, "warmup": Wt}
+    for name in ("bf16", "fp32"):
+        store = store_of(name)
+        esize = store.local_table.element_size()
+        moved, spec = gather_bytes_per_row(store.out_dim, esize, store.pos_map is not None)
+        pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused")
+        pool = torch.randperm(seed_n, generator=gen, device=dev)[:(Kt + Wt) * B]
+        sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(Kt + Wt)]
+        del pool
+        log = torch.zeros((Kt, H + 2), dtype=torch.int64, device=dev)
+        for i in range(Wt):
+            pipe.run(sets[i], args.seed + 5000 + i)
+        torch.cuda.synchronize()
+        pairs = []
+        step_ev = [torch.cuda.Event(enable_timing=True) for _ in range(Kt + 1)]
+        step_ev[0].record()
+        for i in range(Kt):
+            pipe.sample(sets[Wt + i], args.seed + 5000 + Wt + i)
+            pairs.append(kev.pair())
+            capi.check(capi.lib().apt_time_next_gather(*pairs[-1]))
+            pipe.gather()
+            log[i].copy_(pipe.sizes)
+            step_ev[i + 1].record()
+        torch.cuda.synchronize()
+        assert int(pipe.misses.item()) == 0
+        us = [kev.ms(pr) * 1e3 for pr in pairs]
+        rows = log[:, H].cpu().tolist()
+        edges = log[:, H + 1].cpu().tolist()
+        frac = [r * moved / (t * 1e-6) / 1e9 / HBM_PEAK_GBPS for r, t in zip(rows, us)]
+        step_ms = [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(Kt)]
+        # the same batches back to back without events or size copies: wall time per batch
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(Kt):
+            pipe.run(sets[Wt + i], args.seed + 5000 + Wt + i)
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / Kt
+        q_us, q_frac = quantiles(us), quantiles(frac)
+        out[name] = {
+            "rows": sum(rows) / Kt, "bytes_per_row": moved, "bytes_per_row_definition": spec,
+            "us_median": q_us["median"], "us_p10": q_us["p10"], "us_p90": q_us["p90"], "us_min": q_us["min"],
+            "us_max": q_us["max"],
+            # fraction of 8 TB/s of each launch (its own rows over its own duration); p10 = the slow end
+            "frac": q_frac["median"], "frac_p10": q_frac["p10"], "frac_p90": q_frac["p90"],
+            "frac_min": q_frac["min"], "frac_max": q_frac["max"],
+            "frac_by_definition_bytes": q_frac["median"] * spec / moved,
+            "GBps_median": q_frac["median"] * HBM_PEAK_GBPS,
+            "ms_per_step": wall * 1e3, "ms_per_step_events": quantiles(step_ms),
+            "edges_per_s": sum(edges) / Kt / wall,
+        }
+        del pipe, log, sets
+    return out
+
+
+def stage_ceilings(capi, dev, N, torch):
+    """The GPU's rate for one random 4-byte access per work item into a table of the rank table's size."""
+    nbytes = max(1 << 20, (N * 4 + 15) // 16 * 16)
+    table = torch.full((nbytes // 4,), -1, dtype=torch.int32, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    n = 8_000_000
+    res = {"table_bytes": nbytes, "accesses_per_launch": n}
+    for mode, name in ((0, "load"), (1, "store"), (2, "atomic_min"), (3, "atomic_min_returning"), (4, "load_16B")):
+        ts = []
+        for rep in range(7):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            capi.check(capi.lib().apt_synth_random_access(mode, capi._ptr(table), nbytes, n, rep + 1,
+                                                          capi._ptr(sink), capi._stream()))
+            e1.record()
+            torch.cuda.synchronize()
+            if rep >= 2:
+                ts.append(e0.elapsed_time(e1) * 1e-3)
+        ts.sort()
+        res[name + "_G_per_s"] = n / ts[len(ts) // 2] / 1e9
+    del table, sink
+    return res
+
 
 def seconds_per_call(torch, fn, reps=10, warm=3):
     """Mean duration of fn() on the current stream: `reps` back-to-back calls between two events."""
@@ -430,30 +566,18 @@ def main():
     ev = lambda: torch.cuda.Event(enable_timing=True)
     staged = args.driver != "graph"   # a graph replay cannot be bracketed stage by stage
 
-    # HIP events that ride on the gather dispatch itself (kernel begin / kernel end)
-    hip = ctypes.CDLL("libamdhip64.so")
-    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
-    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
-    hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+    kev = KernelEvents()           # HIP events that ride on a kernel's dispatch (kernel begin / kernel end)
+    H = len(hops)
 
-    def kernel_events():
-        a, b = ctypes.c_void_p(), ctypes.c_void_p()
-        assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
-        return a, b
-
-    def kernel_ms(pair):
-        ms = ctypes.c_float()
-        rc = hip.hipEventElapsedTime(ctypes.byref(ms), pair[0], pair[1])
-        assert rc == 0, f"hipEventElapsedTime -> {rc}"
-        return ms.value
-
-    def run_step(p, i, kev=None):
+    def run_step(p, i, gk=None, sk=None):
         seeds, key = seed_sets[i], args.seed + 100 + i
-        if kev is None:
+        if gk is None:
             p.run(seeds, key)
             return
+        if sk is not None:   # the last hop's sampling kernel records its begin / end
+            capi.check(capi.lib().apt_time_next_sample(H - 1, sk[0], sk[1]))
         p.sample(seeds, key)
-        capi.check(capi.lib().apt_time_next_gather(kev[0], kev[1]))   # the gather dispatch records its begin / end
+        capi.check(capi.lib().apt_time_next_gather(gk[0], gk[1]))   # the gather dispatch records its begin / end
         p.gather()
 
     # ---- warm-up
@@ -464,26 +588,37 @@ def main():
     # ---- timed region: exactly K steps on one stream.  Gather dispatches carry two HIP events that the
     # GPU stamps when the kernel begins and ends (no extra packets on the stream); what is left of the
     # region is sampling + relabel, dispatch gaps included.  Such a dispatch costs the host a little more
-    # to enqueue, which would show in launch-bound small workloads, so up to 16 evenly spaced steps carry them.
-    every = max(1, -(-K // 16))
-    kevs = [kernel_events() if staged and i % every == 0 else None for i in range(K)]
+    # to enqueue, which would show in launch-bound small workloads, so up to 32 evenly spaced steps carry them
+    # (and the last hop's sampling kernel of the same steps).
+    every = max(1, -(-K // 32))
+    timed_steps = [i for i in range(K) if staged and i % every == 0]
+    gkevs = {i: kev.pair() for i in timed_steps}
+    skevs = {i: kev.pair() for i in timed_steps} if args.driver == "fused" else {}
     start, stop = ev(), ev()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start.record()
     for i in range(K):
-        run_step(pipe, W + i, kevs[i])
+        run_step(pipe, W + i, gkevs.get(i), skevs.get(i))
     stop.record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    sample_us = None
     if staged:
-        timed = [k for k in kevs if k is not None]
-        gather_ms = sorted(kernel_ms(k) for k in timed)
-        t_gather = sum(gather_ms) / len(timed) * K
+        gather_ms = sorted(kev.ms(gkevs[i]) for i in timed_steps)
+        t_gather = sum(gather_ms) / len(gather_ms) * K
         t_sample = start.elapsed_time(stop) - t_gather
-        for a, b in timed:
-            hip.hipEventDestroy(a)
-            hip.hipEventDestroy(b)
+        if skevs:
+            sample_us = {i: kev.ms(skevs[i]) * 1e3 for i in timed_steps}
+
+    # ---- the same K steps once more, one event between steps: the spread of the per-step time
+    marks = [ev() for _ in range(K + 1)]
+    marks[0].record()
+    for i in range(K):
+        run_step(pipe, W + i)
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    per_step_ms = quantiles([marks[i].elapsed_time(marks[i + 1]) for i in range(K)])
 
     if args.calibration_copy_mib > 0:
         a = torch.ones(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev)
@@ -496,6 +631,7 @@ def main():
     # graph driver this pass also provides the stage timings
     edges = rows = 0
     hop_sizes = []
+    last_hop = {}        # step -> (frontier rows, sampled edges) of the last hop, for the steps whose kernel was timed
     if not staged:
         t_sample = t_gather = 0.0
     for i in range(K):
@@ -510,11 +646,15 @@ def main():
             t_sample += m[0].elapsed_time(m[1])
             t_gather += m[1].elapsed_time(m[2])
         sizes = stage_pipe.sizes.cpu().tolist()
+        if sample_us is not None and i in sample_us:
+            last_hop[i] = (sizes[H - 1], int(stage_pipe.counts[H - 1][:sizes[H - 1]].sum().item()))
         edges += sizes[-1]
         rows += sizes[len(hops)] if requests is None else int(stage_pipe.request_sizes[0].item())
         hop_sizes.append(sizes[:-1])
     request_sizes = None if requests is None else stage_pipe.request_sizes.cpu().tolist()
-    bytes_per_row = 2 * w["dim"] * esize + 16          # row read + row write + id + position
+    # bytes per gathered row: what the launch moves (an identity store has no position map to read) and the
+    # figure of the roofline definition (always 16 bytes of id + position)
+    bytes_per_row, bytes_per_row_def = gather_bytes_per_row(w["dim"], esize, store.pos_map is not None)
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
 
@@ -595,6 +735,54 @@ def main():
                                  hops=hops, indices=indices, indptr=indptr, K=K, lo=lo, min_vids=min_vids, N=N,
                                  P=P, pos_map=pos_map, requests=requests, seed_sets=seed_sets, torch=torch, W=W)
 
+    # ---- the north-star sentence's own shape: batch 1024 on this graph, bf16 and fp32 rows
+    target = None
+    if args.target_leg == "on" or (args.target_leg == "auto" and args.workload == "full" and requests is None):
+        extra = {}
+
+        def store_of(name):
+            want = torch.bfloat16 if name == "bf16" else torch.float32
+            if feats.dtype == want:
+                return store
+            extra.clear()                                  # one extra table at a time
+            extra[name] = synth.random_features(N, w["dim"], want, args.seed + 1, dev)
+            return capi.FeatStore(extra[name])
+
+        target = stage_target_shape(args=args, capi=capi, dev=dev, graph=graph, hops=hops, kev=kev,
+                                    MiniBatchPipeline=MiniBatchPipeline, N=N, seed_n=seed_n, store_of=store_of,
+                                    synth=synth, torch=torch)
+        extra.clear()
+        torch.cuda.empty_cache()
+
+    # ---- what bounds the sampling kernel: random transactions.  The GPU's rate for them, measured here.
+    ceilings = stage_ceilings(capi, dev, N, torch) if args.ceilings != "off" else None
+    roofline_sampling = None
+    if sample_us and last_hop:
+        steps_ = sorted(last_hop)
+        us_ = [sample_us[i] for i in steps_]
+        r_ = sum(last_hop[i][0] for i in steps_) / len(steps_)
+        e_ = sum(last_hop[i][1] for i in steps_) / len(steps_)
+        t_ = sum(us_) / len(us_) * 1e-6
+        alg = 24 * r_ + 16 * e_ + (8 * r_ if graph.adj_pos_map is not None else 0)
+        # per frontier row one random line for its indptr pair, per sampled slot one random index load and one
+        # random rank-table read (atomics for the slots that bid come on top and are not counted here)
+        acc = r_ + 2 * e_
+        q = quantiles(us_)
+        roofline_sampling = {
+            "bound": "hbm", "kernel": f"sample_kernel, hop {H} of {H} (fanout {hops[-1]}), rank-table bids included",
+            "achieved": alg / t_ / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / t_ / 1e9 / HBM_PEAK_GBPS,
+            "traffic": None, "algorithmic_bytes_per_launch": alg, "bytes_per_row": "24 + 16 k, k = min(fanout, degree)",
+            "rows_per_launch": r_, "edges_per_launch": e_, "avg_launch_us": t_ * 1e6,
+            "launch_us_min_median_max": [q["min"], q["median"], q["max"]],
+            "random_accesses_per_launch": acc, "random_accesses_G_per_s": acc / t_ / 1e9,
+            "random_load_ceiling_G_per_s": ceilings["load_G_per_s"] if ceilings else None,
+            "frac_of_random_load_ceiling": acc / t_ / 1e9 / ceilings["load_G_per_s"] if ceilings else None,
+            "timing": f"HIP events carried by {len(steps_)} of the {K} dispatches of the timed region",
+        }
+
+    tkey = (args.workload, w["dtype"], w["dim"], B)
+    traffic_row = MEASURED_GATHER_TRAFFIC_PER_ROW.get(tkey) if not args.fan_out and requests is None else None
+
     out = {
         "metric": "sampled edges/s (3-hop 15,10,5) + feature-gather GB/s as % of HBM peak",
         "value": edges_per_s,
@@ -615,29 +803,37 @@ def main():
                         f"{'with' if args.replace else 'without'} replacement, relabel per hop, "
                         f"gather of all input nodes" + part_note,
             "batch": B, "fan_out": w["fan_out"], "feature_dtype": w["dtype"], "driver": args.driver,
+            "graph": "R-MAT a=.57 b=.19 c=.19, CSR built on the GPU: multigraph rows (an id may repeat in a row), "
+                     "unsorted, no dedup",
         },
         "roofline": {
             "bound": "hbm", "kernel": "gather_kernel",
             "achieved": gather_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": gather_gbps / HBM_PEAK_GBPS,
-            "traffic": (MEASURED_GATHER_TRAFFIC_PER_ROW[args.workload] * rows / K
-                        if args.workload in MEASURED_GATHER_TRAFFIC_PER_ROW and not args.fan_out
-                        and not args.batch_size else None),
+            "traffic": traffic_row[0] * rows / K if traffic_row else None,
+            "traffic_source": traffic_row[1] if traffic_row else None,
             "algorithmic_bytes_per_launch": bytes_per_row * rows / K,
             "bytes_per_row": bytes_per_row, "rows_per_launch": rows / K,
+            # the roofline definition charges 16 bytes of id + position per row whether or not the store has a
+            # position map; achieved / frac above use the bytes this launch moves
+            "bytes_per_row_definition": bytes_per_row_def,
+            "frac_by_definition_bytes": gather_gbps / HBM_PEAK_GBPS * bytes_per_row_def / bytes_per_row,
             "avg_launch_us": t_gather / K * 1e3,
             "launch_us_min_median_max": ([gather_ms[0] * 1e3, gather_ms[len(gather_ms) // 2] * 1e3,
                                           gather_ms[-1] * 1e3] if staged else None),
-            "timing": (f"HIP events carried by {len(timed)} of the {K} gather dispatches of the timed region "
+            "timing": (f"HIP events carried by {len(timed_steps)} of the {K} gather dispatches of the timed region "
                        f"(kernel begin / end)" if staged else "HIP events recorded around each gather launch of an untimed pass"),
-
         },
+        "roofline_sampling": roofline_sampling,
         "cpu_baseline": cpu,
         "aggregation": agg,
         "block_formats": fmt,
         "cache_build": cache_build,
         "shuffle": shuffle,
         "stages": {
+            "target_shape": target,
+            "per_step_ms": per_step_ms,
+            "random_access_ceilings": ceilings,
             "in_flight": in_flight,
             "edges_per_step": edges / K,
             "input_nodes_per_step": rows / K,

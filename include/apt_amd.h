@@ -217,6 +217,11 @@ int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
  * hipEventRecord bracket includes.  Both are hipEvent_t created by the caller;
  * one-shot; NULL, NULL cancels. */
 int apt_time_next_gather(void* start_event, void* stop_event);
+/* The same hook for the sampling kernel: the next sampling launch made by the
+ * calling thread with hop index `hop` (apt_sample_neighbors, or that hop inside
+ * apt_minibatch_sample) records the two events on its dispatch.  One-shot;
+ * NULL, NULL cancels. */
+int apt_time_next_sample(int hop, void* start_event, void* stop_event);
 
 /* Row permutation of a dense [rows, dim] table, the on-GPU halves of
  * FeatShuffle (src/feat_shuffle.cc:9-30) and the row gather by inverse_idx in

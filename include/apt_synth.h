@@ -31,6 +31,18 @@ int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_rows, int64_t row_beg
  * the FETCH_SIZE / WRITE_SIZE hardware counters. */
 int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
+/* Random-access probe: num_accesses accesses, one per work item, each to a
+ * pseudo-random 4-byte word of `table` (device memory, table_bytes long).
+ * The sampling and relabel kernels are bound by the number of such
+ * transactions, not by bytes; the benchmark measures the GPU's rate for them
+ * with this call and quotes the kernels against it.
+ *   mode  0 load, 1 store, 2 atomicMin (result unused), 3 atomicMin (result
+ *         used), 4 aligned 16-byte load
+ *   salt  varies the address sequence between calls
+ *   sink  device uint32[1] (never written in practice; keeps loads alive) */
+int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
+                            uint32_t salt, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
