@@ -36,6 +36,7 @@ struct GatherParams {
   int scatter;               // 1: out[index[r]] = in[r] (pack); rows come from local_table
   int64_t num_out_rows;      // scatter only
   uint8_t* named;            // scatter only, optional: named[v] = 1 for every output row v that is written
+  int store_policy;          // kStore* (apt_set_tuning gather_store_policy)
 };
 
 template <int V> struct VecT;
@@ -63,6 +64,29 @@ __device__ __forceinline__ const char* source_row(const GatherParams& p, int64_t
   }
   if (v >= p.num_local_rows) return nullptr;
   return p.local_table + v * p.local_row_bytes + p.col_offset_bytes;
+}
+
+// How a lane stores its 16 bytes of a gathered row.
+//   0 (shipped)  write-through: the line goes on to memory as it is written
+//                instead of staying dirty in this XCD's L2 until the release at
+//                the end of the kernel writes the whole L2 back; what that
+//                write-back costs shows on short launches (24.5 against 25.9 us
+//                on 235 k rows of 256 bytes, 25.0 against 26.5 us on 124 k rows of
+//                400 bytes; nothing on 700 k rows and more)
+//   1            non-temporal store (streaming hint only)
+//   2            plain store
+// Narrower vectors (row geometry not 16-byte aligned) always use 1.
+enum : int { kStoreWriteThrough = 0, kStoreNonTemporal = 1, kStorePlain = 2 };
+
+template <int V>
+__device__ __forceinline__ void store_row_vec(typename VecT<V>::type val, typename VecT<V>::type* dst, int policy) {
+  if (V == 16 && policy == kStoreWriteThrough) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(val) : "memory");
+  } else if (policy == kStorePlain) {
+    *dst = val;
+  } else {
+    __builtin_nontemporal_store(val, dst);
+  }
 }
 
 // LPR lanes per row, R rows per group per step, V bytes per lane access.
@@ -111,8 +135,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
       }
 #pragma unroll
       for (int k = 0; k < R; ++k) {
-        if (dst[k] != nullptr)
-          __builtin_nontemporal_store(val[k], reinterpret_cast<Vec*>(dst[k]) + c);
+        if (dst[k] != nullptr) store_row_vec<V>(val[k], reinterpret_cast<Vec*>(dst[k]) + c, p.store_policy);
       }
     }
   }
@@ -137,6 +160,7 @@ struct TimingArm {
 int tuning_gather_rows();        // 0 = default
 int tuning_gather_max_blocks();  // 0 = default
 int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
+int tuning_gather_store_policy();
 
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
@@ -253,6 +277,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.scatter = 0;
   p.num_out_rows = 0;
   p.named = nullptr;
+  p.store_policy = tuning_gather_store_policy();
   arm.rearm();
   return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
 }
@@ -293,6 +318,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
   p.scatter = scatter;
   p.num_out_rows = scatter ? num_rows_other : 0;
   p.named = named;
+  p.store_policy = tuning_gather_store_policy();
   arm.rearm();
   return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
 }

@@ -28,6 +28,8 @@ static int g_sample_min_workgroups = 0;
 int tuning_sample_min_workgroups() { return g_sample_min_workgroups; }
 static int g_gather_vector_bytes = 0;
 int tuning_gather_vector_bytes() { return g_gather_vector_bytes; }
+static int g_gather_store_policy = 0;
+int tuning_gather_store_policy() { return g_gather_store_policy; }
 static int g_block_fused_scan = 1;
 int tuning_block_fused_scan() { return g_block_fused_scan; }
 
@@ -74,6 +76,12 @@ extern "C" int apt_set_tuning(const char* key, int value) {
     if (value != 0 && value != 2 && value != 4 && value != 8 && value != 16)
       return apt::fail(APT_EINVAL, "apt_set_tuning: gather_vector_bytes must be 0, 2, 4, 8 or 16");
     apt::g_gather_vector_bytes = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "gather_store_policy") == 0) {
+    if (value < 0 || value > 2)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: gather_store_policy must be 0 (write-through), 1 (non-temporal) or 2 (plain)");
+    apt::g_gather_store_policy = value;
     return APT_OK;
   }
   if (std::strcmp(key, "block_fused_scan") == 0) {

@@ -89,6 +89,8 @@ def parse_args():
                          "features (the shape the 60 %%-of-peak gather target is stated on) and report it under "
                          "stages.target_shape; auto = only for workload full")
     ap.add_argument("--target_steps", type=int, default=100)
+    ap.add_argument("--event_steps", type=int, default=32,
+                    help="how many (evenly spaced) steps of the timed region carry kernel events")
     ap.add_argument("--ceilings", default="auto", choices=["auto", "on", "off"],
                     help="measure the GPU's rate for random 4-byte loads / stores / atomics (what bounds the sampling "
                          "kernel) and quote the last hop's sampling kernel against it; auto = on")
@@ -588,9 +590,9 @@ def main():
     # ---- timed region: exactly K steps on one stream.  Gather dispatches carry two HIP events that the
     # GPU stamps when the kernel begins and ends (no extra packets on the stream); what is left of the
     # region is sampling + relabel, dispatch gaps included.  Such a dispatch costs the host a little more
-    # to enqueue, which would show in launch-bound small workloads, so up to 32 evenly spaced steps carry them
+    # to enqueue, which would show in launch-bound small workloads, so a limited number of evenly spaced steps (--event_steps) carry them
     # (and the last hop's sampling kernel of the same steps).
-    every = max(1, -(-K // 32))
+    every = max(1, -(-K // max(1, args.event_steps)))
     timed_steps = [i for i in range(K) if staged and i % every == 0]
     gkevs = {i: kev.pair() for i in timed_steps}
     skevs = {i: kev.pair() for i in timed_steps} if args.driver == "fused" else {}

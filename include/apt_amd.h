@@ -60,6 +60,9 @@ int apt_abi_version(void);
  *   "gather_max_blocks"      cap on the gather grid (rows are strided over)
  *   "gather_vector_bytes"    2|4|8|16: widest load/store a lane of the gather uses
  *                            (16 = global_load_dwordx4 where alignment allows)
+ *   "gather_store_policy"    how the gather stores a row's 16-byte pieces: 0 (default;
+ *                            0 here is a value, not "default of the day") write-through
+ *                            stores, 1 non-temporal stores, 2 plain stores
  *   "minibatch_payload_bits" width of the id field of rank-table entries (0 = as
  *                            narrow as the plan allows); wider = fewer epochs
  *                            between table refills (used to test the refill)
