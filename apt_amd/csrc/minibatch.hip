@@ -71,6 +71,7 @@ struct HopParams {
   const uint32_t* state;     // [0] epoch, [1] payload bits (see mb_begin_kernel)
   int last;                  // last hop: ids are not written back to the table
   int64_t* nodes;            // growing unique list
+  int64_t nodes_cap;         // its capacity: an id beyond it (counters corrupted by the caller) is dropped, not written
   int64_t* n_next;           // receives the size of the list after this hop
   uint64_t* flags;           // owner bit per item, one word per wavefront-load
   uint32_t* tile_cnt;
@@ -144,11 +145,11 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, in
 template <bool FIRST>
 __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p) {
   const HopSizes s = hop_sizes(p);
-  const uint32_t tb = table_base(p.state);
+  const RankEpoch ep = rank_epoch(p.state);
   const RankTable t{p.table, p.table_len, p.state, p.displaced};
   for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < s.nn;
        j += static_cast<int64_t>(gridDim.x) * kMbBlock)
-    p.relabeled[j] = rank_table_bid(t, tb, FIRST, p.neighbors[j], s.ns, j);
+    p.relabeled[j] = rank_table_bid(t, ep, FIRST, p.neighbors[j], s.ns, j);
 }
 
 // Item i of a hop: FIRST -> seeds followed by neighbours (index = bid);
@@ -253,8 +254,10 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
         v = p.neighbors[i];
         p.relabeled[i] = id;
       }
-      p.nodes[id] = v;
-      if (!p.last) p.table[v] = table_base(p.state) + static_cast<uint32_t>(id);
+      if (id < p.nodes_cap) {
+        p.nodes[id] = v;
+        if (!p.last) p.table[v] = table_base(p.state) + static_cast<uint32_t>(id);
+      }
     }
   }
   if (blockIdx.x == tiles - 1 && threadIdx.x == 0) *p.n_next = running;
@@ -454,6 +457,7 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
   hp.table_len = rank_table_len;
   hp.state = state;
   hp.nodes = nodes;
+  hp.nodes_cap = L.caps[num_hops];
   hp.flags = reinterpret_cast<uint64_t*>(ws + L.flags_off);
   hp.tile_cnt = reinterpret_cast<uint32_t*>(ws + L.tile_off);
   hp.displaced = reinterpret_cast<uint8_t*>(ws + L.displaced_off);

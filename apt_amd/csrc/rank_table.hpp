@@ -23,6 +23,20 @@ struct RankTable {
 // Smallest entry value of the current batch.
 __device__ __forceinline__ uint32_t table_base(const uint32_t* state) { return state[0] << state[1]; }
 
+// The epoch state of a batch, read once per kernel: it does not change while a
+// batch's kernels run, but the compiler cannot know that and would fetch it from
+// memory again after every atomic (a dependent load on the path of every bid).
+struct RankEpoch {
+  uint32_t epoch, bits, base;   // base = epoch << bits, the smallest entry value of the batch
+};
+__device__ __forceinline__ RankEpoch rank_epoch(const uint32_t* state) {
+  RankEpoch e;
+  e.epoch = state[0];
+  e.bits = state[1];
+  e.base = e.epoch << e.bits;
+  return e;
+}
+
 // Slot j (of ns * fanout) of a hop with ns frontier rows sampled node v.
 //   v already in the batch (id < ns in the table)  -> its id, no atomic;
 //   otherwise bid ns + j: the smallest bid owns the node.  A returning
@@ -34,8 +48,9 @@ __device__ __forceinline__ uint32_t table_base(const uint32_t* state) { return s
 //   never flagged.)
 // first_hop: the table holds seed indices, not ids, so hits cannot be resolved
 // yet and ownership is decided by re-reading the table; no flags are kept.
-__device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, uint32_t tb, bool first_hop,
+__device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const RankEpoch& ep, bool first_hop,
                                                   int64_t v, int64_t ns, int64_t j) {
+  const uint32_t tb = ep.base;
   if (v < 0) return v <= kSlotOwner ? -1 : v;  // padding; never one of the two states above
   if (v >= t.len) return -1;  // an id the table cannot hold: treated as padding
   const uint32_t first_bid = tb + static_cast<uint32_t>(ns);
@@ -53,7 +68,7 @@ __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, uint32_t t
   if (old < bid) return old < first_bid ? static_cast<int64_t>(old - tb) : kSlotLoser;
   // old > bid: this slot is the smallest so far.  If old belongs to this batch it
   // is a bid of this hop (ids are below first_bid): that slot has been displaced.
-  if ((old >> t.state[1]) == t.state[0]) t.displaced[old - first_bid] = 1;
+  if ((old >> ep.bits) == ep.epoch) t.displaced[old - first_bid] = 1;
   return kSlotOwner;
 }
 

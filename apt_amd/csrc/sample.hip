@@ -135,6 +135,8 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   const int tile = G * p.rows_per_group;
   if (static_cast<int64_t>(blockIdx.x) * tile >= n) return;  // block-uniform
   const uint64_t seed = p.seed_dev != nullptr ? *p.seed_dev : p.seed;
+  RankEpoch ep{0, 0, 0};
+  if (p.table.entries != nullptr) ep = rank_epoch(p.table.state);
 
   const int tid = threadIdx.x;
   const int grp = tid / LPS;
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
           // First hop of the fused driver: the row's seed bids for its node with
           // its own index, like its neighbours below (seeds may repeat).
           if (p.first_hop != 0 && p.table.entries != nullptr && l == 0 && node >= 0 && node < p.table.len)
-            atomicMin(&p.table.entries[node], table_base(p.table.state) + static_cast<uint32_t>(gis[u]));
+            atomicMin(&p.table.entries[node], ep.base + static_cast<uint32_t>(gis[u]));
           pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, node, seed, p.hop);
           if (l == 0) {
             const int64_t cnt = REPLACE ? (deg > 0 ? fanout : 0) : (deg < fanout ? deg : fanout);
@@ -211,12 +213,11 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
       for (int u = 0; u < U; ++u)
         if (gis[u] < n && l < fanout) p.out[gis[u] * fanout + l] = val[u];
       if (p.table.entries != nullptr) {
-        const uint32_t tb = table_base(p.table.state);
         int64_t rel[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
           rel[u] = (gis[u] < n && l < fanout)
-                       ? rank_table_bid(p.table, tb, p.first_hop != 0, val[u], n, gis[u] * fanout + l)
+                       ? rank_table_bid(p.table, ep, p.first_hop != 0, val[u], n, gis[u] * fanout + l)
                        : -1;
 #pragma unroll
         for (int u = 0; u < U; ++u)
