@@ -45,6 +45,15 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   Tensor rank_table, mb_workspace;
   int64_t mb_batch = -1;
   std::vector<int64_t> mb_fanouts;
+  // sample_blocks' output buffers (upper-bound sized), handed out in turn: what call k returned stays
+  // untouched until call k + ring; ring 0 = fresh tensors on every call
+  struct BlockBuffers {
+    Tensor nodes, sizes, format_ws;
+    std::vector<Tensor> nb, rl, ct, row, col, csc;
+    bool formats = false;
+  };
+  std::vector<BlockBuffers> mb_ring;
+  int64_t mb_ring_size = 2, mb_ring_pos = 0;
 };
 
 State& S() {
@@ -92,6 +101,14 @@ void SetRngSeed(IdType seed) {
 }
 
 void SetStrict(bool strict) { S().strict = strict; }
+
+// How many sets of output buffers sample_blocks hands out in turn (0 = fresh tensors on every call).
+void SetBlockBufferRing(IdType sets) {
+  TORCH_CHECK(sets >= 0 && sets <= 64, "npc: set_block_buffer_ring: 0..64 sets");
+  S().mb_ring_size = sets;
+  S().mb_ring.clear();
+  S().mb_ring_pos = 0;
+}
 
 // reference src/cache_feats.cc:14-61
 void CacheFeatsShared(IdType num_total_nodes, Tensor localnode_feats, Tensor cached_feats,
@@ -270,14 +287,54 @@ std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts,
     cap[h] = apt_minibatch_capacity(B, fan.data(), H, h);
     TORCH_CHECK(cap[h] > 0, "npc: sample_blocks: unsupported batch / fanouts");
   }
-  auto nodes = torch::empty({cap[H]}, i64_opts());
-  auto sizes = torch::zeros({H + 2 + (with_formats ? H : 0)}, i64_opts());
-  std::vector<Tensor> nb(H), rl(H), ct(H);
+  // Output buffers at their upper bounds: a set of the ring (reused, see State::mb_ring) or fresh ones.
+  State::BlockBuffers fresh;
+  State::BlockBuffers* bufp = &fresh;
+  if (s.mb_ring_size > 0) {
+    if (static_cast<int64_t>(s.mb_ring.size()) != s.mb_ring_size) s.mb_ring.assign(s.mb_ring_size, State::BlockBuffers());
+    bufp = &s.mb_ring[s.mb_ring_pos];
+    s.mb_ring_pos = (s.mb_ring_pos + 1) % s.mb_ring_size;
+  }
+  State::BlockBuffers& b = *bufp;
+  const bool fits = b.nodes.defined() && b.nodes.numel() == cap[H] && static_cast<int>(b.nb.size()) == H &&
+                    b.sizes.numel() == H + 2 + (with_formats ? H : 0) && (!with_formats || b.formats) &&
+                    [&] {
+                      for (int h = 0; h < H; ++h)
+                        if (b.nb[h].numel() != cap[h] * fan[h] || b.ct[h].numel() != cap[h]) return false;
+                      return true;
+                    }();
+  if (!fits) {
+    b = State::BlockBuffers();
+    b.nodes = torch::empty({cap[H]}, i64_opts());
+    b.sizes = torch::empty({H + 2 + (with_formats ? H : 0)}, i64_opts());
+    b.nb.resize(H); b.rl.resize(H); b.ct.resize(H);
+    for (int h = 0; h < H; ++h) {
+      b.nb[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+      b.rl[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+      b.ct[h] = torch::empty({cap[h]}, i64_opts());
+    }
+    if (with_formats) {
+      size_t need = 256;
+      for (int h = 0; h < H; ++h) {
+        const size_t bytes = apt_block_workspace_bytes(cap[h], fan[h], cap[h + 1], 0);
+        TORCH_CHECK(bytes > 0, "npc: sample_blocks: block sizes out of range");
+        need = std::max(need, bytes);
+      }
+      b.format_ws = torch::empty({static_cast<int64_t>(need)}, u8);   // the hops run one after the other
+      b.row.resize(H); b.col.resize(H); b.csc.resize(H);
+      for (int h = 0; h < H; ++h) {
+        b.row[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+        b.col[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
+        b.csc[h] = torch::empty({cap[h] + 1}, i64_opts());
+      }
+      b.formats = true;
+    }
+  }
+  b.sizes.zero_();
+  Tensor &nodes = b.nodes, &sizes = b.sizes;
+  std::vector<Tensor>&nb = b.nb, &rl = b.rl, &ct = b.ct, &row = b.row, &col = b.col, &csc = b.csc;
   std::vector<int64_t*> nbp(H), rlp(H), ctp(H);
   for (int h = 0; h < H; ++h) {
-    nb[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
-    rl[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
-    ct[h] = torch::empty({cap[h]}, i64_opts());
     nbp[h] = nb[h].data_ptr<int64_t>();
     rlp[h] = rl[h].data_ptr<int64_t>();
     ctp[h] = ct[h].data_ptr<int64_t>();
@@ -289,24 +346,13 @@ std::vector<Tensor> SampleBlocks(Tensor seeds, std::vector<int64_t> hop_fanouts,
                                       static_cast<size_t>(s.mb_workspace.numel()), stream());
   if (rc != APT_OK) s.mb_workspace = Tensor();  // re-initialised by the next call
   check(rc);
-  std::vector<Tensor> row(H), col(H), csc(H);
   if (with_formats) {
-    size_t need = 256;
-    for (int h = 0; h < H; ++h) {
-      const size_t b = apt_block_workspace_bytes(cap[h], fan[h], cap[h + 1], 0);
-      TORCH_CHECK(b > 0, "npc: sample_blocks: block sizes out of range");
-      need = std::max(need, b);
-    }
-    auto ws = torch::empty({static_cast<int64_t>(need)}, u8);   // the hops run one after the other
     int64_t* dev_sizes = sizes.data_ptr<int64_t>();
-    for (int h = 0; h < H; ++h) {
-      row[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
-      col[h] = torch::empty({cap[h] * fan[h]}, i64_opts());
-      csc[h] = torch::empty({cap[h] + 1}, i64_opts());
+    for (int h = 0; h < H; ++h)
       check(apt_block_formats(rlp[h], cap[h], dev_sizes + h, fan[h], cap[h + 1], row[h].data_ptr<int64_t>(),
                               col[h].data_ptr<int64_t>(), csc[h].data_ptr<int64_t>(), dev_sizes + H + 2 + h, nullptr,
-                              nullptr, nullptr, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream()));
-    }
+                              nullptr, nullptr, b.format_ws.data_ptr(), static_cast<size_t>(b.format_ws.numel()),
+                              stream()));
   }
   auto host = sizes.cpu();  // the one wait of the batch
   const int64_t* hs = host.data_ptr<int64_t>();
@@ -542,6 +588,18 @@ Tensor FeatShuffle(Tensor inputs, Tensor send_offset, Tensor recv_offset, Tensor
                          torch::TensorOptions().dtype(torch::kUInt8).device(device()));
   check(apt_scatter_rows(x.data_ptr(), i64(perm), perm.numel(), feat_dim, static_cast<int>(x.element_size()),
                          out.data_ptr(), n_out, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream()));
+  if (S().strict) {
+    // The reference's pack is index_select_backward (src/feat_shuffle.cc:14-16): rows named more than once
+    // add up.  The scatter keeps one of them, which is the same thing only for a permutation without
+    // repeats (what ShuffleSeeds produces).  The flags tell: as many rows named as entries <=> no repeats and
+    // nothing out of range; otherwise the sum is formed the reference's way.
+    const int64_t named = ws.narrow(0, 0, n_out).sum().item<int64_t>();
+    if (named != perm.numel()) {
+      TORCH_CHECK_INDEX(perm.numel() == 0 || (perm.min().item<int64_t>() >= 0 && perm.max().item<int64_t>() < n_out),
+                        "npc: feat_shuffle: permutation entry outside [0, ", n_out, ")");
+      out = torch::zeros({n_out, feat_dim}, x.options()).index_add_(0, perm, x);
+    }
+  }
   return out;
 }
 
@@ -684,7 +742,8 @@ TORCH_LIBRARY(npc, m) {
       .def("register_graph_partition", &RegisterGraphPartition)
       .def("set_topology", &SetTopology)
       .def("set_rng_seed", &SetRngSeed)
-      .def("set_strict", &SetStrict);
+      .def("set_strict", &SetStrict)
+      .def("set_block_buffer_ring", &SetBlockBufferRing);
 }
 
 }  // namespace npc

@@ -59,8 +59,15 @@ def set_rng_seed(seed: int) -> None:
 
 
 def set_strict(strict: bool) -> None:
-    """strict (default): load_subtensor raises when a requested node has no row here."""
+    """strict (default): load_subtensor raises when a requested node has no row here, and the pack
+    direction of feat_shuffle checks its permutation (repeated entries add up, as in the reference)."""
     _npc.set_strict(strict)
+
+
+def set_block_buffer_ring(sets: int) -> None:
+    """sample_blocks hands out `sets` sets of output buffers in turn (default 2): the tensors of call k
+    are overwritten by call k + sets.  0 = fresh tensors on every call."""
+    _npc.set_block_buffer_ring(int(sets))
 
 
 # ---------------------------------------------------------------- hot path
@@ -176,27 +183,6 @@ def sddmm_u_add_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset
 
 def sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset):
     return _npc.sddmm_u_mul_v(coo_row, coo_col, lhs, rhs, coo_offset, lhs_offset, rhs_offset)
-
-
-class Aggregate(torch.autograd.Function):
-    """reference python/npc/model/sageconv.py:100-114: forward sums source rows
-    into destinations over the concatenated COO blocks; backward is the same
-    operator with the edge direction and the two offset tables swapped."""
-
-    @staticmethod
-    def forward(ctx, graph, X, X_offset, out_offset):
-        ctx.graph = graph
-        all_coo_row, all_coo_col, coo_offset = graph
-        out = _npc.spmm_copy_u_sum(all_coo_row, all_coo_col, X, coo_offset, X_offset, out_offset)
-        ctx.save_for_backward(X_offset, out_offset)
-        return out
-
-    @staticmethod
-    def backward(ctx, dZ):
-        all_coo_row, all_coo_col, coo_offset = ctx.graph
-        X_offset, out_offset = ctx.saved_tensors
-        dX = _npc.spmm_copy_u_sum(all_coo_col, all_coo_row, dZ.contiguous(), coo_offset, out_offset, X_offset)
-        return None, dX, None, None
 
 
 def srcdst_to_vir(fanout: int, dst: torch.Tensor, src: torch.Tensor) -> torch.Tensor:

@@ -219,6 +219,20 @@ def test_operator_layer_caches_and_buckets(orc, capi):
     assert torch.equal(fwd, h[perm])
     bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm, 16, 0)
     assert torch.equal(bwd, h)                                  # pack undoes unpack
+    # the pack direction is index_select_backward (reference src/feat_shuffle.cc:14-16): rows that several
+    # entries name add up, rows nobody names are zero
+    rep = perm.clone()
+    rep[100:300] = perm[0:200]
+    rep[4000:4100] = perm[0]
+    g = torch.randn(5000, 16, device=DEV)
+    got = npc.feat_shuffle(g, recv_off, dev_off, rep, 16, 0)
+    want = torch.zeros(5000, 16, device=DEV).index_add_(0, rep, g)
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-4)          # two atomic sums of up to 102 rows, in different orders
+    assert bool((got[perm[200:300]] == 0).all()) and bool((got[perm[4000:4100]] == 0).all())
+    with pytest.raises(IndexError):
+        bad = perm.clone()
+        bad[7] = 5000
+        npc.feat_shuffle(g, recv_off, dev_off, bad, 16, 0)
 
 
 def test_partitioned_store_pipeline(orc, capi):
@@ -383,6 +397,20 @@ def test_operator_layer_fused_sampler(orc, capi):
     assert sizes[:2] == [50, len(want_in)] and np.array_equal(nodes.cpu().numpy(), want_in)
     assert np.array_equal(hops[0][0].cpu().numpy(), want_blocks[0]["neighbors"])
     assert np.array_equal(hops[0][2].cpu().numpy(), want_blocks[0]["counts"])
+    nodes, hops = nodes.clone(), [tuple(t.clone() for t in hops[0])]      # the ring below overwrites the originals
+    # output buffers come from a ring of two sets: a call's tensors stay untouched during the next call and
+    # are overwritten by the one after; with a ring of 0 every call gets fresh tensors
+    s1, n1, h1 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10)
+    keep = (n1.clone(), h1[0][1].clone())
+    s2, n2, h2 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 11)
+    assert n2.data_ptr() != n1.data_ptr() and torch.equal(n1, keep[0]) and torch.equal(h1[0][1], keep[1])
+    s3, n3, h3 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 12)
+    assert n3.data_ptr() == n1.data_ptr() and h3[0][1].data_ptr() == h1[0][1].data_ptr()
+    npc.ops.set_block_buffer_ring(0)
+    outs = [npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10 + k) for k in range(3)]
+    assert len({o[1].data_ptr() for o in outs}) == 3
+    assert torch.equal(outs[0][1], keep[0]) and torch.equal(outs[0][2][0][1], keep[1])   # same key, same batch
+    npc.ops.set_block_buffer_ring(2)
     # the same call with the blocks' COO + CSC emitted before its one wait
     sizes_f, nodes_f, hops_f, fmts = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9, formats=True)
     assert sizes_f == sizes and torch.equal(nodes_f, nodes) and torch.equal(hops_f[0][1], hops[0][1])

@@ -80,9 +80,10 @@ def test_gpu_virtual_nodes(orc, capi):
 
 
 @pytest.mark.gpu
-def test_aggregate_autograd(orc, capi):
-    """Aggregate (reference python/npc/model/sageconv.py:100-114): forward and
-    backward against torch's own index_add on the GPU in fp32."""
+def test_spmm_operator_both_directions(orc, capi):
+    """spmm_copy_u_sum over a block and over the same block with the edges reversed and the two offset
+    tables swapped (how the reference forms the gradient, python/npc/model/sageconv.py:100-114), against
+    torch's own index_add on the GPU in fp32."""
     import torch
 
     import apt_amd as npc
@@ -92,12 +93,9 @@ def test_aggregate_autograd(orc, capi):
     row = torch.from_numpy(rng.integers(0, n_src, n_dst * fanout)).to("cuda:0")
     coo_off = torch.tensor([0, row.numel()], device="cuda:0")
     x_off, out_off = torch.tensor([0, n_src], device="cuda:0"), torch.tensor([0, n_dst], device="cuda:0")
-    X = torch.randn(n_src, dim, device="cuda:0", requires_grad=True)
-    out = npc.ops.Aggregate.apply((row, col, coo_off), X, x_off, out_off)
-    w = torch.randn_like(out)
-    (out * w).sum().backward()
-    X2 = X.detach().clone().requires_grad_(True)
-    ref = torch.zeros(n_dst, dim, device="cuda:0").index_add(0, col, X2[row])
-    (ref * w).sum().backward()
-    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-5)
-    assert torch.allclose(X.grad, X2.grad, rtol=1e-5, atol=1e-5)
+    x = torch.randn(n_src, dim, device="cuda:0")
+    out = npc.spmm_copy_u_sum(row, col, x, coo_off, x_off, out_off)
+    assert torch.allclose(out, torch.zeros(n_dst, dim, device="cuda:0").index_add(0, col, x[row]), rtol=1e-5, atol=1e-5)
+    dz = torch.randn(n_dst, dim, device="cuda:0")
+    dx = npc.spmm_copy_u_sum(col, row, dz, coo_off, out_off, x_off)
+    assert torch.allclose(dx, torch.zeros(n_src, dim, device="cuda:0").index_add(0, row, dz[col]), rtol=1e-5, atol=1e-5)
