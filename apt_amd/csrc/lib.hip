@@ -30,6 +30,8 @@ static int g_gather_vector_bytes = 0;
 int tuning_gather_vector_bytes() { return g_gather_vector_bytes; }
 static int g_gather_store_policy = 0;
 int tuning_gather_store_policy() { return g_gather_store_policy; }
+static int g_relabel_lds = 1;
+int tuning_relabel_lds() { return g_relabel_lds; }
 static int g_block_fused_scan = 1;
 int tuning_block_fused_scan() { return g_block_fused_scan; }
 
@@ -82,6 +84,10 @@ extern "C" int apt_set_tuning(const char* key, int value) {
     if (value < 0 || value > 2)
       return apt::fail(APT_EINVAL, "apt_set_tuning: gather_store_policy must be 0 (write-through), 1 (non-temporal) or 2 (plain)");
     apt::g_gather_store_policy = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "relabel_lds") == 0) {
+    apt::g_relabel_lds = value != 0;
     return APT_OK;
   }
   if (std::strcmp(key, "block_fused_scan") == 0) {

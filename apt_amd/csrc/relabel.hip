@@ -286,6 +286,108 @@ __global__ __launch_bounds__(kRelBlock) void relabel_lookup_kernel(RelabelParams
   }
 }
 
+// ---------------------------------------------------------------------------
+// Small inputs (the first hop of a batch, hops of small batches): the whole
+// relabel in one workgroup with the hash table in LDS, one launch instead of
+// five and no global atomics.  The item keys are copied into LDS (64 KB for
+// 8192 items); the table (2 slots per item, 4 bytes each: the index of the
+// key's first item so far) takes another 64 KB.  A probe compares keys through
+// the index a slot holds; claiming an empty slot is a CAS, lowering the index
+// of a key that is already there an atomic minimum, both on LDS.  After a
+// barrier an item owns its key iff its slot holds its own index; owners are
+// ranked with ballots and a prefix over the workgroup's wavefronts, write their
+// ids to the output and leave their rank in the slot for the key's other items.
+constexpr int kLdsRelBlock = 1024;
+constexpr int kLdsRelMaxItems = 8192;
+constexpr int kLdsRelSlots = 2 * kLdsRelMaxItems;
+constexpr int kLdsRelPerThread = kLdsRelMaxItems / kLdsRelBlock;
+constexpr uint32_t kLdsEmpty = 0xFFFFFFFFu;
+int tuning_relabel_lds();  // 1 (default) = inputs that fit take the LDS path
+
+__global__ __launch_bounds__(kLdsRelBlock) void relabel_lds_kernel(RelabelParams p) {
+  __shared__ int64_t s_key[kLdsRelMaxItems];
+  __shared__ uint32_t s_table[kLdsRelSlots];
+  __shared__ uint32_t s_wave[kLdsRelPerThread][kLdsRelBlock / kWave];
+  const RelSizes s = rel_sizes(p);   // items <= kLdsRelMaxItems (the host checked the upper bounds)
+  const int tid = threadIdx.x;
+  const int lane = lane_id(), wave = tid / kWave;
+  // Few values live per thread (a slot per item and a bit mask): keys are read back from LDS where needed,
+  // so that nothing spills.  The keys are requested first, the table is cleared while they are on their way.
+  {
+    int64_t key[kLdsRelPerThread];
+#pragma unroll
+    for (int k = 0; k < kLdsRelPerThread; ++k) {
+      const int i = k * kLdsRelBlock + tid;
+      key[k] = i < s.items ? item_at(p, s, i) : -1;
+    }
+    uint4* t4 = reinterpret_cast<uint4*>(s_table);
+    const uint4 ones = make_uint4(kLdsEmpty, kLdsEmpty, kLdsEmpty, kLdsEmpty);
+#pragma unroll
+    for (int q = 0; q < kLdsRelSlots / 4 / kLdsRelBlock; ++q) t4[q * kLdsRelBlock + tid] = ones;
+#pragma unroll
+    for (int k = 0; k < kLdsRelPerThread; ++k) s_key[k * kLdsRelBlock + tid] = key[k];
+  }
+  __syncthreads();
+  // Insert: the smallest item index per key ends up in the key's slot (a CAS claims an empty slot, an atomic
+  // minimum lowers the index of a key that is already there).
+  uint32_t slot[kLdsRelPerThread];
+#pragma unroll
+  for (int k = 0; k < kLdsRelPerThread; ++k) {
+    const uint32_t i = static_cast<uint32_t>(k * kLdsRelBlock + tid);
+    const int64_t key = s_key[i];
+    slot[k] = kLdsEmpty;
+    if (key < 0) continue;  // padding (and the items past the end)
+    uint32_t q = static_cast<uint32_t>((static_cast<uint64_t>(key) * 0x9E3779B97F4A7C15ull) >> 50);  // 14 bits
+    uint32_t cur = atomicCAS(&s_table[q], kLdsEmpty, i);   // what the slot held before
+    while (cur != kLdsEmpty) {
+      if (s_key[cur] == key) {  // whichever item of this key holds the slot now
+        if (cur > i) atomicMin(&s_table[q], i);
+        break;
+      }
+      q = (q + 1) & (kLdsRelSlots - 1);
+      cur = atomicCAS(&s_table[q], kLdsEmpty, i);
+    }
+    slot[k] = q;
+  }
+  __syncthreads();
+  // owners, in item order: round k covers items [k * 1024, (k + 1) * 1024)
+  uint32_t own = 0;
+#pragma unroll
+  for (int k = 0; k < kLdsRelPerThread; ++k) {
+    const uint32_t i = static_cast<uint32_t>(k * kLdsRelBlock + tid);
+    const bool mine = slot[k] != kLdsEmpty && s_table[slot[k]] == i;
+    own |= (mine ? 1u : 0u) << k;
+    const uint64_t m = ballot(mine);
+    if (lane == 0) s_wave[k][wave] = static_cast<uint32_t>(__popcll(m));
+  }
+  __syncthreads();   // every ownership read of the table is done: owners now leave their rank in their slot
+  uint32_t running = 0;
+#pragma unroll
+  for (int k = 0; k < kLdsRelPerThread; ++k) {
+    uint32_t before = running;
+#pragma unroll
+    for (int w = 0; w < kLdsRelBlock / kWave; ++w) {
+      const uint32_t c = s_wave[k][w];
+      if (w < wave) before += c;
+      running += c;
+    }
+    const bool mine = (own >> k) & 1;
+    const uint64_t m = ballot(mine);
+    if (mine) s_table[slot[k]] = before + static_cast<uint32_t>(rank_below(m));
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < kLdsRelPerThread; ++k) {
+    const int64_t i = static_cast<int64_t>(k) * kLdsRelBlock + tid;
+    if (i >= s.items) continue;
+    const int64_t key = s_key[i];
+    const uint32_t r = key < 0 ? 0 : s_table[slot[k]];
+    if ((own >> k) & 1) p.unique[r] = key;
+    if (i >= s.ns) p.relabeled[i - s.ns] = key < 0 ? key : static_cast<int64_t>(r);
+  }
+  if (tid == 0) *p.num_unique = running;
+}
+
 }  // namespace apt
 
 extern "C" size_t apt_relabel_workspace_bytes(int64_t num_items) {
@@ -325,6 +427,22 @@ static int relabel_enqueue(const int64_t* seeds, int64_t num_seeds, const int64_
                            int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev, char* ws,
                            hipStream_t st) {
   const int64_t items = num_seeds + num_neighbors;
+  if (items <= kLdsRelMaxItems && tuning_relabel_lds() != 0) {
+    // the whole input fits one workgroup's LDS: one launch, no workspace
+    RelabelParams q{};
+    q.seeds = seeds;
+    q.ns = num_seeds;
+    q.ns_dev = num_seeds_dev;
+    q.neighbors = neighbors;
+    q.nn = num_neighbors;
+    q.stride = neighbor_stride;
+    q.unique = unique;
+    q.relabeled = relabeled;
+    q.num_unique = num_unique_dev;
+    hipLaunchKernelGGL(relabel_lds_kernel, dim3(1), dim3(kLdsRelBlock), 0, st, q);
+    APT_LAUNCH_CHECK("relabel_lds_kernel");
+    return APT_OK;
+  }
   const RelabelLayout L = relabel_layout(items);
   RelabelParams p;
   p.seeds = seeds;

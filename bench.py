@@ -83,6 +83,9 @@ def parse_args():
     ap.add_argument("--cache_build", action="store_true",
                     help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
                          "cached feature table) and one step of the all-strategies dry run")
+    ap.add_argument("--relabel_small", action="store_true",
+                    help="also time apt_relabel on first-hop-sized inputs: one workgroup with the table in LDS "
+                         "against the passes over a table in device memory")
     ap.add_argument("--tune", type=str, default="", help="kernel-variant knobs, e.g. sample_lanes_per_row=16")
     ap.add_argument("--target_leg", default="auto", choices=["auto", "on", "off"],
                     help="after the timed region also run batch 1024 on the same graph with 128 x bf16 and 128 x fp32 "
@@ -193,6 +196,51 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
             "edges_per_s": sum(edges) / Kt / wall,
         }
         del pipe, log, sets
+    return out
+
+
+def stage_relabel_small(capi, dev, N, torch):
+    """apt_relabel on inputs the size of a batch's first hop: the single-workgroup LDS kernel against the five
+    passes over a table in device memory (relabel_lds switched off).  Twenty calls are captured into a HIP
+    graph and replayed, so the host's share of a call is not in the figure."""
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+
+    def us_per_call(fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(reps):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (5 * reps) * 1e3
+
+    out = []
+    for ns, f in ((256, 15), (1024, 5), (512, 10), (1024, 7)):
+        seeds = torch.randperm(N, generator=gen, device=dev)[:ns].contiguous()
+        nbrs = torch.randint(0, N, (ns * f,), generator=gen, device=dev)
+        nbrs[::3] = seeds[torch.randint(0, ns, (nbrs[::3].numel(),), generator=gen, device=dev)]   # repeats of the seeds
+        uniq = torch.empty(ns * (f + 1), dtype=torch.int64, device=dev)
+        rel = torch.empty(ns * f, dtype=torch.int64, device=dev)
+        cnt = torch.empty(1, dtype=torch.int64, device=dev)
+        ws = torch.empty(capi.relabel_workspace_bytes(ns * (f + 1)), dtype=torch.uint8, device=dev)
+        row = {"seeds": ns, "fanout": f, "items": ns * (f + 1)}
+        for key, lds in (("lds_one_launch_us", 1), ("device_table_five_launches_us", 0)):
+            capi.set_tuning("relabel_lds", lds)
+            row[key] = us_per_call(lambda: capi.relabel(seeds, nbrs, unique=uniq, relabeled=rel, num_unique_dev=cnt,
+                                                        workspace=ws, sync=False))
+        capi.set_tuning("relabel_lds", 1)
+        out.append(row)
     return out
 
 
@@ -756,6 +804,8 @@ def main():
         extra.clear()
         torch.cuda.empty_cache()
 
+    relabel_small = stage_relabel_small(capi, dev, N, torch) if args.relabel_small else None
+
     # ---- what bounds the sampling kernel: random transactions.  The GPU's rate for them, measured here.
     ceilings = stage_ceilings(capi, dev, N, torch) if args.ceilings != "off" else None
     roofline_sampling = None
@@ -832,6 +882,7 @@ def main():
         "block_formats": fmt,
         "cache_build": cache_build,
         "shuffle": shuffle,
+        "relabel_small": relabel_small,
         "stages": {
             "target_shape": target,
             "per_step_ms": per_step_ms,

@@ -60,6 +60,9 @@ int apt_abi_version(void);
  *   "gather_max_blocks"      cap on the gather grid (rows are strided over)
  *   "gather_vector_bytes"    2|4|8|16: widest load/store a lane of the gather uses
  *                            (16 = global_load_dwordx4 where alignment allows)
+ *   "relabel_lds"            1 (default; 0 = off) apt_relabel handles inputs of up to 8192
+ *                            items in one workgroup with its hash table in LDS (one launch)
+ *                            instead of the passes over a table in device memory
  *   "gather_store_policy"    how the gather stores a row's 16-byte pieces: 0 (default;
  *                            0 here is a value, not "default of the day") write-through
  *                            stores, 1 non-temporal stores, 2 plain stores

@@ -197,6 +197,44 @@ def test_relabel_device_side_count(orc, capi):
     assert np.array_equal(host(r)[:real * f], want_r)
 
 
+def test_relabel_lds_path_and_table_path(orc, capi):
+    """Inputs of up to 8192 items are relabelled by one workgroup with its table in LDS, larger ones by
+    the passes over a table in device memory; both against the oracle on the same small inputs (the
+    switch selects the path), at the size limit, with keys that collide in the LDS table, with padding
+    and with a device-side count."""
+    rng = np.random.default_rng(5)
+    G = 0x9E3779B97F4A7C15
+    inv = pow(G, -1, 1 << 64)
+    # keys whose LDS slot (top 14 bits of key * G) is the same: one long probe chain
+    chain = np.array([k for k in ((t * inv) % (1 << 64) for t in range(1, 3000)) if k < (1 << 62)][:900],
+                     dtype=np.int64)
+    assert len({(int(k) * G % (1 << 64)) >> 50 for k in chain}) == 1 and len(chain) > 500
+    cases = [
+        (rng.permutation(50_000)[:1024], rng.integers(0, 50_000, 1024 * 7)),             # 8192 items: the limit
+        (rng.permutation(50_000)[:1024], rng.integers(0, 50_000, 1024 * 7 + 1)),         # one more: table path
+        (np.arange(8192), np.array([], dtype=np.int64)),                                 # all distinct, table half full
+        (np.array([], dtype=np.int64), np.full(8192, 7)),                                # one key 8192 times
+        (chain[:64][::-1].copy(), chain[rng.integers(0, len(chain), 6000)]),
+        (np.array([5, -1, 5, 9]), np.where(rng.random(4000) < 0.3, -1, rng.integers(0, 60, 4000))),
+        (rng.integers(0, 1 << 40, 100), rng.integers(0, 1 << 40, 3000)),
+        (np.array([111_059_955, 0]), rng.integers(111_059_900, 111_059_956, 700)),
+    ]
+    try:
+        for lds in (1, 0):
+            capi.set_tuning("relabel_lds", lds)
+            for seeds, nbrs in cases:
+                _relabel_case(orc, capi, np.asarray(seeds, np.int64), np.asarray(nbrs, np.int64))
+            # device-side count on a small plan (first hop of a batch of 1024 at fanout 5)
+            seeds, nbrs = rng.permutation(100_000)[:1024], rng.integers(0, 100_000, 1024 * 5)
+            cnt = torch.tensor([700], dtype=torch.int64, device=DEV)
+            u, r, nu = capi.relabel(dev(seeds), dev(nbrs), num_seeds_dev=cnt, neighbor_stride=5, sync=False)
+            want_u, want_r = orc.relabel(seeds[:700], nbrs[:3500])
+            n = int(nu.item())
+            assert n == len(want_u) and np.array_equal(host(u)[:n], want_u) and np.array_equal(host(r)[:3500], want_r)
+    finally:
+        capi.set_tuning("relabel_lds", 1)
+
+
 # ------------------------------------------------------------------ gather
 def _rand_table(rng, rows, dim, dtype):
     if dtype == torch.float32:
