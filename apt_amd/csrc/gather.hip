@@ -165,7 +165,8 @@ int tuning_gather_store_policy();
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int R = tuning_gather_rows();
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = 1;
+  // two rows per lane group in flight: with write-through stores 2-4 % faster than one at every size measured
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
   const int groups = kGatherBlock / LPR;
   // With a device-side count the host size is only an upper bound: a capped
   // grid that strides over the rows avoids dispatching workgroups that would
