@@ -82,6 +82,8 @@ SYMBOLS = {
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
     "apt_synth_random_access": (_I, [_I, _P, _I64, _I64, C.c_uint32, _P, _P]),
+    "apt_synth_grid_barrier": (_I, [_I, _I, _P, _P, _P]),
+    "apt_synth_empty_launches": (_I, [_I, _P, _P]),
     "apt_time_next_sample": (_I, [_I, _P, _P]),
 }
 

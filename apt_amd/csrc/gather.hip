@@ -67,16 +67,23 @@ __device__ __forceinline__ const char* source_row(const GatherParams& p, int64_t
 }
 
 // How a lane stores its 16 bytes of a gathered row.
-//   0 (shipped)  write-through: the line goes on to memory as it is written
-//                instead of staying dirty in this XCD's L2 until the release at
-//                the end of the kernel writes the whole L2 back; what that
-//                write-back costs shows on short launches (24.5 against 25.9 us
-//                on 235 k rows of 256 bytes, 25.0 against 26.5 us on 124 k rows of
-//                400 bytes; nothing on 700 k rows and more)
-//   1            non-temporal store (streaming hint only)
-//   2            plain store
-// Narrower vectors (row geometry not 16-byte aligned) always use 1.
-enum : int { kStoreWriteThrough = 0, kStoreNonTemporal = 1, kStorePlain = 2 };
+//   write-through  the line goes on to the memory side as it is written instead
+//                  of staying dirty in this XCD's L2 until the release at the
+//                  end of the kernel writes the whole L2 back: the launch itself
+//                  is 6-10 % shorter.  But the output then fills the memory-side
+//                  cache, and what the next kernels of the batch kept there (the
+//                  sampler's rank table) is gone: after a launch that writes
+//                  185 MB the last hop's sampling kernel takes 84 instead of
+//                  72 us and the batch is 3-4 % slower; after one that writes
+//                  62 MB nothing is lost and the batch is 1-2 % faster.
+//   non-temporal   streaming hint; the output does not displace anything.
+//   plain          neither.
+// kStoreAuto (shipped) decides per launch, on the device, from the rows it
+// actually gathers: write-through while the output is at most half of the
+// 256 MB memory-side cache, non-temporal beyond.  Narrower vectors (row geometry
+// not 16-byte aligned) have no write-through form and use non-temporal stores.
+enum : int { kStoreAuto = 0, kStoreNonTemporal = 1, kStorePlain = 2, kStoreWriteThrough = 3 };
+constexpr int64_t kWriteThroughMaxBytes = int64_t{128} << 20;
 
 template <int V>
 __device__ __forceinline__ void store_row_vec(typename VecT<V>::type val, typename VecT<V>::type* dst, int policy) {
@@ -99,6 +106,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
   const int l = threadIdx.x % LPR;
   const int64_t vec_per_row = p.out_row_bytes / V;
   const int64_t rows_per_block = static_cast<int64_t>(kGroups) * R;
+  int policy = p.store_policy;
+  if (policy == kStoreAuto) policy = n * p.out_row_bytes <= kWriteThroughMaxBytes ? kStoreWriteThrough : kStoreNonTemporal;
   int64_t misses = 0;
   for (int64_t base = static_cast<int64_t>(blockIdx.x) * rows_per_block; base < n;
        base += static_cast<int64_t>(gridDim.x) * rows_per_block) {
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
       }
 #pragma unroll
       for (int k = 0; k < R; ++k) {
-        if (dst[k] != nullptr) store_row_vec<V>(val[k], reinterpret_cast<Vec*>(dst[k]) + c, p.store_policy);
+        if (dst[k] != nullptr) store_row_vec<V>(val[k], reinterpret_cast<Vec*>(dst[k]) + c, policy);
       }
     }
   }
@@ -165,8 +174,9 @@ int tuning_gather_store_policy();
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int R = tuning_gather_rows();
-  // two rows per lane group in flight: with write-through stores 2-4 % faster than one at every size measured
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
+  // Rows per lane group in flight: two where the launch can be one that stores write-through (2-4 % faster
+  // than one there), one for launches whose upper bound is far beyond that (there one is as good or better).
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? 2 : 1;
   const int groups = kGatherBlock / LPR;
   // With a device-side count the host size is only an upper bound: a capped
   // grid that strides over the rows avoids dispatching workgroups that would

@@ -81,8 +81,9 @@ extern "C" int apt_set_tuning(const char* key, int value) {
     return APT_OK;
   }
   if (std::strcmp(key, "gather_store_policy") == 0) {
-    if (value < 0 || value > 2)
-      return apt::fail(APT_EINVAL, "apt_set_tuning: gather_store_policy must be 0 (write-through), 1 (non-temporal) or 2 (plain)");
+    if (value < 0 || value > 3)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: gather_store_policy must be 0 (by output size), 1 (non-temporal), "
+                                   "2 (plain) or 3 (write-through)");
     apt::g_gather_store_policy = value;
     return APT_OK;
   }

@@ -143,6 +143,88 @@ extern "C" int apt_synth_random_access(int mode, void* table, int64_t table_byte
   return APT_OK;
 }
 
+namespace apt {
+
+// Grid-wide barrier between co-resident workgroups, for measuring what one costs
+// (the alternative to ending a kernel and launching the next).  The spin is
+// bounded: a workgroup that waits too long reports it and leaves, and so does
+// every other one at its next barrier, so the kernel always ends.
+__device__ __forceinline__ bool probe_grid_barrier(unsigned* count, unsigned* gen, unsigned groups, unsigned* fail) {
+  __shared__ int ok;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ok = 1;
+    const unsigned g = __hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();
+    if (atomicAdd(count, 1u) == groups - 1) {
+      __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __threadfence();
+      atomicAdd(gen, 1u);
+    } else {
+      unsigned spins = 0;
+      while (__hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g) {
+        __builtin_amdgcn_s_sleep(2);
+        if (++spins > (1u << 20) || __hip_atomic_load(fail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+          ok = 0;
+          atomicAdd(fail, 1u);
+          break;
+        }
+      }
+    }
+    __threadfence();
+  }
+  __syncthreads();
+  return ok != 0;
+}
+
+// state: [0] arrivals, [64] generation, [128] failures (words; a line each).  Every phase a thread writes one
+// word that a thread of another workgroup reads after the barrier, so the barrier's fences carry data.
+__global__ __launch_bounds__(kSynBlock) void grid_barrier_probe_kernel(unsigned* state, uint32_t* buf, int phases) {
+  const unsigned groups = gridDim.x;
+  uint32_t acc = 0;
+  for (int p = 0; p < phases; ++p) {
+    buf[static_cast<size_t>(blockIdx.x) * kSynBlock + threadIdx.x] = acc + p;
+    if (!probe_grid_barrier(state, state + 64, groups, state + 128)) return;
+    const unsigned other = (blockIdx.x + 1 + p) % groups;
+    acc += __builtin_nontemporal_load(&buf[static_cast<size_t>(other) * kSynBlock + threadIdx.x]);
+  }
+  if (acc == 0x12345679u) buf[0] = acc;
+}
+
+__global__ void empty_probe_kernel(uint32_t* buf) {
+  if (buf == nullptr) buf[0] = 1;
+}
+
+}  // namespace apt
+
+extern "C" int apt_synth_grid_barrier(int num_groups, int phases, void* state, void* buf, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_groups >= 1 && phases >= 0 && state != nullptr && buf != nullptr, APT_EINVAL,
+              "apt_synth_grid_barrier: bad arguments");
+  int dev = 0, cus = 0, per_cu = 0;
+  APT_HIP(hipGetDevice(&dev));
+  APT_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  APT_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, grid_barrier_probe_kernel, kSynBlock, 0));
+  // every workgroup must be resident at once, with room to spare for whatever else runs
+  APT_REQUIRE(static_cast<int64_t>(num_groups) * 2 <= static_cast<int64_t>(cus) * per_cu, APT_ELIMIT,
+              "apt_synth_grid_barrier: %d workgroups cannot be resident together on %d CUs", num_groups, cus);
+  hipLaunchKernelGGL(grid_barrier_probe_kernel, dim3(static_cast<unsigned>(num_groups)), dim3(kSynBlock), 0,
+                     static_cast<hipStream_t>(stream), static_cast<unsigned*>(state), static_cast<uint32_t*>(buf), phases);
+  APT_LAUNCH_CHECK("grid_barrier_probe_kernel");
+  return APT_OK;
+}
+
+extern "C" int apt_synth_empty_launches(int count, void* buf, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(count >= 0 && buf != nullptr, APT_EINVAL, "apt_synth_empty_launches: bad arguments");
+  for (int i = 0; i < count; ++i) {
+    hipLaunchKernelGGL(empty_probe_kernel, dim3(64), dim3(kSynBlock), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint32_t*>(buf));
+    APT_LAUNCH_CHECK("empty_probe_kernel");
+  }
+  return APT_OK;
+}
+
 extern "C" int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream) {
   using namespace apt;
   APT_REQUIRE(bytes >= 0 && bytes % 16 == 0, APT_EINVAL, "apt_synth_copy: bytes must be a multiple of 16");

@@ -83,6 +83,15 @@ def parse_args():
     ap.add_argument("--cache_build", action="store_true",
                     help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
                          "cached feature table) and one step of the all-strategies dry run")
+    ap.add_argument("--gather_sizes", action="store_true",
+                    help="also time the gather kernel alone on 0 .. 940 k random rows of this workload's table "
+                         "(device-side count, every launch with its own events): what a launch costs before it moves a byte")
+    ap.add_argument("--frontier_order", action="store_true",
+                    help="also time the last hop's sampling on the frontier in first-occurrence order (as the relabel "
+                         "leaves it) and in node-id order")
+    ap.add_argument("--phase_costs", action="store_true",
+                    help="also measure what separates two dependent phases: a launch boundary (chain of empty kernels) "
+                         "against a grid-wide barrier inside one kernel of 32..256 co-resident workgroups")
     ap.add_argument("--relabel_small", action="store_true",
                     help="also time apt_relabel on first-hop-sized inputs: one workgroup with the table in LDS "
                          "against the passes over a table in device memory")
@@ -199,31 +208,117 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
     return out
 
 
+def graph_replay_us(torch, fn, reps=10, replays=5):
+    """us per call of fn(): `reps` calls captured into a HIP graph on a side stream and replayed, so that
+    the host's share of a call is not in the figure."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=torch.cuda.Stream()):
+        for _ in range(reps):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (replays * reps) * 1e3
+
+
+def stage_gather_sizes(capi, dev, kev, store, N, torch):
+    """The gather kernel alone on n random rows (distinct ids per launch, so the memory-side cache serves
+    nothing twice), device-side count under a host bound of 1 081 344 rows (what batch 1024 allocates): the
+    duration of a launch that gathers nothing is what every launch pays before it moves a byte."""
+    cap = 1024 * 6 * 11 * 16
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    pool = torch.randperm(N, generator=gen, device=dev)[:cap * 8].contiguous()
+    out = torch.empty((cap, store.out_dim), dtype=store.dtype, device=dev)
+    esize = store.local_table.element_size()
+    moved, _ = gather_bytes_per_row(store.out_dim, esize, store.pos_map is not None)
+    rows = []
+    for n in (0, 1024, 16384, 65536, 131072, 235000, 470000, 940000):
+        n_dev = torch.tensor([n], dtype=torch.int64, device=dev)
+        us = []
+        for rep in range(45):
+            off = (rep * 917519) % (pool.numel() - cap)
+            pr = kev.pair()
+            capi.check(capi.lib().apt_time_next_gather(*pr))
+            capi.gather_rows(store, pool[off:off + cap], num_index_dev=n_dev, out=out)
+            torch.cuda.synchronize()
+            t = kev.ms(pr) * 1e3
+            if rep >= 5:
+                us.append(t)
+        q = quantiles(us)
+        rows.append({"rows": n, "us_min": q["min"], "us_median": q["median"], "us_p90": q["p90"],
+                     "GBps_median": n * moved / q["median"] / 1e3})
+    del pool, out
+    # least-squares line through the medians of the launches that move data: us = fixed + bytes / rate
+    pts = [(r["rows"] * moved / 1e6, r["us_median"]) for r in rows if 16384 <= r["rows"] <= 470000]
+    mx = sum(x for x, _ in pts) / len(pts)
+    my = sum(y for _, y in pts) / len(pts)
+    slope = sum((x - mx) * (y - my) for x, y in pts) / sum((x - mx) ** 2 for x, _ in pts)
+    return {"bytes_per_row": moved, "launches": rows,
+            "fit_16k_to_470k_rows": {"fixed_us": my - slope * mx, "streaming_GBps": 1e3 / slope}}
+
+
+def stage_frontier_order(args, capi, dev, graph, hops, seed_sets, stage_pipe, torch, W):
+    """The last hop's sampling (no relabel marking) on its frontier as the relabel leaves it and in node-id order."""
+    H = len(hops)
+    stage_pipe.sample(seed_sets[W], args.seed + 100 + W)
+    torch.cuda.synchronize()
+    n = int(stage_pipe.sizes[H - 1].item())
+    front = stage_pipe.nodes[:n].clone()
+    srt = torch.sort(front).values.contiguous()
+    f = hops[-1]
+    out = torch.empty(n * f, dtype=torch.int64, device=dev)
+    cnt = torch.empty(n, dtype=torch.int64, device=dev)
+    res = {"rows": n, "fanout": f}
+    for name, fr in (("first_occurrence_order_us", front), ("node_id_order_us", srt)):
+        res[name] = graph_replay_us(torch, lambda: capi.sample_neighbors(graph, fr, f, args.replace, 7, H - 1,
+                                                                         out_neighbors=out, out_counts=cnt))
+    del front, srt, out, cnt
+    return res
+
+
+def stage_phase_costs(capi, dev, torch):
+    """A launch boundary against a grid-wide barrier (us per dependent phase)."""
+    L = capi.lib()
+    buf = torch.zeros(1024 * 256, dtype=torch.int32, device=dev)
+    state = torch.zeros(192, dtype=torch.int32, device=dev)
+
+    def best_ms(fn, reps=6):
+        best = None
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1)
+            best = t if best is None or t < best else best
+        return best
+
+    launches = lambda n: capi.check(L.apt_synth_empty_launches(n, capi._ptr(buf), capi._stream()))
+    res = {"dependent_empty_launch_us": (best_ms(lambda: launches(44)) - best_ms(lambda: launches(4))) / 40 * 1e3,
+           "grid_barrier_us_per_phase": {}}
+    for groups in (32, 64, 128, 256):
+        run = lambda ph: capi.check(L.apt_synth_grid_barrier(groups, ph, capi._ptr(state), capi._ptr(buf), capi._stream()))
+        res["grid_barrier_us_per_phase"][str(groups)] = (best_ms(lambda: run(44)) - best_ms(lambda: run(4))) / 40 * 1e3
+    res["barrier_failures"] = int(state[128].item())
+    return res
+
+
 def stage_relabel_small(capi, dev, N, torch):
     """apt_relabel on inputs the size of a batch's first hop: the single-workgroup LDS kernel against the five
     passes over a table in device memory (relabel_lds switched off).  Twenty calls are captured into a HIP
     graph and replayed, so the host's share of a call is not in the figure."""
     gen = torch.Generator(device=dev)
     gen.manual_seed(11)
-
-    def us_per_call(fn, reps=20):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=side):
-            for _ in range(reps):
-                fn()
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / (5 * reps) * 1e3
 
     out = []
     for ns, f in ((256, 15), (1024, 5), (512, 10), (1024, 7)):
@@ -237,8 +332,8 @@ def stage_relabel_small(capi, dev, N, torch):
         row = {"seeds": ns, "fanout": f, "items": ns * (f + 1)}
         for key, lds in (("lds_one_launch_us", 1), ("device_table_five_launches_us", 0)):
             capi.set_tuning("relabel_lds", lds)
-            row[key] = us_per_call(lambda: capi.relabel(seeds, nbrs, unique=uniq, relabeled=rel, num_unique_dev=cnt,
-                                                        workspace=ws, sync=False))
+            row[key] = graph_replay_us(torch, lambda: capi.relabel(seeds, nbrs, unique=uniq, relabeled=rel,
+                                                                   num_unique_dev=cnt, workspace=ws, sync=False), reps=20)
         capi.set_tuning("relabel_lds", 1)
         out.append(row)
     return out
@@ -805,6 +900,13 @@ def main():
         torch.cuda.empty_cache()
 
     relabel_small = stage_relabel_small(capi, dev, N, torch) if args.relabel_small else None
+    phase_costs = stage_phase_costs(capi, dev, torch) if args.phase_costs else None
+    gather_sizes = None
+    if args.gather_sizes and requests is None:
+        gather_sizes = stage_gather_sizes(capi, dev, kev, store, N, torch)
+    frontier_order = None
+    if args.frontier_order and requests is None and args.driver == "fused":
+        frontier_order = stage_frontier_order(args, capi, dev, graph, hops, seed_sets, stage_pipe, torch, W)
 
     # ---- what bounds the sampling kernel: random transactions.  The GPU's rate for them, measured here.
     ceilings = stage_ceilings(capi, dev, N, torch) if args.ceilings != "off" else None
@@ -820,6 +922,11 @@ def main():
         # random rank-table read (atomics for the slots that bid come on top and are not counted here)
         acc = r_ + 2 * e_
         q = quantiles(us_)
+        # new nodes of the hop: each costs at least one atomic (the bid that ends up owning it)
+        new_nodes = sum(hop_sizes[i][H] - hop_sizes[i][H - 1] for i in steps_) / len(steps_)
+        bound_us = None
+        if ceilings:
+            bound_us = (acc / ceilings["load_G_per_s"] + new_nodes / ceilings["atomic_min_returning_G_per_s"]) * 1e-3
         roofline_sampling = {
             "bound": "hbm", "kernel": f"sample_kernel, hop {H} of {H} (fanout {hops[-1]}), rank-table bids included",
             "achieved": alg / t_ / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": alg / t_ / 1e9 / HBM_PEAK_GBPS,
@@ -829,6 +936,10 @@ def main():
             "random_accesses_per_launch": acc, "random_accesses_G_per_s": acc / t_ / 1e9,
             "random_load_ceiling_G_per_s": ceilings["load_G_per_s"] if ceilings else None,
             "frac_of_random_load_ceiling": acc / t_ / 1e9 / ceilings["load_G_per_s"] if ceilings else None,
+            # the time those loads and one atomic per new node take at this GPU's measured rates for them
+            "new_nodes_per_launch": new_nodes,
+            "random_atomic_ceiling_G_per_s": ceilings["atomic_min_returning_G_per_s"] if ceilings else None,
+            "transaction_bound_us": bound_us, "frac_of_transaction_bound": bound_us / (t_ * 1e6) if bound_us else None,
             "timing": f"HIP events carried by {len(steps_)} of the {K} dispatches of the timed region",
         }
 
@@ -883,6 +994,9 @@ def main():
         "cache_build": cache_build,
         "shuffle": shuffle,
         "relabel_small": relabel_small,
+        "phase_costs": phase_costs,
+        "gather_sizes": gather_sizes,
+        "frontier_order": frontier_order,
         "stages": {
             "target_shape": target,
             "per_step_ms": per_step_ms,

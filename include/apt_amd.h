@@ -63,9 +63,10 @@ int apt_abi_version(void);
  *   "relabel_lds"            1 (default; 0 = off) apt_relabel handles inputs of up to 8192
  *                            items in one workgroup with its hash table in LDS (one launch)
  *                            instead of the passes over a table in device memory
- *   "gather_store_policy"    how the gather stores a row's 16-byte pieces: 0 (default;
- *                            0 here is a value, not "default of the day") write-through
- *                            stores, 1 non-temporal stores, 2 plain stores
+ *   "gather_store_policy"    how the gather stores a row's 16-byte pieces: 0 (default; 0 here
+ *                            is a value, not "default of the day") chosen per launch from
+ *                            the bytes it writes (write-through up to 128 MB, non-temporal
+ *                            beyond), 1 non-temporal, 2 plain, 3 write-through
  *   "minibatch_payload_bits" width of the id field of rank-table entries (0 = as
  *                            narrow as the plan allows); wider = fewer epochs
  *                            between table refills (used to test the refill)

@@ -43,6 +43,21 @@ int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream);
 int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
                             uint32_t salt, void* sink, void* stream);
 
+/* What a step between two dependent phases costs, two ways.
+ * apt_synth_grid_barrier: one kernel of num_groups workgroups (256 threads) that
+ *   run `phases` phases separated by a grid-wide barrier (arrival counter and
+ *   generation word in device memory); in every phase a thread writes a word
+ *   that another workgroup reads after the barrier.  The spin is bounded: if a
+ *   workgroup gives up, state[128] counts it and the kernel ends.
+ *   state  device uint32[192], all zero before the first call (arrivals at word
+ *          0, generation at 64, failures at 128)
+ *   buf    device uint32[num_groups * 256]
+ *   num_groups is limited to half of what can be resident at once.
+ * apt_synth_empty_launches: `count` launches of an empty kernel, each dependent
+ *   on the one before by stream order. */
+int apt_synth_grid_barrier(int num_groups, int phases, void* state, void* buf, void* stream);
+int apt_synth_empty_launches(int count, void* buf, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
