@@ -26,7 +26,10 @@ HBM_PEAK_GBPS = 8000.0
 # figure depends on, (workload, feature dtype, feature dim, batch); a run with any other combination reports
 # traffic null.  Each entry names the profiles/ file that holds the counter readings.
 MEASURED_GATHER_TRAFFIC_PER_ROW = {
-    ("full", "bf16", 128, 4096): (520.0, "profiles/gather_kernel_full_pmc.txt"),   # (190.5 MB + 184.7 MB) / 721651 rows
+    ("full", "bf16", 128, 4096): (519.9, "profiles/gather_kernel_full_pmc.txt"),           # (190.5 MB + 184.7 MB) / 721651 rows
+    ("target", "bf16", 128, 1024): (519.0, "profiles/gather_kernel_target_bf16_pmc.txt"),  # (61.8 MB + 59.8 MB) / 234193 rows
+    ("target", "fp32", 128, 1024): (1029.8, "profiles/gather_kernel_target_fp32_pmc.txt"),
+    ("medium", "fp32", 100, 1024): (917.3, "profiles/gather_kernel_medium_pmc.txt"),       # 400-byte rows straddle lines
 }
 
 WORKLOADS = {
@@ -200,6 +203,8 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
             "frac": q_frac["median"], "frac_p10": q_frac["p10"], "frac_p90": q_frac["p90"],
             "frac_min": q_frac["min"], "frac_max": q_frac["max"],
             "frac_by_definition_bytes": q_frac["median"] * spec / moved,
+            "traffic_bytes_per_row": MEASURED_GATHER_TRAFFIC_PER_ROW.get(("target", name, store.out_dim, B), (None, None))[0],
+            "traffic_source": MEASURED_GATHER_TRAFFIC_PER_ROW.get(("target", name, store.out_dim, B), (None, None))[1],
             "GBps_median": q_frac["median"] * HBM_PEAK_GBPS,
             "ms_per_step": wall * 1e3, "ms_per_step_events": quantiles(step_ms),
             "edges_per_s": sum(edges) / Kt / wall,
@@ -255,15 +260,17 @@ def stage_gather_sizes(capi, dev, kev, store, N, torch):
                 us.append(t)
         q = quantiles(us)
         rows.append({"rows": n, "us_min": q["min"], "us_median": q["median"], "us_p90": q["p90"],
-                     "GBps_median": n * moved / q["median"] / 1e3})
+                     "GBps_median": n * moved / q["median"] / 1e3,
+                     # the kernel's own rule: write-through stores while the output is at most 128 MB
+                     "stores": "write-through" if n * store.out_dim * esize <= (128 << 20) else "non-temporal"})
     del pool, out
-    # least-squares line through the medians of the launches that move data: us = fixed + bytes / rate
-    pts = [(r["rows"] * moved / 1e6, r["us_median"]) for r in rows if 16384 <= r["rows"] <= 470000]
+    # least-squares line through the medians of the write-through launches that move data: us = fixed + bytes / rate
+    pts = [(r["rows"] * moved / 1e6, r["us_median"]) for r in rows if r["rows"] >= 16384 and r["stores"] == "write-through"]
     mx = sum(x for x, _ in pts) / len(pts)
     my = sum(y for _, y in pts) / len(pts)
     slope = sum((x - mx) * (y - my) for x, y in pts) / sum((x - mx) ** 2 for x, _ in pts)
     return {"bytes_per_row": moved, "launches": rows,
-            "fit_16k_to_470k_rows": {"fixed_us": my - slope * mx, "streaming_GBps": 1e3 / slope}}
+            "fit_write_through_launches_from_16k_rows": {"fixed_us": my - slope * mx, "streaming_GBps": 1e3 / slope}}
 
 
 def stage_frontier_order(args, capi, dev, graph, hops, seed_sets, stage_pipe, torch, W):
@@ -750,7 +757,8 @@ def main():
     elapsed = time.perf_counter() - t0
     sample_us = None
     if staged:
-        gather_ms = sorted(kev.ms(gkevs[i]) for i in timed_steps)
+        gather_ms_by_step = [kev.ms(gkevs[i]) for i in timed_steps]
+        gather_ms = sorted(gather_ms_by_step)
         t_gather = sum(gather_ms) / len(gather_ms) * K
         t_sample = start.elapsed_time(stop) - t_gather
         if skevs:
@@ -984,6 +992,8 @@ def main():
             "avg_launch_us": t_gather / K * 1e3,
             "launch_us_min_median_max": ([gather_ms[0] * 1e3, gather_ms[len(gather_ms) // 2] * 1e3,
                                           gather_ms[-1] * 1e3] if staged else None),
+            "launch_us_by_timed_step": ({str(i): round(t * 1e3, 2) for i, t in zip(timed_steps, gather_ms_by_step)}
+                                        if staged else None),
             "timing": (f"HIP events carried by {len(timed_steps)} of the {K} gather dispatches of the timed region "
                        f"(kernel begin / end)" if staged else "HIP events recorded around each gather launch of an untimed pass"),
         },
