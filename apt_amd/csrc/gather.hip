@@ -17,6 +17,7 @@ namespace apt {
 
 constexpr int kGatherBlock = 256;
 constexpr int kGatherPersistentBlocks = 16384;
+constexpr int kGatherResidentBlocks = 2048;   // 256 CUs x 8 workgroups of 256 threads
 
 struct GatherParams {
   const char* local_table;
@@ -37,6 +38,7 @@ struct GatherParams {
   int64_t num_out_rows;      // scatter only
   uint8_t* named;            // scatter only, optional: named[v] = 1 for every output row v that is written
   int store_policy;          // kStore* (apt_set_tuning gather_store_policy)
+  int64_t wt_tail_bytes;     // kStoreAuto on a large output: the last bytes written go write-through
 };
 
 template <int V> struct VecT;
@@ -80,10 +82,17 @@ __device__ __forceinline__ const char* source_row(const GatherParams& p, int64_t
 //   plain          neither.
 // kStoreAuto (shipped) decides per launch, on the device, from the rows it
 // actually gathers: write-through while the output is at most half of the
-// 256 MB memory-side cache, non-temporal beyond.  Narrower vectors (row geometry
-// not 16-byte aligned) have no write-through form and use non-temporal stores.
+// 256 MB memory-side cache; beyond that non-temporal, except for the 64 MB that
+// the kernel writes last, which would otherwise be what the release at its end
+// still has to write back.  That tail is a trade, not a gain: on a 185 MB output
+// every 16 MB of it take 0.6 us off the launch and add about as much to the next
+// batch's sampling kernel (70.2 -> 67.6 us and 71.4 -> 72.7 us at 64 MB); the
+// batch is at its shortest between 48 and 64 MB (0.2119 against 0.2125 ms).
+// Narrower vectors (row geometry not 16-byte aligned) have no write-through form
+// and use non-temporal stores.
 enum : int { kStoreAuto = 0, kStoreNonTemporal = 1, kStorePlain = 2, kStoreWriteThrough = 3 };
 constexpr int64_t kWriteThroughMaxBytes = int64_t{128} << 20;
+constexpr int64_t kWriteThroughTailMiB = 64;
 
 template <int V>
 __device__ __forceinline__ void store_row_vec(typename VecT<V>::type val, typename VecT<V>::type* dst, int policy) {
@@ -106,11 +115,18 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
   const int l = threadIdx.x % LPR;
   const int64_t vec_per_row = p.out_row_bytes / V;
   const int64_t rows_per_block = static_cast<int64_t>(kGroups) * R;
-  int policy = p.store_policy;
-  if (policy == kStoreAuto) policy = n * p.out_row_bytes <= kWriteThroughMaxBytes ? kStoreWriteThrough : kStoreNonTemporal;
+  int launch_policy = p.store_policy;
+  // rows from wt_from on are stored write-through: everything when the output is small, else the part the kernel
+  // writes last
+  int64_t wt_from = n;
+  if (launch_policy == kStoreAuto) {
+    launch_policy = kStoreNonTemporal;
+    wt_from = n * p.out_row_bytes <= kWriteThroughMaxBytes ? 0 : n - p.wt_tail_bytes / p.out_row_bytes;
+  }
   int64_t misses = 0;
   for (int64_t base = static_cast<int64_t>(blockIdx.x) * rows_per_block; base < n;
        base += static_cast<int64_t>(gridDim.x) * rows_per_block) {
+    const int policy = base >= wt_from ? kStoreWriteThrough : launch_policy;
     const char* src[R];
     char* dst[R];
 #pragma unroll
@@ -170,19 +186,26 @@ int tuning_gather_rows();        // 0 = default
 int tuning_gather_max_blocks();  // 0 = default
 int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
 int tuning_gather_store_policy();
+int tuning_gather_wt_tail_mib();  // 0 = kWriteThroughTailMiB
 
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   int R = tuning_gather_rows();
-  // Rows per lane group in flight: two where the launch can be one that stores write-through (2-4 % faster
-  // than one there), one for launches whose upper bound is far beyond that (there one is as good or better).
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? 2 : 1;
+  // Rows per lane group in flight: two (with the settings alternating inside one process on the batch's own
+  // launches, two are 1-3 % faster than one at a quarter of a million rows and at three quarters; four are slower).
+  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
   const int groups = kGatherBlock / LPR;
   // With a device-side count the host size is only an upper bound: a capped
   // grid that strides over the rows avoids dispatching workgroups that would
-  // find nothing to do.
+  // find nothing to do.  Where the bound says the launch is a small one, the cap
+  // is what the CUs hold at once (8 workgroups each): 23.7 against 24.4 us for
+  // the 235 k rows of a batch of 1024; for 725 k rows every cap from 2048 to
+  // 16384 gives the same 67 us.
   int64_t max_blocks = tuning_gather_max_blocks();
-  if (max_blocks <= 0) max_blocks = p.n_dev != nullptr ? kGatherPersistentBlocks : (1 << 20);
+  if (max_blocks <= 0)
+    max_blocks = p.n_dev == nullptr                                    ? (1 << 20)
+                 : p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? kGatherResidentBlocks
+                                                                      : kGatherPersistentBlocks;
   int64_t blocks = ceil_div(p.n, static_cast<int64_t>(groups) * R);
   if (blocks > max_blocks) blocks = max_blocks;
   const dim3 grid(static_cast<unsigned>(blocks)), block(kGatherBlock);
@@ -289,6 +312,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.num_out_rows = 0;
   p.named = nullptr;
   p.store_policy = tuning_gather_store_policy();
+  p.wt_tail_bytes = (tuning_gather_wt_tail_mib() > 0 ? int64_t{tuning_gather_wt_tail_mib()} : kWriteThroughTailMiB) << 20;
   arm.rearm();
   return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
 }
@@ -330,6 +354,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
   p.num_out_rows = scatter ? num_rows_other : 0;
   p.named = named;
   p.store_policy = tuning_gather_store_policy();
+  p.wt_tail_bytes = (tuning_gather_wt_tail_mib() > 0 ? int64_t{tuning_gather_wt_tail_mib()} : kWriteThroughTailMiB) << 20;
   arm.rearm();
   return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
 }

@@ -30,6 +30,8 @@ static int g_gather_vector_bytes = 0;
 int tuning_gather_vector_bytes() { return g_gather_vector_bytes; }
 static int g_gather_store_policy = 0;
 int tuning_gather_store_policy() { return g_gather_store_policy; }
+static int g_gather_wt_tail_mib = 0;
+int tuning_gather_wt_tail_mib() { return g_gather_wt_tail_mib; }
 static int g_relabel_lds = 1;
 int tuning_relabel_lds() { return g_relabel_lds; }
 static int g_block_fused_scan = 1;
@@ -85,6 +87,11 @@ extern "C" int apt_set_tuning(const char* key, int value) {
       return apt::fail(APT_EINVAL, "apt_set_tuning: gather_store_policy must be 0 (by output size), 1 (non-temporal), "
                                    "2 (plain) or 3 (write-through)");
     apt::g_gather_store_policy = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "gather_wt_tail_mib") == 0) {
+    APT_REQUIRE(value >= 0 && value <= 1024, APT_EINVAL, "apt_set_tuning: gather_wt_tail_mib must be in [0, 1024]");
+    apt::g_gather_wt_tail_mib = value;
     return APT_OK;
   }
   if (std::strcmp(key, "relabel_lds") == 0) {

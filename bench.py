@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # figure depends on, (workload, feature dtype, feature dim, batch); a run with any other combination reports
 # traffic null.  Each entry names the profiles/ file that holds the counter readings.
 MEASURED_GATHER_TRAFFIC_PER_ROW = {
-    ("full", "bf16", 128, 4096): (519.9, "profiles/gather_kernel_full_pmc.txt"),           # (190.5 MB + 184.7 MB) / 721651 rows
+    ("full", "bf16", 128, 4096): (520.2, "profiles/gather_kernel_full_pmc.txt"),           # (190.7 MB + 184.7 MB) / 721651 rows
     ("target", "bf16", 128, 1024): (519.0, "profiles/gather_kernel_target_bf16_pmc.txt"),  # (61.8 MB + 59.8 MB) / 234193 rows
     ("target", "fp32", 128, 1024): (1029.8, "profiles/gather_kernel_target_fp32_pmc.txt"),
     ("medium", "fp32", 100, 1024): (917.3, "profiles/gather_kernel_medium_pmc.txt"),       # 400-byte rows straddle lines
@@ -109,6 +109,15 @@ def parse_args():
     ap.add_argument("--ceilings", default="auto", choices=["auto", "on", "off"],
                     help="measure the GPU's rate for random 4-byte loads / stores / atomics (what bounds the sampling "
                          "kernel) and quote the last hop's sampling kernel against it; auto = on")
+    ap.add_argument("--alternate", type=str, default="",
+                    help="settings to compare inside this one process, separated by '/', each a '+'-joined list of "
+                         "knob=value (e.g. gather_wt_tail_mib=1/gather_wt_tail_mib=64): the batches of the timed region "
+                         "are run again and again with the settings taking turns (stages.alternate); two processes, "
+                         "let alone two boxes, differ by more than most knobs do")
+    ap.add_argument("--alternate_batch", type=int, default=0, help="batch size of --alternate (0 = the workload's)")
+    ap.add_argument("--ceiling_table_mib", type=str, default="",
+                    help="comma-separated table sizes in MiB: repeat the random-access measurement for each "
+                         "(stages.random_access_by_table_size)")
     return ap.parse_args()
 
 def quantiles(xs):
@@ -346,9 +355,77 @@ def stage_relabel_small(capi, dev, N, torch):
     return out
 
 
-def stage_ceilings(capi, dev, N, torch):
-    """The GPU's rate for one random 4-byte access per work item into a table of the rank table's size."""
-    nbytes = max(1 << 20, (N * 4 + 15) // 16 * 16)
+def stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, seed_lo, store, B, torch, dev):
+    """Kernel-variant knobs against each other inside one process: six rounds, in each of which every setting
+    runs the same 35 batches on one stream (wall time) and 20 more whose gather and last-hop sampling dispatches
+    carry events.  The first five batches after a change of setting still run behind the previous setting's
+    gather and are left out.  -> per setting: medians over the rounds."""
+    import statistics as st
+    settings = []
+    for text in args.alternate.split("/"):
+        knobs = dict((kv.split("=")[0], int(kv.split("=")[1])) for kv in text.split("+"))
+        settings.append((text, knobs))
+    touched = sorted({k for _, knobs in settings for k in knobs})
+    default_of = lambda k: 1 if k in ("minibatch_fuse_mark", "relabel_lds", "block_fused_scan") else 0
+    H, NB = len(hops), 40
+    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(args.seed + 31)
+    pool = seed_lo + torch.randperm(seed_n, generator=gen, device=dev)[:NB * B]
+    sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(NB)]
+    res = {text: {"ms": [], "gather_us": [], "sample_us": []} for text, _ in settings}
+    for i in range(NB):
+        pipe.run(sets[i], args.seed + 900 + i)
+    torch.cuda.synchronize()
+    try:
+        for rnd in range(7):
+            for text, knobs in settings:
+                for k in touched:
+                    capi.set_tuning(k, knobs.get(k, default_of(k)))
+                for i in range(5):
+                    pipe.run(sets[i], args.seed + 900 + i)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(5, NB):
+                    pipe.run(sets[i], args.seed + 900 + i)
+                torch.cuda.synchronize()
+                ms = (time.perf_counter() - t0) / (NB - 5) * 1e3
+                gp, sp = [], []
+                for i in range(5, 25):
+                    g, s = kev.pair(), kev.pair()
+                    if args.driver == "fused":
+                        capi.check(capi.lib().apt_time_next_sample(H - 1, s[0], s[1]))
+                    pipe.sample(sets[i], args.seed + 900 + i)
+                    capi.check(capi.lib().apt_time_next_gather(g[0], g[1]))
+                    pipe.gather()
+                    gp.append(g)
+                    sp.append(s)
+                torch.cuda.synchronize()
+                g_us = st.median(kev.ms(p) * 1e3 for p in gp)
+                s_us = st.median(kev.ms(p) * 1e3 for p in sp) if args.driver == "fused" else None
+                if rnd > 0:   # the first round warms up
+                    res[text]["ms"].append(ms)
+                    res[text]["gather_us"].append(g_us)
+                    res[text]["sample_us"].append(s_us)
+    finally:
+        for k in touched:
+            capi.set_tuning(k, default_of(k))
+        for kv in filter(None, args.tune.split(",")):
+            capi.set_tuning(kv.split("=")[0], int(kv.split("=")[1]))
+    out = {"batch": B, "rounds": 6, "batches_per_round": NB - 5, "settings": []}
+    for text, _ in settings:
+        r = res[text]
+        out["settings"].append({
+            "setting": text, "ms_per_batch_median": st.median(r["ms"]), "ms_per_batch_by_round": r["ms"],
+            "gather_us_median": st.median(r["gather_us"]),
+            "last_hop_sample_us_median": st.median(r["sample_us"]) if args.driver == "fused" else None})
+    return out
+
+
+def stage_ceilings(capi, dev, N, torch, table_bytes=None):
+    """The GPU's rate for one random 4-byte access per work item into a table of the rank table's size
+    (or of table_bytes)."""
+    nbytes = table_bytes if table_bytes else max(1 << 20, (N * 4 + 15) // 16 * 16)
     table = torch.full((nbytes // 4,), -1, dtype=torch.int32, device=dev)
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     n = 8_000_000
@@ -916,8 +993,15 @@ def main():
     if args.frontier_order and requests is None and args.driver == "fused":
         frontier_order = stage_frontier_order(args, capi, dev, graph, hops, seed_sets, stage_pipe, torch, W)
 
+    alternate = None
+    if args.alternate and requests is None:
+        alternate = stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, seed_lo, store,
+                                    args.alternate_batch or B, torch, dev)
+
     # ---- what bounds the sampling kernel: random transactions.  The GPU's rate for them, measured here.
     ceilings = stage_ceilings(capi, dev, N, torch) if args.ceilings != "off" else None
+    ceilings_by_size = [stage_ceilings(capi, dev, N, torch, int(float(m) * (1 << 20)) // 16 * 16)
+                        for m in args.ceiling_table_mib.split(",") if m.strip()] or None
     roofline_sampling = None
     if sample_us and last_hop:
         steps_ = sorted(last_hop)
@@ -1005,12 +1089,14 @@ def main():
         "shuffle": shuffle,
         "relabel_small": relabel_small,
         "phase_costs": phase_costs,
+        "alternate": alternate,
         "gather_sizes": gather_sizes,
         "frontier_order": frontier_order,
         "stages": {
             "target_shape": target,
             "per_step_ms": per_step_ms,
             "random_access_ceilings": ceilings,
+            "random_access_by_table_size": ceilings_by_size,
             "in_flight": in_flight,
             "edges_per_step": edges / K,
             "input_nodes_per_step": rows / K,

@@ -65,8 +65,12 @@ int apt_abi_version(void);
  *                            instead of the passes over a table in device memory
  *   "gather_store_policy"    how the gather stores a row's 16-byte pieces: 0 (default; 0 here
  *                            is a value, not "default of the day") chosen per launch from
- *                            the bytes it writes (write-through up to 128 MB, non-temporal
- *                            beyond), 1 non-temporal, 2 plain, 3 write-through
+ *                            the bytes it writes (write-through up to 128 MB; beyond that
+ *                            non-temporal except for the part written last, see
+ *                            "gather_wt_tail_mib"), 1 non-temporal, 2 plain, 3 write-through
+ *   "gather_wt_tail_mib"     with policy 0 and an output above 128 MB: how many MiB at the
+ *                            end of the output are stored write-through (0 = default, 64;
+ *                            1 = practically none)
  *   "minibatch_payload_bits" width of the id field of rank-table entries (0 = as
  *                            narrow as the plan allows); wider = fewer epochs
  *                            between table refills (used to test the refill)

@@ -301,6 +301,32 @@ def test_gather_empty_and_device_count(orc, capi):
     assert np.array_equal(o[:2500], table[idx[:2500]]) and np.all(o[2500:] == 5.0)
 
 
+def test_gather_store_rules_give_the_same_rows(capi):
+    """An output above 128 MB is stored non-temporal except for its end, which goes write-through (how much is a
+    knob); whatever the split, and with every forced policy, the rows are those of torch's index_select.  The
+    device-side count decides where the end is."""
+    from apt_amd import synth
+    n_rows, D, n = 1_000_000, 128, 600_000                       # 600 k rows of 256 B: 154 MB
+    feats = synth.random_features(n_rows, D, torch.bfloat16, 4, DEV)
+    idx = torch.randint(0, n_rows, (n,), device=DEV)
+    want = feats.index_select(0, idx).view(torch.int16)
+    fs = capi.FeatStore(feats)
+    n_dev = torch.tensor([n - 12_345], device=DEV)
+    try:
+        for policy, tail in ((0, 0), (0, 1), (0, 32), (0, 1024), (1, 0), (2, 0), (3, 0)):
+            capi.set_tuning("gather_store_policy", policy)
+            capi.set_tuning("gather_wt_tail_mib", tail)
+            out = capi.gather_rows(fs, idx)
+            assert torch.equal(out.view(torch.int16), want), (policy, tail)
+            out = torch.zeros_like(out)
+            capi.gather_rows(fs, idx, num_index_dev=n_dev, out=out)
+            k = int(n_dev.item())
+            assert torch.equal(out[:k].view(torch.int16), want[:k]) and not out[k:].any(), (policy, tail)
+    finally:
+        capi.set_tuning("gather_store_policy", 0)
+        capi.set_tuning("gather_wt_tail_mib", 0)
+
+
 def test_permute_scatter_rows(orc, capi):
     rng = np.random.default_rng(10)
     for dim, dtype in [(16, torch.float32), (256, torch.float32), (64, torch.bfloat16), (3, torch.float32)]:
