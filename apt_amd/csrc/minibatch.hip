@@ -287,7 +287,16 @@ __global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
   const int64_t ns = actual_count(p.ns_cap[h], p.ns_dev[h]);
   for (int64_t j = (static_cast<int64_t>(blockIdx.x) - p.block_begin[h]) * kMbBlock + threadIdx.x;
        j < nn; j += blocks * kMbBlock) {
-    if (p.relabeled[h][j] > kSlotOwner) continue;  // an id, or padding (any other negative value)
+    const int64_t r = p.relabeled[h][j];
+    if (r >= kSlotStatesEnd) continue;  // an id, or padding (any other negative value)
+    if (via_owner && r >= kSlotLoserSaw) {
+      // the slot that was seen with a smaller bid holds the node's id by now, unless it was displaced itself
+      const int64_t id = p.relabeled[h][r - kSlotLoserSaw];
+      if (id >= 0) {
+        p.relabeled[h][j] = id;
+        continue;
+      }
+    }
     const int64_t e = p.table[p.neighbors[h][j]] - tb;
     // via_owner: e is the winning bid ns + slot; the winner's slot holds the id
     // (it is an owner, so its slot is final and never pending).

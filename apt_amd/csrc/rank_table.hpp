@@ -6,12 +6,19 @@
 
 namespace apt {
 
-// States of a relabeled[] slot before its compact id is known.  They are the two
-// most negative values, so that no id a graph can hold, valid or corrupt, is
-// mistaken for one: a negative id is padding and passes through unchanged, as in
-// the hash-table relabel.
+// States of a relabeled[] slot before its compact id is known.  They are the
+// 2^32 + 2 most negative values, and the bidding turns a (corrupt) neighbour id
+// in that range into plain padding, so that no id a graph can hold is mistaken
+// for a state; every other negative id is padding that passes through
+// unchanged, as in the hash-table relabel.
 constexpr int64_t kSlotLoser = INT64_MIN;      // another slot holds a smaller bid for the same node
 constexpr int64_t kSlotOwner = INT64_MIN + 1;  // bid placed and, so far, the smallest for its node
+// kSlotLoserSaw + s: like kSlotLoser, and slot s of the hop was seen holding a
+// smaller bid for the node.  Slot s got kSlotOwner when it bid, so after the
+// owners are placed it holds the node's id, unless a still smaller bid displaced
+// it later (then it holds kSlotOwner until the lookup pass reaches it).
+constexpr int64_t kSlotLoserSaw = INT64_MIN + 2;
+constexpr int64_t kSlotStatesEnd = kSlotLoserSaw + (int64_t{1} << 32);
 
 struct RankTable {
   uint32_t* entries;        // one per node: (epoch << payload bits) | id or bid
@@ -51,7 +58,7 @@ __device__ __forceinline__ RankEpoch rank_epoch(const uint32_t* state) {
 __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const RankEpoch& ep, bool first_hop,
                                                   int64_t v, int64_t ns, int64_t j) {
   const uint32_t tb = ep.base;
-  if (v < 0) return v <= kSlotOwner ? -1 : v;  // padding; never one of the two states above
+  if (v < 0) return v < kSlotStatesEnd ? -1 : v;  // padding; never one of the states above
   if (v >= t.len) return -1;  // an id the table cannot hold: treated as padding
   const uint32_t first_bid = tb + static_cast<uint32_t>(ns);
   const uint32_t bid = first_bid + static_cast<uint32_t>(j);
@@ -63,9 +70,10 @@ __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const Rank
     return kSlotOwner;
   }
   if (cur < first_bid) return static_cast<int64_t>(cur - tb);
-  if (cur < bid) return kSlotLoser;
+  if (cur < bid) return kSlotLoserSaw + static_cast<int64_t>(cur - first_bid);
   const uint32_t old = atomicMin(&t.entries[v], bid);
-  if (old < bid) return old < first_bid ? static_cast<int64_t>(old - tb) : kSlotLoser;
+  if (old < bid)
+    return old < first_bid ? static_cast<int64_t>(old - tb) : kSlotLoserSaw + static_cast<int64_t>(old - first_bid);
   // old > bid: this slot is the smallest so far.  If old belongs to this batch it
   // is a bid of this hop (ids are below first_bid): that slot has been displaced.
   if ((old >> ep.bits) == ep.epoch) t.displaced[old - first_bid] = 1;

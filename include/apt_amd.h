@@ -314,7 +314,9 @@ int apt_cluster_reqs(const int64_t* ids, int64_t n, const int64_t* n_dev,
  *                   the library: calls may follow each other on one stream
  *                   without any clearing in between.  A node id outside
  *                   [0, rank_table_len) is treated like padding (no edge, not
- *                   in the node list).
+ *                   in the node list): a negative one appears unchanged in
+ *                   relabeled[], except that the 2^32 + 2 most negative
+ *                   values, which the driver uses for slot states, become -1.
  *   nodes           device int64[capacity(num_hops)]: the unique node list;
  *                   its first sizes[h] entries are the frontier of hop h and
  *                   the source nodes of hop h-1's block, its first

@@ -137,7 +137,8 @@ def test_fused_driver_passes_corrupt_negative_ids_through(orc, capi):
     indices = indices.copy()
     rng = np.random.default_rng(2)
     hit = rng.permutation(len(indices))[: len(indices) // 10]
-    indices[hit] = rng.choice(np.array([-1, -2, -3, -4, -(2 ** 40), np.iinfo(np.int64).min + 2]), size=len(hit))
+    # (the fused driver keeps the 2^32 + 2 most negative values for its own slot states and turns such an id into -1)
+    indices[hit] = rng.choice(np.array([-1, -2, -3, -4, -(2 ** 40), np.iinfo(np.int64).min + 2 ** 33]), size=len(hit))
     og = orc.Graph(indptr, indices)
     dg = capi.Graph(dev(indptr), dev(indices))
     hops = [5, 10, 15]
