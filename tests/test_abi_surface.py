@@ -70,6 +70,10 @@ def test_argument_checks_need_no_gpu():
         assert L.apt_set_tuning(key, 0) == 0
     assert L.apt_set_tuning(b"block_fused_scan", 1) == 0
     assert L.apt_set_tuning(b"gather_vector_bytes", 3) != 0
+    for key in (b"relabel_lds",):
+        assert L.apt_set_tuning(key, 0) == 0 and L.apt_set_tuning(key, 1) == 0
+    assert L.apt_set_tuning(b"gather_wt_tail_mib", 64) == 0 and L.apt_set_tuning(b"gather_wt_tail_mib", 0) == 0
+    assert L.apt_set_tuning(b"gather_wt_tail_mib", -1) != 0
     assert L.apt_time_next_gather(None, None) == 0
 
 

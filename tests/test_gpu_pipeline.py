@@ -461,7 +461,12 @@ def test_fused_driver_random_configurations(orc, capi):
             pipe = MiniBatchPipeline(dg, None, B, hops, replace=replace, gather=False, fused=fused)
             pipe.run(dev(seeds), key)
             res = pipe.result()
-            assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in), (case, hops, B, replace, fused)
+            pipe.run(dev(seeds), key)                            # and again on the same buffers and table
+            again = pipe.result()
+            what = (case, hops, B, replace, fused)
+            assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in), what
+            assert torch.equal(again["input_nodes"], res["input_nodes"]), what
+            assert res["num_edges"] == again["num_edges"] == sum(int(b["counts"].sum()) for b in want_blocks), what
             for got, want in zip(res["blocks"], want_blocks):
                 for k in ("neighbors", "relabeled", "counts", "unique"):
-                    assert np.array_equal(got[k].cpu().numpy(), want[k]), (case, hops, B, replace, fused, k)
+                    assert np.array_equal(got[k].cpu().numpy(), want[k]), what + (k,)
