@@ -33,7 +33,9 @@
 // captured HIP graph replays correctly; when the epochs run out (every
 // 2^(32-P) - 1 calls) that kernel refills the table.
 // On the last hop the owners' ids are not even written to the table: the few
-// slots that lost a race fetch the id from the winner's output slot instead.
+// slots that lost a race fetch the id from an output slot instead: the one they
+// saw ahead of them when they lost (rank_table.hpp), or, if that one was
+// displaced itself, the winner's.
 #include "common.hpp"
 #include "rank_table.hpp"
 
