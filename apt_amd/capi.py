@@ -63,6 +63,11 @@ SYMBOLS = {
     "apt_minibatch_sample": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
                                   _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
                                   _SZ, _P]),
+    "apt_minibatch_sample_deferred": (_I, [C.POINTER(CGraph), _P, _I64, C.POINTER(C.c_int), _I, _I, _U64, _P,
+                                           _P, _I64, _P, C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), _P, _P,
+                                           _SZ, _P, _P]),
+    "apt_minibatch_lookup": (_I, [_P, _P]),
+    "apt_gather_rows_with_lookup": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P, _P]),
     "apt_count_ids": (_I, [_P, _I64, _P, _P, _I64, _P]),
     "apt_csr_row_degrees": (_I, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "apt_csr_copy_rows": (_I, [_P, _P, _I64, _P, _I64, _P, _I64, _P, _P]),
@@ -258,15 +263,36 @@ def relabel(seeds, neighbors, num_seeds_dev=None, neighbor_stride=0, unique=None
     return unique, relabeled, num_unique_dev
 
 
-def gather_rows(store, index, num_index_dev=None, out=None, miss_count=None):
-    """out[r, :] = feature row of node index[r] -> out [n, out_dim]."""
+def gather_rows(store, index, num_index_dev=None, out=None, miss_count=None, pending=None):
+    """out[r, :] = feature row of node index[r] -> out [n, out_dim].
+    pending: what MinibatchPlan.launch(defer_lookup=True) left to do (a PendingLookup); it is carried out in the
+    same launch."""
     index = _dev_i64(index, "index")
     n = index.numel()
     if out is None:
         out = torch.empty((n, store.out_dim), dtype=store.dtype, device=index.device)
-    check(lib().apt_gather_rows(C.byref(store.c), _ptr(index), n, _ptr(num_index_dev), _ptr(out),
-                                _ptr(miss_count), _stream()))
+    if pending is None:
+        check(lib().apt_gather_rows(C.byref(store.c), _ptr(index), n, _ptr(num_index_dev), _ptr(out),
+                                    _ptr(miss_count), _stream()))
+    else:
+        check(lib().apt_gather_rows_with_lookup(C.byref(store.c), _ptr(index), n, _ptr(num_index_dev), _ptr(out),
+                                                _ptr(miss_count), C.addressof(pending.c), _stream()))
+        pending.open = False
     return out
+
+
+class PendingLookup:
+    """Host-side description of a batch's last relabel pass (apt_pending_lookup)."""
+
+    def __init__(self):
+        self.c = (C.c_uint64 * 64)()
+        self.open = False       # filled and not yet carried out
+
+    def run(self):
+        """Carries the pass out as a launch of its own (if it is still open)."""
+        if self.open:
+            check(lib().apt_minibatch_lookup(C.addressof(self.c), _stream()))
+            self.open = False
 
 
 def _rows2d(t, name):
@@ -405,6 +431,7 @@ class MinibatchPlan:
         self.relabeled = [torch.empty(max(self.caps[h] * f, 1), **i64) for h, f in enumerate(self.fanouts)]
         self.counts = [torch.empty(max(self.caps[h], 1), **i64) for h in range(H)] if want_counts else None
         self.sizes = torch.zeros(H + 2, **i64)
+        self.pending = PendingLookup()
         self.rng_seed_dev = torch.zeros(1, **i64)
         self.table = table if table is not None else rank_table(graph.num_total_nodes, dev)
         self.table_len = graph.num_total_nodes
@@ -417,17 +444,24 @@ class MinibatchPlan:
         # the table and workspace were initialised on the current stream; the plan may be used on any
         torch.cuda.current_stream().synchronize()
 
-    def launch(self, seeds, rng_seed=None):
-        """Asynchronous.  rng_seed=None reads the seed from self.rng_seed_dev."""
+    def launch(self, seeds, rng_seed=None, defer_lookup=False):
+        """Asynchronous.  rng_seed=None reads the seed from self.rng_seed_dev.
+        defer_lookup: the relabel's last pass is left to the caller, who passes self.pending to gather_rows
+        (or calls self.pending.run()); until then relabeled[] is not final."""
         seeds = _dev_i64(seeds, "seeds")
         if seeds.numel() != self.batch:
             raise AptError(f"expected {self.batch} seeds, got {seeds.numel()}")
-        check(lib().apt_minibatch_sample(
-            C.byref(self.graph.c), _ptr(seeds), self.batch, self._cf, len(self.fanouts),
-            int(self.replace), 0 if rng_seed is None else int(rng_seed) & 0xFFFFFFFFFFFFFFFF,
-            _ptr(self.rng_seed_dev) if rng_seed is None else None, _ptr(self.table), self.table_len,
-            _ptr(self.nodes), self._nb, self._rl, self._ct, _ptr(self.sizes), _ptr(self.workspace),
-            self.workspace.numel(), _stream()))
+        args = (C.byref(self.graph.c), _ptr(seeds), self.batch, self._cf, len(self.fanouts),
+                int(self.replace), 0 if rng_seed is None else int(rng_seed) & 0xFFFFFFFFFFFFFFFF,
+                _ptr(self.rng_seed_dev) if rng_seed is None else None, _ptr(self.table), self.table_len,
+                _ptr(self.nodes), self._nb, self._rl, self._ct, _ptr(self.sizes), _ptr(self.workspace),
+                self.workspace.numel(), _stream())
+        self.pending.run()          # a pass still open from an earlier call goes first
+        if defer_lookup:
+            check(lib().apt_minibatch_sample_deferred(*args, C.addressof(self.pending.c)))
+            self.pending.open = True
+        else:
+            check(lib().apt_minibatch_sample(*args))
 
 
 def synth_copy(src, dst):

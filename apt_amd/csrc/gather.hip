@@ -12,6 +12,7 @@
 #include <hip/hip_ext.h>
 
 #include "common.hpp"
+#include "rank_table.hpp"
 
 namespace apt {
 
@@ -39,6 +40,7 @@ struct GatherParams {
   uint8_t* named;            // scatter only, optional: named[v] = 1 for every output row v that is written
   int store_policy;          // kStore* (apt_set_tuning gather_store_policy)
   int64_t wt_tail_bytes;     // kStoreAuto on a large output: the last bytes written go write-through
+  int lookup_blocks;         // the first workgroups of the grid do a batch's pending relabel lookups instead
 };
 
 template <int V> struct VecT;
@@ -106,8 +108,11 @@ __device__ __forceinline__ void store_row_vec(typename VecT<V>::type val, typena
 }
 
 // LPR lanes per row, R rows per group per step, V bytes per lane access.
+// A batch's pending relabel lookups (rank_table.hpp) can ride in the first
+// workgroups of the grid: they wait on a few dependent random reads while the
+// rest of the grid streams rows.
 template <int V, int LPR, int R>
-__global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
+__device__ __forceinline__ void gather_rows_of_block(const GatherParams& p, int64_t block, int64_t num_blocks) {
   using Vec = typename VecT<V>::type;
   constexpr int kGroups = kGatherBlock / LPR;
   const int64_t n = actual_count(p.n, p.n_dev);
@@ -124,8 +129,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
     wt_from = n * p.out_row_bytes <= kWriteThroughMaxBytes ? 0 : n - p.wt_tail_bytes / p.out_row_bytes;
   }
   int64_t misses = 0;
-  for (int64_t base = static_cast<int64_t>(blockIdx.x) * rows_per_block; base < n;
-       base += static_cast<int64_t>(gridDim.x) * rows_per_block) {
+  for (int64_t base = block * rows_per_block; base < n; base += num_blocks * rows_per_block) {
     const int policy = base >= wt_from ? kStoreWriteThrough : launch_policy;
     const char* src[R];
     char* dst[R];
@@ -169,6 +173,30 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
               static_cast<unsigned long long>(misses));
 }
 
+template <int V, int LPR, int R>
+__global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
+  gather_rows_of_block<V, LPR, R>(p, blockIdx.x, gridDim.x);
+}
+
+// The gather with a batch's pending relabel lookups in its grid (16-byte vectors, two rows in flight): the
+// grid's first workgroups do the lookup pass, whose dependent reads are then on their way while the rest stream
+// rows.  The lookup blocks are numbered after the gather's and the workgroup ids rotated, rather than numbering
+// them first and subtracting: written that way the row loop came out at 42 VGPRs instead of 40, and the 2048
+// workgroups that the grid of a small launch is capped at no longer ran together (27 instead of 22 us for
+// 235 k rows).
+template <int LPR>
+__global__ __launch_bounds__(kGatherBlock) void gather_with_lookup_kernel(GatherParams p, LookupParams lp) {
+  static_assert(kGatherBlock == kLookupBlock, "the lookup pass runs in workgroups of the gather's size");
+  const int64_t num_blocks = static_cast<int64_t>(gridDim.x) - p.lookup_blocks;
+  int64_t block = static_cast<int64_t>(blockIdx.x) + num_blocks;
+  if (block >= static_cast<int64_t>(gridDim.x)) block -= gridDim.x;
+  if (block >= num_blocks) {
+    lookup_block(lp, block - num_blocks);
+    return;
+  }
+  gather_rows_of_block<16, LPR, 2>(p, block, num_blocks);
+}
+
 static thread_local hipEvent_t t_gather_start = nullptr, t_gather_stop = nullptr;
 
 // Takes the one-shot events off the thread at entry; rearm() hands them to the
@@ -188,27 +216,32 @@ int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
 int tuning_gather_store_policy();
 int tuning_gather_wt_tail_mib();  // 0 = kWriteThroughTailMiB
 
-template <int V, int LPR>
-static int launch_gather_r(const GatherParams& p, hipStream_t st) {
-  int R = tuning_gather_rows();
-  // Rows per lane group in flight: two (with the settings alternating inside one process on the batch's own
-  // launches, two are 1-3 % faster than one at a quarter of a million rows and at three quarters; four are slower).
-  if (R != 1 && R != 2 && R != 4 && R != 8) R = 2;
-  const int groups = kGatherBlock / LPR;
-  // With a device-side count the host size is only an upper bound: a capped
-  // grid that strides over the rows avoids dispatching workgroups that would
-  // find nothing to do.  Where the bound says the launch is a small one, the cap
-  // is what the CUs hold at once (8 workgroups each): 23.7 against 24.4 us for
-  // the 235 k rows of a batch of 1024; for 725 k rows every cap from 2048 to
-  // 16384 gives the same 67 us.
+// Grid of a gather launch.  With a device-side count the host size is only an
+// upper bound: a capped grid that strides over the rows avoids dispatching
+// workgroups that would find nothing to do.  Where the bound says the launch is
+// a small one, the cap is what the CUs hold at once (8 workgroups each): 23.7
+// against 24.4 us for the 235 k rows of a batch of 1024; for 725 k rows every
+// cap from 2048 to 16384 gives the same 67 us.
+static int64_t gather_blocks(const GatherParams& p, int groups, int R) {
   int64_t max_blocks = tuning_gather_max_blocks();
   if (max_blocks <= 0)
     max_blocks = p.n_dev == nullptr                                    ? (1 << 20)
                  : p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? kGatherResidentBlocks
                                                                       : kGatherPersistentBlocks;
-  int64_t blocks = ceil_div(p.n, static_cast<int64_t>(groups) * R);
-  if (blocks > max_blocks) blocks = max_blocks;
-  const dim3 grid(static_cast<unsigned>(blocks)), block(kGatherBlock);
+  return std::min(ceil_div(p.n, static_cast<int64_t>(groups) * R), max_blocks);
+}
+
+// Rows per lane group in flight: two (with the settings alternating inside one process on the batch's own
+// launches, two are 1-3 % faster than one at a quarter of a million rows and at three quarters; four are slower).
+static int gather_rows_in_flight() {
+  const int R = tuning_gather_rows();
+  return (R == 1 || R == 2 || R == 4 || R == 8) ? R : 2;
+}
+
+template <int V, int LPR>
+static int launch_gather_r(const GatherParams& p, hipStream_t st) {
+  const int R = gather_rows_in_flight();
+  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, R))), block(kGatherBlock);
   // One-shot measurement hook: the launch itself records the two events
   // (kernel begin / kernel end), see apt_time_next_gather.
   hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;
@@ -262,12 +295,42 @@ static int launch_gather(const GatherParams& p, int elem_size, hipStream_t st) {
   }
 }
 
+// The gather with a pending lookup pass in its launch; false when this launch's geometry has no such kernel
+// (rows not movable as 16-byte vectors, or a rows-in-flight setting other than two): the caller then runs the
+// pass on its own.
+template <int LPR>
+static void launch_gather_with_lookup_r(GatherParams& p, const PendingLookup& lookup, hipStream_t st) {
+  p.lookup_blocks = static_cast<int>(lookup.blocks);
+  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, 2) + p.lookup_blocks)), block(kGatherBlock);
+  hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;
+  t_gather_start = t_gather_stop = nullptr;
+  if (ev0 != nullptr || ev1 != nullptr)
+    hipExtLaunchKernelGGL((gather_with_lookup_kernel<LPR>), grid, block, 0, st, ev0, ev1, 0, p, lookup.lp);
+  else
+    hipLaunchKernelGGL((gather_with_lookup_kernel<LPR>), grid, block, 0, st, p, lookup.lp);
+}
+
+static bool launch_gather_with_lookup(GatherParams& p, int elem_size, const PendingLookup& lookup, hipStream_t st) {
+  if (lookup.blocks == 0 || vector_bytes(p, elem_size) != 16 || gather_rows_in_flight() != 2) return false;
+  const int64_t vec_per_row = p.out_row_bytes / 16;
+  if (vec_per_row <= 8) launch_gather_with_lookup_r<8>(p, lookup, st);
+  else if (vec_per_row <= 16) launch_gather_with_lookup_r<16>(p, lookup, st);
+  else if (vec_per_row <= 32) launch_gather_with_lookup_r<32>(p, lookup, st);
+  else launch_gather_with_lookup_r<64>(p, lookup, st);
+  return true;
+}
+
 }  // namespace apt
 
-extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
-                               int64_t num_index, const int64_t* num_index_dev, void* out,
-                               int64_t* miss_count, void* stream) {
-  using namespace apt;
+extern "C" int apt_minibatch_lookup(const apt_pending_lookup* pending, void* stream);
+
+namespace apt {
+static int gather_rows(const apt_feat_store* store, const int64_t* index, int64_t num_index,
+                       const int64_t* num_index_dev, void* out, int64_t* miss_count, void* stream,
+                       const apt_pending_lookup* pending) {
+  const PendingLookup* lookup = reinterpret_cast<const PendingLookup*>(pending);
+  APT_REQUIRE(lookup == nullptr || lookup->magic == kPendingMagic, APT_EINVAL,
+              "apt_gather_rows_with_lookup: pending was not filled by apt_minibatch_sample_deferred");
   const TimingArm arm;  // a call that returns before its launch must not leave the events armed
   APT_REQUIRE(store != nullptr, APT_EINVAL, "apt_gather_rows: store is NULL");
   APT_REQUIRE(num_index >= 0, APT_EINVAL, "apt_gather_rows: num_index %lld < 0",
@@ -290,7 +353,7 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
               APT_EINVAL, "apt_gather_rows: cache rows need cache_table and pos_map");
   APT_REQUIRE(store->num_local_rows >= 0 && store->num_cache_rows >= 0, APT_EINVAL,
               "apt_gather_rows: negative row count");
-  if (num_index == 0) return APT_OK;
+  if (num_index == 0) return lookup != nullptr ? apt_minibatch_lookup(pending, stream) : APT_OK;
   APT_REQUIRE(index != nullptr && out != nullptr, APT_EINVAL,
               "apt_gather_rows: index/out is NULL");
   GatherParams p;
@@ -313,8 +376,36 @@ extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index
   p.named = nullptr;
   p.store_policy = tuning_gather_store_policy();
   p.wt_tail_bytes = (tuning_gather_wt_tail_mib() > 0 ? int64_t{tuning_gather_wt_tail_mib()} : kWriteThroughTailMiB) << 20;
+  p.lookup_blocks = 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (lookup != nullptr) {
+    arm.rearm();
+    if (launch_gather_with_lookup(p, store->elem_size, *lookup, st)) {
+      APT_LAUNCH_CHECK("gather_with_lookup_kernel");
+      return APT_OK;
+    }
+    const TimingArm again;  // nothing was launched: the events stay for the plain launch below
+    if (const int rc = apt_minibatch_lookup(pending, stream)) return rc;
+    again.rearm();
+    return launch_gather(p, store->elem_size, st);
+  }
   arm.rearm();
-  return launch_gather(p, store->elem_size, static_cast<hipStream_t>(stream));
+  return launch_gather(p, store->elem_size, st);
+}
+}  // namespace apt
+
+extern "C" int apt_gather_rows(const apt_feat_store* store, const int64_t* index,
+                               int64_t num_index, const int64_t* num_index_dev, void* out,
+                               int64_t* miss_count, void* stream) {
+  return apt::gather_rows(store, index, num_index, num_index_dev, out, miss_count, stream, nullptr);
+}
+
+extern "C" int apt_gather_rows_with_lookup(const apt_feat_store* store, const int64_t* index,
+                                           int64_t num_index, const int64_t* num_index_dev, void* out,
+                                           int64_t* miss_count, const apt_pending_lookup* pending,
+                                           void* stream) {
+  APT_REQUIRE(pending != nullptr, APT_EINVAL, "apt_gather_rows_with_lookup: pending is NULL");
+  return apt::gather_rows(store, index, num_index, num_index_dev, out, miss_count, stream, pending);
 }
 
 extern "C" int apt_time_next_gather(void* start_event, void* stop_event) {
@@ -355,6 +446,7 @@ static int permute_common(const void* in, const int64_t* perm, int64_t n, int64_
   p.named = named;
   p.store_policy = tuning_gather_store_policy();
   p.wt_tail_bytes = (tuning_gather_wt_tail_mib() > 0 ? int64_t{tuning_gather_wt_tail_mib()} : kWriteThroughTailMiB) << 20;
+  p.lookup_blocks = 0;
   arm.rearm();
   return launch_gather(p, elem_size, static_cast<hipStream_t>(stream));
 }

@@ -265,46 +265,8 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
   if (blockIdx.x == tiles - 1 && threadIdx.x == 0) *p.n_next = running;
 }
 
-struct LookupParams {
-  int num_hops;
-  int64_t block_begin[kMaxHops + 1];  // workgroup ranges per hop
-  const int64_t* neighbors[kMaxHops];
-  int64_t* relabeled[kMaxHops];
-  const int64_t* ns_dev[kMaxHops];
-  int64_t ns_cap[kMaxHops];
-  int64_t fanout[kMaxHops];
-  const uint32_t* table;
-  const uint32_t* state;
-  int last_is_bid;  // the last hop's table entries are still bids (see HopParams::last)
-};
-
 // Slots that lost the ownership race read the winner's id (all hops at once).
-__global__ __launch_bounds__(kMbBlock) void mb_lookup_kernel(LookupParams p) {
-  int h = 0;
-  while (h + 1 < p.num_hops && static_cast<int64_t>(blockIdx.x) >= p.block_begin[h + 1]) ++h;
-  const int64_t nn = actual_count(p.ns_cap[h], p.ns_dev[h]) * p.fanout[h];
-  const int64_t blocks = p.block_begin[h + 1] - p.block_begin[h];
-  const uint32_t tb = table_base(p.state);
-  const bool via_owner = p.last_is_bid && h == p.num_hops - 1;
-  const int64_t ns = actual_count(p.ns_cap[h], p.ns_dev[h]);
-  for (int64_t j = (static_cast<int64_t>(blockIdx.x) - p.block_begin[h]) * kMbBlock + threadIdx.x;
-       j < nn; j += blocks * kMbBlock) {
-    const int64_t r = p.relabeled[h][j];
-    if (r >= kSlotStatesEnd) continue;  // an id, or padding (any other negative value)
-    if (via_owner && r >= kSlotLoserSaw) {
-      // the slot that was seen with a smaller bid holds the node's id by now, unless it was displaced itself
-      const int64_t id = p.relabeled[h][r - kSlotLoserSaw];
-      if (id >= 0) {
-        p.relabeled[h][j] = id;
-        continue;
-      }
-    }
-    const int64_t e = p.table[p.neighbors[h][j]] - tb;
-    // via_owner: e is the winning bid ns + slot; the winner's slot holds the id
-    // (it is an owner, so its slot is final and never pending).
-    p.relabeled[h][j] = via_owner ? p.relabeled[h][e - ns] : e;
-  }
-}
+__global__ __launch_bounds__(kLookupBlock) void mb_lookup_kernel(LookupParams p) { lookup_block(p, blockIdx.x); }
 
 __global__ void mb_zero_state_kernel(uint32_t* state) { state[threadIdx.x] = 0; }
 
@@ -418,14 +380,17 @@ extern "C" int64_t apt_minibatch_capacity(int64_t batch, const int* hop_fanouts,
   return L.caps[hop];
 }
 
-extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
-                                    const int* hop_fanouts, int num_hops, int replace,
-                                    uint64_t rng_seed, const uint64_t* rng_seed_dev,
-                                    void* rank_table, int64_t rank_table_len, int64_t* nodes,
-                                    int64_t* const* neighbors, int64_t* const* relabeled,
-                                    int64_t* const* counts, int64_t* sizes, void* workspace,
-                                    size_t workspace_bytes, void* stream) {
-  using namespace apt;
+namespace apt {
+static int minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                            const int* hop_fanouts, int num_hops, int replace, uint64_t rng_seed,
+                            const uint64_t* rng_seed_dev, void* rank_table, int64_t rank_table_len,
+                            int64_t* nodes, int64_t* const* neighbors, int64_t* const* relabeled,
+                            int64_t* const* counts, int64_t* sizes, void* workspace,
+                            size_t workspace_bytes, void* stream, PendingLookup* defer) {
+  if (defer != nullptr) {
+    defer->magic = kPendingMagic;
+    defer->blocks = 0;
+  }
   APT_REQUIRE(graph != nullptr, APT_EINVAL, "apt_minibatch_sample: graph is NULL");
   APT_REQUIRE(batch >= 0, APT_EINVAL, "apt_minibatch_sample: batch %lld < 0", (long long)batch);
   APT_REQUIRE(hop_fanouts != nullptr && num_hops >= 1 && num_hops <= kMaxHops, APT_ELIMIT,
@@ -548,7 +513,52 @@ extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds
     nblocks += std::max<int64_t>(1, std::min<int64_t>(ceil_div(L.caps[h] * hop_fanouts[h], kMbBlock), 2048));
   }
   lp.block_begin[num_hops] = nblocks;
-  hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kMbBlock), 0, st, lp);
+  if (defer != nullptr) {  // the caller runs the pass: with the gather, or through apt_minibatch_lookup
+    defer->blocks = static_cast<uint32_t>(nblocks);
+    defer->lp = lp;
+    return APT_OK;
+  }
+  hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kLookupBlock), 0, st, lp);
+  APT_LAUNCH_CHECK("mb_lookup_kernel");
+  return APT_OK;
+}
+}  // namespace apt
+
+extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                                    const int* hop_fanouts, int num_hops, int replace,
+                                    uint64_t rng_seed, const uint64_t* rng_seed_dev,
+                                    void* rank_table, int64_t rank_table_len, int64_t* nodes,
+                                    int64_t* const* neighbors, int64_t* const* relabeled,
+                                    int64_t* const* counts, int64_t* sizes, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  return apt::minibatch_sample(graph, seeds, batch, hop_fanouts, num_hops, replace, rng_seed, rng_seed_dev,
+                               rank_table, rank_table_len, nodes, neighbors, relabeled, counts, sizes,
+                               workspace, workspace_bytes, stream, nullptr);
+}
+
+extern "C" int apt_minibatch_sample_deferred(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                                             const int* hop_fanouts, int num_hops, int replace,
+                                             uint64_t rng_seed, const uint64_t* rng_seed_dev,
+                                             void* rank_table, int64_t rank_table_len, int64_t* nodes,
+                                             int64_t* const* neighbors, int64_t* const* relabeled,
+                                             int64_t* const* counts, int64_t* sizes, void* workspace,
+                                             size_t workspace_bytes, void* stream,
+                                             apt_pending_lookup* pending) {
+  APT_REQUIRE(pending != nullptr, APT_EINVAL, "apt_minibatch_sample_deferred: pending is NULL");
+  return apt::minibatch_sample(graph, seeds, batch, hop_fanouts, num_hops, replace, rng_seed, rng_seed_dev,
+                               rank_table, rank_table_len, nodes, neighbors, relabeled, counts, sizes,
+                               workspace, workspace_bytes, stream,
+                               reinterpret_cast<apt::PendingLookup*>(pending));
+}
+
+extern "C" int apt_minibatch_lookup(const apt_pending_lookup* pending, void* stream) {
+  using namespace apt;
+  const PendingLookup* q = reinterpret_cast<const PendingLookup*>(pending);
+  APT_REQUIRE(q != nullptr && q->magic == kPendingMagic, APT_EINVAL,
+              "apt_minibatch_lookup: pending was not filled by apt_minibatch_sample_deferred");
+  if (q->blocks == 0) return APT_OK;
+  hipLaunchKernelGGL(mb_lookup_kernel, dim3(q->blocks), dim3(kLookupBlock), 0, static_cast<hipStream_t>(stream),
+                     q->lp);
   APT_LAUNCH_CHECK("mb_lookup_kernel");
   return APT_OK;
 }

@@ -80,4 +80,61 @@ __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const Rank
   return kSlotOwner;
 }
 
+// The pass that gives the slots that lost their race the winner's id, for all
+// hops of a batch at once.  It depends on the placing of the last hop's owners
+// and on nothing after it, and nothing but the caller's reading of relabeled[]
+// depends on it, so it can run as a kernel of its own (mb_lookup_kernel) or
+// ride along in the launch of the feature gather that follows the sampling
+// (gather.hip): the gather is bound by bandwidth, this pass by a few dependent
+// random reads.
+constexpr int kLookupBlock = 256;
+struct LookupParams {
+  int num_hops;
+  int64_t block_begin[APT_MAX_HOPS + 1];  // workgroup ranges per hop
+  const int64_t* neighbors[APT_MAX_HOPS];
+  int64_t* relabeled[APT_MAX_HOPS];
+  const int64_t* ns_dev[APT_MAX_HOPS];
+  int64_t ns_cap[APT_MAX_HOPS];
+  int64_t fanout[APT_MAX_HOPS];
+  const uint32_t* table;
+  const uint32_t* state;
+  int last_is_bid;  // the last hop's table entries are still bids (its ids are not written back)
+};
+
+// Work of workgroup `block` (of block_begin[num_hops]) of the pass; kLookupBlock threads.
+__device__ __forceinline__ void lookup_block(const LookupParams& p, int64_t block) {
+  int h = 0;
+  while (h + 1 < p.num_hops && block >= p.block_begin[h + 1]) ++h;
+  const int64_t ns = actual_count(p.ns_cap[h], p.ns_dev[h]);
+  const int64_t nn = ns * p.fanout[h];
+  const int64_t blocks = p.block_begin[h + 1] - p.block_begin[h];
+  const uint32_t tb = table_base(p.state);
+  const bool via_owner = p.last_is_bid && h == p.num_hops - 1;
+  for (int64_t j = (block - p.block_begin[h]) * kLookupBlock + threadIdx.x; j < nn; j += blocks * kLookupBlock) {
+    const int64_t r = p.relabeled[h][j];
+    if (r >= kSlotStatesEnd) continue;  // an id, or padding (any other negative value)
+    if (via_owner && r >= kSlotLoserSaw) {
+      // the slot that was seen with a smaller bid holds the node's id by now, unless it was displaced itself
+      const int64_t id = p.relabeled[h][r - kSlotLoserSaw];
+      if (id >= 0) {
+        p.relabeled[h][j] = id;
+        continue;
+      }
+    }
+    const int64_t e = p.table[p.neighbors[h][j]] - tb;
+    // via_owner: e is the winning bid ns + slot; the winner's slot holds the id
+    // (it is an owner, so its slot is final and never pending).
+    p.relabeled[h][j] = via_owner ? p.relabeled[h][e - ns] : e;
+  }
+}
+
+// What apt_pending_lookup holds.
+struct PendingLookup {
+  uint32_t magic;   // kPendingMagic when blocks and lp are valid
+  uint32_t blocks;  // workgroups of the pass; 0: nothing to do
+  LookupParams lp;
+};
+constexpr uint32_t kPendingMagic = 0x4C4B5550u;
+static_assert(sizeof(PendingLookup) <= sizeof(apt_pending_lookup), "apt_pending_lookup is too small");
+
 }  // namespace apt

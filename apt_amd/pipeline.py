@@ -22,7 +22,7 @@ from . import capi
 
 class MiniBatchPipeline:
     def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
-                 use_graph=False, requests=None, formats=False):
+                 use_graph=False, requests=None, formats=False, defer_lookup=False):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
         --fan_out list reversed).
 
@@ -33,6 +33,11 @@ class MiniBatchPipeline:
         which are gathered; the other buckets are the per-owner request lists
         that the reference would send (left in `request_ids`, grouped by
         bucket, sizes in `request_sizes`).
+
+        defer_lookup: run() lets the relabel's last pass (slots that lost the race for a node read the winner's id)
+        ride in the launch of the gather that follows it instead of launching it before: 3-5 % less time per
+        batch, while that launch gets 2-3 us longer (it is no longer the gather alone).  Only where the gather
+        is what follows the sampling (fused driver, features gathered, no requests, no formats).
 
         formats: True or "csc" also emits every hop's block as COO + CSC (+ CSR
         with True), what DGL derives from (row, col) in the reference
@@ -90,6 +95,9 @@ class MiniBatchPipeline:
             self.format_streams = [torch.cuda.Stream(device=dev) for _ in self.fanouts]
             self.format_fork = torch.cuda.Event()
             self.format_done = [torch.cuda.Event() for _ in self.fanouts]
+        # the relabel's last pass can ride in the gather's launch when the gather is what follows the sampling
+        self.can_defer_lookup = (bool(defer_lookup) and self.fused and self.features is not None
+                                 and requests is None and not formats)
         self.seeds = None
         self.sizes_host = None
         self.format_edges_host = None
@@ -121,14 +129,14 @@ class MiniBatchPipeline:
     def _capture(self):
         self.static_seeds = torch.zeros(self.caps[0], dtype=torch.int64, device=self.device)
         # run once eagerly so lazy initialisation happens outside the capture
-        self.plan.launch(self.static_seeds, rng_seed=None)
+        self.plan.launch(self.static_seeds, rng_seed=None, defer_lookup=self.can_defer_lookup)
         self.emit_formats()
         if self.features is not None:
             self.gather()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self.plan.launch(self.static_seeds, rng_seed=None)
+            self.plan.launch(self.static_seeds, rng_seed=None, defer_lookup=self.can_defer_lookup)
             self.emit_formats(join=False)
             if self.features is not None:
                 self.gather()
@@ -136,13 +144,15 @@ class MiniBatchPipeline:
         self.graph_exec = g
 
     # ------------------------------------------------------------ public
-    def sample(self, seeds, rng_seed):
-        """Sampling + relabel for every hop, asynchronous."""
+    def sample(self, seeds, rng_seed, defer_lookup=False):
+        """Sampling + relabel for every hop, asynchronous.
+        defer_lookup (fused driver, no requests, no formats): the relabel's last pass, which only the blocks'
+        compact ids wait for, is left to ride in the launch of the gather() that must follow."""
         if seeds.numel() != self.caps[0]:
             raise ValueError(f"expected {self.caps[0]} seeds, got {seeds.numel()}")
         self.seeds = seeds
         if self.fused:
-            self.plan.launch(seeds, rng_seed)
+            self.plan.launch(seeds, rng_seed, defer_lookup=defer_lookup and self.can_defer_lookup)
         else:
             self._sample_unfused(seeds, rng_seed)
 
@@ -178,8 +188,9 @@ class MiniBatchPipeline:
         H = len(self.fanouts)
         index = self.nodes if self.fused else self.frontier[H]
         if self.requests is None:
+            pending = self.plan.pending if self.fused and self.plan.pending.open else None
             capi.gather_rows(self.feat, index, num_index_dev=self._size(H), out=self.features,
-                             miss_count=self.misses)
+                             miss_count=self.misses, pending=pending)
             return
         rq = self.requests
         capi.cluster_reqs(index, rq["feat_pos_map"], rq["remote_worker_map"], rq["min_vids"],
@@ -197,7 +208,7 @@ class MiniBatchPipeline:
             self.seeds = self.static_seeds
             self.graph_exec.replay()
             return
-        self.sample(seeds, rng_seed)
+        self.sample(seeds, rng_seed, defer_lookup=True)
         self.emit_formats(join=False)
         if self.features is not None:
             self.gather()
@@ -228,6 +239,8 @@ class MiniBatchPipeline:
         apt_amd.layers take) instead of dicts; they live in this pipeline's buffers
         like everything else, so a training step must finish with them before the
         pipeline runs its next batch."""
+        if self.fused and self.plan.pending.open:      # sampled with the last pass deferred and never gathered
+            self.plan.pending.run()
         sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
         fmt_edges = None
         if self.formats is not None:

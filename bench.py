@@ -109,6 +109,10 @@ def parse_args():
     ap.add_argument("--ceilings", default="auto", choices=["auto", "on", "off"],
                     help="measure the GPU's rate for random 4-byte loads / stores / atomics (what bounds the sampling "
                          "kernel) and quote the last hop's sampling kernel against it; auto = on")
+    ap.add_argument("--defer_lookup", default="off", choices=["on", "off"],
+                    help="on: the relabel's last pass rides in the gather's launch instead of being a launch of its "
+                         "own before it (MiniBatchPipeline(defer_lookup=True)); the default run reports the batch "
+                         "time that way under stages.deferred_lookup")
     ap.add_argument("--alternate", type=str, default="",
                     help="settings to compare inside this one process, separated by '/', each a '+'-joined list of "
                          "knob=value (e.g. gather_wt_tail_mib=1/gather_wt_tail_mib=64): the batches of the timed region "
@@ -162,7 +166,10 @@ def gather_bytes_per_row(dim, esize, has_pos_map):
 def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, seed_n, store_of, synth, torch):
     """Batch 1024 on the same graph with 128 x bf16 and 128 x fp32 rows: the shape the gather target
     (>= 60 % of HBM peak) is stated on.  Every gather dispatch carries events; the sizes of every batch are
-    kept on the device and read afterwards, so each launch's rows and duration give its own fraction."""
+    kept on the device and read afterwards, so each launch's rows and duration give its own fraction.
+    The figures are of the gather kernel launched by itself (the relabel's last pass as a launch of its own
+    before it); the pipeline's default lets that pass ride in the gather's launch, which makes the batch
+    shorter and that launch a little longer: `with_lookup_riding` has the same batches that way."""
     B, Kt, Wt, H = 1024, args.target_steps, 20, len(hops)
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.seed + 77)
@@ -171,7 +178,8 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
         store = store_of(name)
         esize = store.local_table.element_size()
         moved, spec = gather_bytes_per_row(store.out_dim, esize, store.pos_map is not None)
-        pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused")
+        pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused",
+                                 defer_lookup=args.defer_lookup == "on")
         pool = torch.randperm(seed_n, generator=gen, device=dev)[:(Kt + Wt) * B]
         sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(Kt + Wt)]
         del pool
@@ -179,30 +187,44 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
         for i in range(Wt):
             pipe.run(sets[i], args.seed + 5000 + i)
         torch.cuda.synchronize()
-        pairs = []
-        step_ev = [torch.cuda.Event(enable_timing=True) for _ in range(Kt + 1)]
-        step_ev[0].record()
-        for i in range(Kt):
-            pipe.sample(sets[Wt + i], args.seed + 5000 + Wt + i)
-            pairs.append(kev.pair())
-            capi.check(capi.lib().apt_time_next_gather(*pairs[-1]))
-            pipe.gather()
-            log[i].copy_(pipe.sizes)
-            step_ev[i + 1].record()
-        torch.cuda.synchronize()
-        assert int(pipe.misses.item()) == 0
-        us = [kev.ms(pr) * 1e3 for pr in pairs]
-        rows = log[:, H].cpu().tolist()
+
+        def timed_pass(defer):
+            pairs = []
+            step_ev = [torch.cuda.Event(enable_timing=True) for _ in range(Kt + 1)]
+            step_ev[0].record()
+            for i in range(Kt):
+                pipe.sample(sets[Wt + i], args.seed + 5000 + Wt + i, defer_lookup=defer)
+                pairs.append(kev.pair())
+                capi.check(capi.lib().apt_time_next_gather(*pairs[-1]))
+                pipe.gather()
+                log[i].copy_(pipe.sizes)
+                step_ev[i + 1].record()
+            torch.cuda.synchronize()
+            assert int(pipe.misses.item()) == 0
+            us = [kev.ms(pr) * 1e3 for pr in pairs]
+            rows = log[:, H].cpu().tolist()
+            frac = [r * moved / (t * 1e-6) / 1e9 / HBM_PEAK_GBPS for r, t in zip(rows, us)]
+            return us, rows, frac, [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(Kt)]
+
+        def wall_pass(defer):
+            """The same batches back to back without events or size copies: wall time per batch."""
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(Kt):
+                pipe.sample(sets[Wt + i], args.seed + 5000 + Wt + i, defer_lookup=defer)
+                pipe.gather()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / Kt
+
+        us, rows, frac, step_ms = timed_pass(False)
         edges = log[:, H + 1].cpu().tolist()
-        frac = [r * moved / (t * 1e-6) / 1e9 / HBM_PEAK_GBPS for r, t in zip(rows, us)]
-        step_ms = [step_ev[i].elapsed_time(step_ev[i + 1]) for i in range(Kt)]
-        # the same batches back to back without events or size copies: wall time per batch
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(Kt):
-            pipe.run(sets[Wt + i], args.seed + 5000 + Wt + i)
-        torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / Kt
+        wall_alone = wall_pass(False)
+        riding = None
+        if pipe.can_defer_lookup:
+            us_r, _, frac_r, _ = timed_pass(True)
+            riding = {"us_median": quantiles(us_r)["median"], "frac": quantiles(frac_r)["median"],
+                      "frac_p10": quantiles(frac_r)["p10"], "ms_per_step": wall_pass(True) * 1e3}
+        wall = riding["ms_per_step"] * 1e-3 if riding else wall_alone     # what a pipeline does by default
         q_us, q_frac = quantiles(us), quantiles(frac)
         out[name] = {
             "rows": sum(rows) / Kt, "bytes_per_row": moved, "bytes_per_row_definition": spec,
@@ -215,8 +237,10 @@ def stage_target_shape(args, capi, dev, graph, hops, kev, MiniBatchPipeline, N, 
             "traffic_bytes_per_row": MEASURED_GATHER_TRAFFIC_PER_ROW.get(("target", name, store.out_dim, B), (None, None))[0],
             "traffic_source": MEASURED_GATHER_TRAFFIC_PER_ROW.get(("target", name, store.out_dim, B), (None, None))[1],
             "GBps_median": q_frac["median"] * HBM_PEAK_GBPS,
-            "ms_per_step": wall * 1e3, "ms_per_step_events": quantiles(step_ms),
+            "ms_per_step": wall * 1e3, "ms_per_step_gather_launched_alone": wall_alone * 1e3,
+            "ms_per_step_events": quantiles(step_ms),
             "edges_per_s": sum(edges) / Kt / wall,
+            "with_lookup_riding": riding,
         }
         del pipe, log, sets
     return out
@@ -395,7 +419,7 @@ def stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, see
                     g, s = kev.pair(), kev.pair()
                     if args.driver == "fused":
                         capi.check(capi.lib().apt_time_next_sample(H - 1, s[0], s[1]))
-                    pipe.sample(sets[i], args.seed + 900 + i)
+                    pipe.sample(sets[i], args.seed + 900 + i, defer_lookup=True)
                     capi.check(capi.lib().apt_time_next_gather(g[0], g[1]))
                     pipe.gather()
                     gp.append(g)
@@ -776,7 +800,7 @@ def main():
 
     def make_pipe(use_graph):
         return MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused",
-                                 use_graph=use_graph, requests=requests)
+                                 use_graph=use_graph, requests=requests, defer_lookup=args.defer_lookup == "on")
 
     pipe = make_pipe(args.driver == "graph")
     # the per-stage pass brackets stages with events, which a graph replay does not allow
@@ -805,7 +829,7 @@ def main():
             return
         if sk is not None:   # the last hop's sampling kernel records its begin / end
             capi.check(capi.lib().apt_time_next_sample(H - 1, sk[0], sk[1]))
-        p.sample(seeds, key)
+        p.sample(seeds, key, defer_lookup=True)   # as run() does: the relabel's last pass rides in the gather's launch
         capi.check(capi.lib().apt_time_next_gather(gk[0], gk[1]))   # the gather dispatch records its begin / end
         p.gather()
 
@@ -867,7 +891,7 @@ def main():
     for i in range(K):
         m = (ev(), ev(), ev())
         m[0].record()
-        stage_pipe.sample(seed_sets[W + i], args.seed + 100 + W + i)
+        stage_pipe.sample(seed_sets[W + i], args.seed + 100 + W + i, defer_lookup=True)
         m[1].record()
         stage_pipe.gather()
         m[2].record()
@@ -887,6 +911,31 @@ def main():
     bytes_per_row, bytes_per_row_def = gather_bytes_per_row(w["dim"], esize, store.pos_map is not None)
     gather_gbps = rows * bytes_per_row / (t_gather * 1e-3) / 1e9
     edges_per_s = edges / elapsed
+
+    # ---- the same K batches with the relabel's last pass riding in the gather's launch
+    # (MiniBatchPipeline(defer_lookup=True)): that launch is then no longer the gather alone, which is why
+    # the timed region above, and with it `roofline`, keeps the pass as a launch of its own
+    deferred = None
+    if args.defer_lookup == "off" and args.driver == "fused" and requests is None:
+        dp = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, defer_lookup=True)
+        for i in range(W):
+            dp.run(seed_sets[i], args.seed + 100 + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            dp.run(seed_sets[W + i], args.seed + 100 + W + i)
+        torch.cuda.synchronize()
+        t_def = time.perf_counter() - t0
+        pairs = []
+        for i in range(min(K, 25)):
+            dp.sample(seed_sets[W + i], args.seed + 100 + W + i, defer_lookup=True)
+            pairs.append(kev.pair())
+            capi.check(capi.lib().apt_time_next_gather(*pairs[-1]))
+            dp.gather()
+        torch.cuda.synchronize()
+        deferred = {"ms_per_step": t_def / K * 1e3, "edges_per_s": edges / t_def,
+                    "gather_launch_with_the_pass_us": sum(kev.ms(pr) for pr in pairs) / len(pairs) * 1e3}
+        del dp
 
     # ---- the same K batches with N batches in flight: N pipelines (own buffers, rank table) on N
     # streams, batches dealt round-robin; reported beside the single-stream figure
@@ -1080,6 +1129,10 @@ def main():
                                         if staged else None),
             "timing": (f"HIP events carried by {len(timed_steps)} of the {K} gather dispatches of the timed region "
                        f"(kernel begin / end)" if staged else "HIP events recorded around each gather launch of an untimed pass"),
+            # with the pipeline's default the batch's last relabel pass rides in the first workgroups of this launch
+            # (--defer_lookup off launches it on its own before the gather); its bytes are not counted above
+            "launch_also_carries": ("the batch's last relabel pass (rank-table lookups of the slots that lost a race)"
+                                    if pipe.can_defer_lookup else None),
         },
         "roofline_sampling": roofline_sampling,
         "cpu_baseline": cpu,
@@ -1098,6 +1151,7 @@ def main():
             "random_access_ceilings": ceilings,
             "random_access_by_table_size": ceilings_by_size,
             "in_flight": in_flight,
+            "deferred_lookup": deferred,
             "edges_per_step": edges / K,
             "input_nodes_per_step": rows / K,
             "sample_relabel_ms": t_sample / K,

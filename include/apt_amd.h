@@ -45,6 +45,13 @@ extern "C" {
 #define APT_EHIP (-4)    /* a HIP runtime call failed */
 
 #define APT_MAX_HOPS 8
+
+/* Filled by apt_minibatch_sample_deferred: the description of a batch's last
+ * relabel pass, for apt_gather_rows_with_lookup or apt_minibatch_lookup to
+ * carry out.  Host memory, opaque, valid while the batch's buffers are. */
+typedef struct apt_pending_lookup {
+  uint64_t opaque[64];
+} apt_pending_lookup;
 #define APT_MAX_BUCKETS 64 /* reference: MAX_NUM_DEVICES 33 (src/cuda/npc_kernel.h:13) */
 
 const char* apt_last_error(void);
@@ -347,6 +354,34 @@ int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t b
                          int64_t* const* neighbors, int64_t* const* relabeled,
                          int64_t* const* counts, int64_t* sizes, void* workspace,
                          size_t workspace_bytes, void* stream);
+
+/* apt_minibatch_sample in two parts, for a caller that gathers the batch's
+ * features right after sampling it (no counterpart in the reference, where
+ * sampling and load_subtensor are separate operators, python/npc/sampler.py:
+ * 187-203 and python/npc/ops.py load_subtensor).  The last pass of the relabel
+ * (slots that lost the race for a node read the winner's id) needs only the
+ * placing of the last hop's owners before it and nothing but relabeled[] after
+ * it, and it waits on a few dependent random reads, while the gather is bound
+ * by bandwidth: apt_minibatch_sample_deferred leaves that pass out and
+ * describes it in *pending; apt_gather_rows_with_lookup runs it in the first
+ * workgroups of the gather's own launch (same stream, no other launch between
+ * the two calls may touch the batch's buffers), apt_minibatch_lookup runs it as
+ * a launch of its own.  Until one of the two has run, relabeled[h] holds slot
+ * states in some places; nodes, neighbors, counts and sizes are final.
+ * Results are those of apt_minibatch_sample + apt_gather_rows, bit for bit. */
+int apt_minibatch_sample_deferred(const apt_graph* graph, const int64_t* seeds, int64_t batch,
+                                  const int* hop_fanouts, int num_hops, int replace,
+                                  uint64_t rng_seed, const uint64_t* rng_seed_dev,
+                                  void* rank_table, int64_t rank_table_len, int64_t* nodes,
+                                  int64_t* const* neighbors, int64_t* const* relabeled,
+                                  int64_t* const* counts, int64_t* sizes, void* workspace,
+                                  size_t workspace_bytes, void* stream,
+                                  apt_pending_lookup* pending);
+int apt_minibatch_lookup(const apt_pending_lookup* pending, void* stream);
+int apt_gather_rows_with_lookup(const apt_feat_store* store, const int64_t* index,
+                                int64_t num_index, const int64_t* num_index_dev, void* out,
+                                int64_t* miss_count, const apt_pending_lookup* pending,
+                                void* stream);
 
 /* Cache construction (the callers of the registries).
  *   apt_count_ids        freq[ids[i]] += 1 for ids in [0, num_total_nodes): the

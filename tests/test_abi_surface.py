@@ -75,6 +75,10 @@ def test_argument_checks_need_no_gpu():
     assert L.apt_set_tuning(b"gather_wt_tail_mib", 64) == 0 and L.apt_set_tuning(b"gather_wt_tail_mib", 0) == 0
     assert L.apt_set_tuning(b"gather_wt_tail_mib", -1) != 0
     assert L.apt_time_next_gather(None, None) == 0
+    blank = (ctypes.c_uint64 * 64)()
+    assert L.apt_minibatch_lookup(ctypes.addressof(blank), None) != 0 and b"pending" in L.apt_last_error()
+    assert L.apt_minibatch_lookup(None, None) != 0
+    assert L.apt_gather_rows_with_lookup(None, None, 0, None, None, None, None, None) != 0
 
 
 REFERENCE_OPS = {   # reference src/pybind.cc:19-47 with the schemas torch infers from the C++ types

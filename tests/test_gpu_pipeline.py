@@ -470,3 +470,59 @@ def test_fused_driver_random_configurations(orc, capi):
             for got, want in zip(res["blocks"], want_blocks):
                 for k in ("neighbors", "relabeled", "counts", "unique"):
                     assert np.array_equal(got[k].cpu().numpy(), want[k]), what + (k,)
+
+
+def test_deferred_lookup_rides_in_the_gather_or_runs_alone(orc, capi):
+    """apt_minibatch_sample_deferred leaves the relabel's last pass to the caller: carried out inside the gather's
+    launch, as a launch of its own, or by result() as a last resort, the batch is the one apt_minibatch_sample
+    gives.  Many repeated neighbours (a dense little graph), so that plenty of slots lose their race."""
+    from apt_amd.pipeline import MiniBatchPipeline
+    indptr, indices, feats = _setup(orc, capi, n=3000, deg=40, dim=64, seed=13)
+    og = orc.Graph(indptr, indices)
+    dg = capi.Graph(dev(indptr), dev(indices))
+    fs = capi.FeatStore(dev(feats))
+    hops = [5, 10, 15]
+    seeds = np.random.default_rng(8).integers(0, 3000, size=700)
+    want_in, want_blocks = orc.sample_blocks(og, seeds, hops, False, 3)
+    want_f, _ = orc.gather_rows(orc.FeatStore(feats), want_in)
+    assert sum(int((b["relabeled"] >= 0).sum()) for b in want_blocks) > 3 * len(want_in)
+
+    def check(res):
+        assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+        for got, want in zip(res["blocks"], want_blocks):
+            for k in ("neighbors", "relabeled", "counts", "unique"):
+                assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+
+    pipe = MiniBatchPipeline(dg, fs, 700, hops, replace=False, defer_lookup=True)
+    assert pipe.can_defer_lookup and not MiniBatchPipeline(dg, fs, 700, hops).can_defer_lookup   # opt-in
+    pipe.sample(dev(seeds), 3, defer_lookup=True)
+    assert pipe.plan.pending.open
+    torch.cuda.synchronize()
+    pending_slots = sum(int((r[: s * f] < -(2 ** 62)).sum()) for r, s, f in
+                        zip(pipe.relabeled, pipe.sizes.cpu().tolist(), hops))
+    assert pending_slots > 0                                    # the pass really was left out
+    pipe.gather()                                               # ... and rides here
+    assert not pipe.plan.pending.open
+    res = pipe.result()
+    check(res)
+    assert np.array_equal(res["features"].cpu().numpy(), want_f)
+    pipe.sample(dev(seeds), 3, defer_lookup=True)
+    pipe.plan.pending.run()                                     # a launch of its own
+    check(pipe.result())
+    pipe.sample(dev(seeds), 3, defer_lookup=True)
+    check(pipe.result())                                        # never gathered: result() carries it out
+    pipe.sample(dev(seeds), 3)                                  # not deferred
+    assert not pipe.plan.pending.open
+    check(pipe.result())
+    # a pipeline that has other readers of the compact ids between sampling and gather does not defer
+    assert not MiniBatchPipeline(dg, fs, 700, hops, formats="csc", defer_lookup=True).can_defer_lookup
+    assert not MiniBatchPipeline(dg, None, 700, hops, gather=False, defer_lookup=True).can_defer_lookup
+    # run() the deferred way, eager and as a replayed graph, on rows that are not 16-byte vectors too (the pass
+    # then runs on its own inside the same call)
+    for store, use_graph in ((fs, False), (fs, True), (capi.FeatStore(dev(feats[:, :63].copy())), False)):
+        p2 = MiniBatchPipeline(dg, store, 700, hops, defer_lookup=True, use_graph=use_graph)
+        for key in (3, 3):
+            p2.run(dev(seeds), key)
+            res = p2.result()
+            check(res)
+            assert res["features"].shape[1] == store.out_dim
