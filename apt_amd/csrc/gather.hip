@@ -18,7 +18,7 @@ namespace apt {
 
 constexpr int kGatherBlock = 256;
 constexpr int kGatherPersistentBlocks = 16384;
-constexpr int kGatherResidentBlocks = 2048;   // 256 CUs x 8 workgroups of 256 threads
+constexpr int kGatherResidentBlocks = 2048;   // 256 CUs x 8 workgroups of 256 threads (if the runtime cannot be asked)
 
 struct GatherParams {
   const char* local_table;
@@ -216,17 +216,36 @@ int tuning_gather_vector_bytes();  // 0 = as wide as alignment allows (16)
 int tuning_gather_store_policy();
 int tuning_gather_wt_tail_mib();  // 0 = kWriteThroughTailMiB
 
+// How many workgroups of a kernel the GPU holds at once (asked once per kernel; 2048 for the plain gather of
+// 16-byte vectors: 8 on each of 256 CUs).
+template <typename Kernel>
+static int64_t resident_blocks(Kernel kernel) {
+  static const int64_t blocks = [kernel] {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kGatherBlock, 0) != hipSuccess ||
+        cus <= 0 || per_cu <= 0) {
+      (void)hipGetLastError();
+      return static_cast<int64_t>(kGatherResidentBlocks);
+    }
+    return static_cast<int64_t>(cus) * per_cu;
+  }();
+  return blocks;
+}
+
 // Grid of a gather launch.  With a device-side count the host size is only an
 // upper bound: a capped grid that strides over the rows avoids dispatching
 // workgroups that would find nothing to do.  Where the bound says the launch is
-// a small one, the cap is what the CUs hold at once (8 workgroups each): 23.7
-// against 24.4 us for the 235 k rows of a batch of 1024; for 725 k rows every
-// cap from 2048 to 16384 gives the same 67 us.
-static int64_t gather_blocks(const GatherParams& p, int groups, int R) {
+// a small one, the cap is what the CUs hold at once (`resident`): 23.7 against
+// 24.4 us for the 235 k rows of a batch of 1024 (and 27 us when the cap is
+// more than what they hold); for 725 k rows every cap from 2048 to 16384 gives
+// the same 67 us.
+static int64_t gather_blocks(const GatherParams& p, int groups, int R, int64_t resident) {
   int64_t max_blocks = tuning_gather_max_blocks();
   if (max_blocks <= 0)
     max_blocks = p.n_dev == nullptr                                    ? (1 << 20)
-                 : p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? kGatherResidentBlocks
+                 : p.n * p.out_row_bytes <= 5 * kWriteThroughMaxBytes ? resident
                                                                       : kGatherPersistentBlocks;
   return std::min(ceil_div(p.n, static_cast<int64_t>(groups) * R), max_blocks);
 }
@@ -241,7 +260,11 @@ static int gather_rows_in_flight() {
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   const int R = gather_rows_in_flight();
-  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, R))), block(kGatherBlock);
+  const int64_t resident = R == 1   ? resident_blocks(gather_kernel<V, LPR, 1>)
+                           : R == 2 ? resident_blocks(gather_kernel<V, LPR, 2>)
+                           : R == 8 ? resident_blocks(gather_kernel<V, LPR, 8>)
+                                    : resident_blocks(gather_kernel<V, LPR, 4>);
+  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, R, resident))), block(kGatherBlock);
   // One-shot measurement hook: the launch itself records the two events
   // (kernel begin / kernel end), see apt_time_next_gather.
   hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;
@@ -301,7 +324,9 @@ static int launch_gather(const GatherParams& p, int elem_size, hipStream_t st) {
 template <int LPR>
 static void launch_gather_with_lookup_r(GatherParams& p, const PendingLookup& lookup, hipStream_t st) {
   p.lookup_blocks = static_cast<int>(lookup.blocks);
-  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, 2) + p.lookup_blocks)), block(kGatherBlock);
+  const int64_t resident = resident_blocks(gather_with_lookup_kernel<LPR>);
+  const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, 2, resident) + p.lookup_blocks)),
+      block(kGatherBlock);
   hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;
   t_gather_start = t_gather_stop = nullptr;
   if (ev0 != nullptr || ev1 != nullptr)
