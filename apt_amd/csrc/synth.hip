@@ -96,7 +96,8 @@ __device__ __forceinline__ uint64_t probe_mix(uint64_t x) {
 // One access per item to a pseudo-random word of a table: what bounds the
 // sampling and relabel kernels (one transaction per sampled id), as opposed to
 // bytes.  MODE 0 load, 1 store, 2 atomicMin without use of the result,
-// 3 atomicMin whose result is used, 4 16-byte load.
+// 3 atomicMin whose result is used, 4 16-byte load, 5 a load and an atomicMin at two
+// independent places (do the two kinds of access add up or overlap?).
 template <int MODE>
 __global__ __launch_bounds__(kSynBlock) void random_access_kernel(uint32_t* table, uint64_t words, int64_t n,
                                                                   uint32_t salt, uint32_t* sink) {
@@ -108,7 +109,11 @@ __global__ __launch_bounds__(kSynBlock) void random_access_kernel(uint32_t* tabl
     else if (MODE == 1) table[w] = static_cast<uint32_t>(i);
     else if (MODE == 2) atomicMin(&table[w], static_cast<uint32_t>(i) | 0x80000000u);
     else if (MODE == 3) acc += atomicMin(&table[w], static_cast<uint32_t>(i) | 0x80000000u);
-    else {
+    else if (MODE == 5) {
+      const uint64_t w2 = probe_mix(static_cast<uint64_t>(i) * 3 + 1 + (static_cast<uint64_t>(salt) << 40)) % words;
+      acc += __builtin_nontemporal_load(&table[w]);
+      atomicMin(&table[w2], static_cast<uint32_t>(i) | 0x80000000u);
+    } else {
       const uint4 v = *reinterpret_cast<const uint4*>(&table[w & ~uint64_t{3}]);
       acc += v.x + v.w;
     }
@@ -121,7 +126,7 @@ __global__ __launch_bounds__(kSynBlock) void random_access_kernel(uint32_t* tabl
 extern "C" int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
                                        uint32_t salt, void* sink, void* stream) {
   using namespace apt;
-  APT_REQUIRE(mode >= 0 && mode <= 4, APT_EINVAL, "apt_synth_random_access: mode %d outside 0..4", mode);
+  APT_REQUIRE(mode >= 0 && mode <= 5, APT_EINVAL, "apt_synth_random_access: mode %d outside 0..5", mode);
   APT_REQUIRE(table != nullptr && sink != nullptr && table_bytes >= 16 && table_bytes % 16 == 0 &&
                   (reinterpret_cast<uintptr_t>(table) & 15) == 0,
               APT_EINVAL, "apt_synth_random_access: table must be 16-byte aligned, a multiple of 16 bytes long");
@@ -137,6 +142,7 @@ extern "C" int apt_synth_random_access(int mode, void* table, int64_t table_byte
     case 1: hipLaunchKernelGGL(random_access_kernel<1>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
     case 2: hipLaunchKernelGGL(random_access_kernel<2>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
     case 3: hipLaunchKernelGGL(random_access_kernel<3>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
+    case 5: hipLaunchKernelGGL(random_access_kernel<5>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
     default: hipLaunchKernelGGL(random_access_kernel<4>, grid, block, 0, st, t, words, num_accesses, salt, sk); break;
   }
   APT_LAUNCH_CHECK("random_access_kernel");

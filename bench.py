@@ -454,7 +454,8 @@ def stage_ceilings(capi, dev, N, torch, table_bytes=None):
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     n = 8_000_000
     res = {"table_bytes": nbytes, "accesses_per_launch": n}
-    for mode, name in ((0, "load"), (1, "store"), (2, "atomic_min"), (3, "atomic_min_returning"), (4, "load_16B")):
+    for mode, name in ((0, "load"), (1, "store"), (2, "atomic_min"), (3, "atomic_min_returning"), (4, "load_16B"),
+                       (5, "load_and_atomic_min_pairs")):
         ts = []
         for rep in range(7):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -37,7 +37,8 @@ int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream);
  * transactions, not by bytes; the benchmark measures the GPU's rate for them
  * with this call and quotes the kernels against it.
  *   mode  0 load, 1 store, 2 atomicMin (result unused), 3 atomicMin (result
- *         used), 4 aligned 16-byte load
+ *         used), 4 aligned 16-byte load, 5 a load and an atomicMin at two
+ *         independent random places per work item
  *   salt  varies the address sequence between calls
  *   sink  device uint32[1] (never written in practice; keeps loads alive) */
 int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
