@@ -1,4 +1,6 @@
-"""Builds libapt_hip.so (the C-ABI HIP library) for gfx950 with hipcc, and libnpc.so.
+"""Builds libapt_hip.so (the C-ABI HIP library) for gfx950 with hipcc, libnpc.so (its torch
+operator binding) and libapt_bench.so (synthetic inputs and measurement helpers of the benchmark
+and the tests: a library of its own, so that libapt_hip.so exports the product ABI only).
 
 Run it as a script (`python apt_amd/build.py`): importing it as `apt_amd.build`
 would first import the package, which needs the libraries this file produces.
@@ -15,7 +17,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libapt_hip.so")
 NPC_LIB = os.path.join(HERE, "libnpc.so")
-SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "minibatch.hip", "spmm.hip", "cache.hip", "block.hip", "synth.hip"]
+BENCH_LIB = os.path.join(HERE, "libapt_bench.so")
+SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "minibatch.hip", "spmm.hip", "cache.hip", "block.hip"]
+BENCH_SOURCES = ["synth.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -35,11 +39,11 @@ def build(force=True, verbose=False):
     headers = [os.path.join(CSRC, h) for h in sorted(os.listdir(CSRC)) if h.endswith(".hpp")]
     headers += [os.path.join(HERE, "..", "include", "apt_amd.h"), os.path.join(HERE, "..", "include", "apt_synth.h")]
     newest_hdr = max(os.path.getmtime(h) for h in headers)
-    objs = []
-    for s in SOURCES:
+    objs, bench_objs = [], []
+    for s in SOURCES + BENCH_SOURCES:
         src = os.path.join(CSRC, s)
         obj = _obj(s)
-        objs.append(obj)
+        (bench_objs if s in BENCH_SOURCES else objs).append(obj)
         stale = (force or not os.path.exists(obj)
                  or os.path.getmtime(obj) < max(os.path.getmtime(src), newest_hdr))
         if stale:
@@ -56,8 +60,9 @@ def build(force=True, verbose=False):
             raise RuntimeError(f"hipcc failed on {s}:\n{text}")
         if verbose and text.strip():
             print(text, file=sys.stderr)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
-    subprocess.check_call(cmd)
+    # -Bsymbolic: each library binds its own helpers (both define apt::last_error_buf)
+    for lib, parts in ((LIB, objs), (BENCH_LIB, bench_objs)):
+        subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", lib, *parts])
     build_torch_binding(verbose=verbose)
     return LIB
 

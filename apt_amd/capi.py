@@ -83,14 +83,19 @@ SYMBOLS = {
     "apt_gat_block": (_I, [_P, _I64, _P, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P]),
     "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
     "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P, _P]),
-    # include/apt_synth.h
+    "apt_time_next_sample": (_I, [_I, _P, _P]),
+}
+
+# every symbol include/apt_synth.h declares (libapt_bench.so: inputs and probes of the benchmark and the tests)
+BENCH_LIB_PATH = os.path.join(_HERE, "libapt_bench.so")
+BENCH_SYMBOLS = {
+    "apt_synth_last_error": (C.c_char_p, []),
     "apt_synth_rmat_fill": (_I, [_P, _I64, _I64, _I64, _I64, _I, _U64, C.c_uint32, C.c_uint32, _P, _P]),
     "apt_synth_copy": (_I, [_P, _P, _I64, _P]),
     "apt_synth_random_access": (_I, [_I, _P, _I64, _I64, C.c_uint32, _P, _P]),
-    "apt_synth_grid_barrier": (_I, [_I, _I, _P, _P, _P]),
-    "apt_synth_empty_launches": (_I, [_I, _P, _P]),
-    "apt_time_next_sample": (_I, [_I, _P, _P]),
+    "apt_synth_symmetrize_fill": (_I, [_P, _P, _I64, _I64, _P, _P, _P, _P]),
 }
+_bench_lib = None
 
 
 def lib():
@@ -113,6 +118,26 @@ def lib():
 def check(status):
     if status != 0:
         raise AptError(f"[{status}] {lib().apt_last_error().decode()}")
+
+
+def bench_lib():
+    """Load libapt_bench.so (built by apt_amd/build.py beside libapt_hip.so).  Raises if absent."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with `python apt_amd/build.py`")
+        L = C.CDLL(BENCH_LIB_PATH)
+        for name, (res, args) in BENCH_SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _bench_lib = L
+    return _bench_lib
+
+
+def bench_check(status):
+    if status != 0:
+        raise AptError(f"[{status}] {bench_lib().apt_synth_last_error().decode()}")
 
 
 def set_tuning(key, value):
@@ -392,11 +417,30 @@ def synth_rmat_fill(indptr, row_begin, num_nodes, num_edges, levels, seed, thr0,
     indices = _dev_i64(indices, "indices")
     if indices.numel() < num_edges:
         raise AptError("synth_rmat_fill: buffer sizes do not match")
-    check(lib().apt_synth_rmat_fill(_ptr(indptr), indptr.numel() - 1, int(row_begin), int(num_nodes),
-                                    int(num_edges), int(levels),
-                                    int(seed) & 0xFFFFFFFFFFFFFFFF, int(thr0), int(thr1),
-                                    _ptr(indices), _stream()))
+    bench_check(bench_lib().apt_synth_rmat_fill(_ptr(indptr), indptr.numel() - 1, int(row_begin), int(num_nodes),
+                                                int(num_edges), int(levels),
+                                                int(seed) & 0xFFFFFFFFFFFFFFFF, int(thr0), int(thr1),
+                                                _ptr(indices), _stream()))
     return indices
+
+
+def synth_symmetrize_fill(fwd_indptr, fwd_indices, indptr, out):
+    """Rows of the symmetrised graph with a self-loop per node, unsorted (apt_synth_symmetrize_fill)."""
+    fwd_indptr, fwd_indices = _dev_i64(fwd_indptr, "fwd_indptr"), _dev_i64(fwd_indices, "fwd_indices")
+    indptr, out = _dev_i64(indptr, "indptr"), _dev_i64(out, "out")
+    n = fwd_indptr.numel() - 1
+    if indptr.numel() != n + 1:
+        raise AptError("synth_symmetrize_fill: indptr must have as many entries as fwd_indptr")
+    cursor = torch.zeros(n, dtype=torch.int32, device=out.device)
+    bench_check(bench_lib().apt_synth_symmetrize_fill(_ptr(fwd_indptr), _ptr(fwd_indices), n, fwd_indices.numel(),
+                                                      _ptr(indptr), _ptr(cursor), _ptr(out), _stream()))
+    return out
+
+
+def synth_random_access(mode, table, num_accesses, salt, sink):
+    """One random 4-byte access per work item into `table` (apt_synth_random_access)."""
+    bench_check(bench_lib().apt_synth_random_access(int(mode), _ptr(table), table.numel() * table.element_size(),
+                                                    int(num_accesses), int(salt), _ptr(sink), _stream()))
 
 
 def rank_table(num_total_nodes, device):
@@ -469,7 +513,7 @@ def synth_copy(src, dst):
     nbytes = src.numel() * src.element_size()
     if dst.numel() * dst.element_size() != nbytes:
         raise AptError("synth_copy: size mismatch")
-    check(lib().apt_synth_copy(_ptr(src), _ptr(dst), nbytes, _stream()))
+    bench_check(bench_lib().apt_synth_copy(_ptr(src), _ptr(dst), nbytes, _stream()))
     return dst
 
 

@@ -217,14 +217,16 @@ int tuning_gather_store_policy();
 int tuning_gather_wt_tail_mib();  // 0 = kWriteThroughTailMiB
 
 // How many workgroups of a kernel the GPU holds at once (asked once per kernel; 2048 for the plain gather of
-// 16-byte vectors: 8 on each of 256 CUs).
-template <typename Kernel>
-static int64_t resident_blocks(Kernel kernel) {
-  static const int64_t blocks = [kernel] {
+// 16-byte vectors: 8 on each of 256 CUs).  The kernel is a template argument, not a function argument: all
+// gather kernels have the same function type, and a cache per type would give every variant the figure of
+// whichever was launched first.
+template <auto Kernel>
+static int64_t resident_blocks() {
+  static const int64_t blocks = [] {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kGatherBlock, 0) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, Kernel, kGatherBlock, 0) != hipSuccess ||
         cus <= 0 || per_cu <= 0) {
       (void)hipGetLastError();
       return static_cast<int64_t>(kGatherResidentBlocks);
@@ -260,10 +262,10 @@ static int gather_rows_in_flight() {
 template <int V, int LPR>
 static int launch_gather_r(const GatherParams& p, hipStream_t st) {
   const int R = gather_rows_in_flight();
-  const int64_t resident = R == 1   ? resident_blocks(gather_kernel<V, LPR, 1>)
-                           : R == 2 ? resident_blocks(gather_kernel<V, LPR, 2>)
-                           : R == 8 ? resident_blocks(gather_kernel<V, LPR, 8>)
-                                    : resident_blocks(gather_kernel<V, LPR, 4>);
+  const int64_t resident = R == 1   ? resident_blocks<gather_kernel<V, LPR, 1>>()
+                           : R == 2 ? resident_blocks<gather_kernel<V, LPR, 2>>()
+                           : R == 8 ? resident_blocks<gather_kernel<V, LPR, 8>>()
+                                    : resident_blocks<gather_kernel<V, LPR, 4>>();
   const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, R, resident))), block(kGatherBlock);
   // One-shot measurement hook: the launch itself records the two events
   // (kernel begin / kernel end), see apt_time_next_gather.
@@ -324,7 +326,7 @@ static int launch_gather(const GatherParams& p, int elem_size, hipStream_t st) {
 template <int LPR>
 static void launch_gather_with_lookup_r(GatherParams& p, const PendingLookup& lookup, hipStream_t st) {
   p.lookup_blocks = static_cast<int>(lookup.blocks);
-  const int64_t resident = resident_blocks(gather_with_lookup_kernel<LPR>);
+  const int64_t resident = resident_blocks<gather_with_lookup_kernel<LPR>>();
   const dim3 grid(static_cast<unsigned>(gather_blocks(p, kGatherBlock / LPR, 2, resident) + p.lookup_blocks)),
       block(kGatherBlock);
   hipEvent_t ev0 = t_gather_start, ev1 = t_gather_stop;

@@ -1,9 +1,17 @@
-// R-MAT neighbour-list generator (benchmark / test input, not on the
-// reference's path).  See include/apt_synth.h.
+// libapt_bench.so: synthetic inputs and measurement helpers for the benchmark
+// and the tests (R-MAT generator, symmetrisation, a plain copy kernel and a
+// random-access probe).  Nothing here is on the reference's path and nothing of
+// it is linked into libapt_hip.so.  See include/apt_synth.h.
 #include "common.hpp"
 #include "../../include/apt_synth.h"
 
 namespace apt {
+
+// This library keeps its own error text (libapt_hip.so is not loaded with it).
+char* last_error_buf() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
 
 constexpr int kSynBlock = 256;
 constexpr int kSynEdgesPerBlock = 4096;
@@ -70,6 +78,42 @@ __global__ __launch_bounds__(kSynBlock) void rmat_fill_kernel(
     if (v >= num_nodes) v %= num_nodes;
     indices[e] = v;
   }
+}
+
+// Rows of the symmetrised graph before sorting: row u = [u (self-loop), the forward
+// neighbours of u, every w with a forward edge w -> u].  A workgroup owns 4096
+// consecutive forward edges; the reverse copy of an edge takes the next free slot
+// of its target's row (a ticket per row, so the order inside that part of a row
+// depends on scheduling; the caller sorts the rows afterwards).
+__global__ __launch_bounds__(kSynBlock) void symmetrize_fill_kernel(
+    const int64_t* __restrict__ fwd_indptr, const int64_t* __restrict__ fwd_indices, int64_t num_nodes,
+    int64_t num_fwd_edges, const int64_t* __restrict__ indptr, uint32_t* __restrict__ cursor,
+    int64_t* __restrict__ out) {
+  __shared__ int64_t s_lo, s_hi;
+  const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kSynEdgesPerBlock;
+  if (e0 >= num_fwd_edges) return;
+  const int64_t e1 = min(e0 + kSynEdgesPerBlock, num_fwd_edges) - 1;
+  if (threadIdx.x == 0) s_lo = row_of_edge(fwd_indptr, 0, num_nodes - 1, e0);
+  if (threadIdx.x == 1) s_hi = row_of_edge(fwd_indptr, 0, num_nodes - 1, e1);
+  __syncthreads();
+  const int64_t lo = s_lo, hi = s_hi;
+  for (int64_t e = e0 + threadIdx.x; e <= e1; e += kSynBlock) {
+    const int64_t u = row_of_edge(fwd_indptr, lo, hi, e);
+    const int64_t v = fwd_indices[e];
+    out[indptr[u] + 1 + (e - fwd_indptr[u])] = v;
+    if (v < 0 || v >= num_nodes) continue;  // the generator never produces one
+    const int64_t out_deg_v = fwd_indptr[v + 1] - fwd_indptr[v];
+    const uint32_t ticket = atomicAdd(&cursor[v], 1u);
+    const int64_t pos = indptr[v] + 1 + out_deg_v + ticket;
+    if (pos < indptr[v + 1]) out[pos] = u;  // always, when indptr was sized from the same edges
+  }
+}
+
+__global__ __launch_bounds__(kSynBlock) void self_loop_kernel(const int64_t* __restrict__ indptr,
+                                                              int64_t num_nodes, int64_t* __restrict__ out) {
+  for (int64_t u = static_cast<int64_t>(blockIdx.x) * kSynBlock + threadIdx.x; u < num_nodes;
+       u += static_cast<int64_t>(gridDim.x) * kSynBlock)
+    out[indptr[u]] = u;
 }
 
 // Plain streaming copy in 16-byte vectors: the known-size reference for
@@ -149,88 +193,6 @@ extern "C" int apt_synth_random_access(int mode, void* table, int64_t table_byte
   return APT_OK;
 }
 
-namespace apt {
-
-// Grid-wide barrier between co-resident workgroups, for measuring what one costs
-// (the alternative to ending a kernel and launching the next).  The spin is
-// bounded: a workgroup that waits too long reports it and leaves, and so does
-// every other one at its next barrier, so the kernel always ends.
-__device__ __forceinline__ bool probe_grid_barrier(unsigned* count, unsigned* gen, unsigned groups, unsigned* fail) {
-  __shared__ int ok;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    ok = 1;
-    const unsigned g = __hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
-    if (atomicAdd(count, 1u) == groups - 1) {
-      __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __threadfence();
-      atomicAdd(gen, 1u);
-    } else {
-      unsigned spins = 0;
-      while (__hip_atomic_load(gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == g) {
-        __builtin_amdgcn_s_sleep(2);
-        if (++spins > (1u << 20) || __hip_atomic_load(fail, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
-          ok = 0;
-          atomicAdd(fail, 1u);
-          break;
-        }
-      }
-    }
-    __threadfence();
-  }
-  __syncthreads();
-  return ok != 0;
-}
-
-// state: [0] arrivals, [64] generation, [128] failures (words; a line each).  Every phase a thread writes one
-// word that a thread of another workgroup reads after the barrier, so the barrier's fences carry data.
-__global__ __launch_bounds__(kSynBlock) void grid_barrier_probe_kernel(unsigned* state, uint32_t* buf, int phases) {
-  const unsigned groups = gridDim.x;
-  uint32_t acc = 0;
-  for (int p = 0; p < phases; ++p) {
-    buf[static_cast<size_t>(blockIdx.x) * kSynBlock + threadIdx.x] = acc + p;
-    if (!probe_grid_barrier(state, state + 64, groups, state + 128)) return;
-    const unsigned other = (blockIdx.x + 1 + p) % groups;
-    acc += __builtin_nontemporal_load(&buf[static_cast<size_t>(other) * kSynBlock + threadIdx.x]);
-  }
-  if (acc == 0x12345679u) buf[0] = acc;
-}
-
-__global__ void empty_probe_kernel(uint32_t* buf) {
-  if (buf == nullptr) buf[0] = 1;
-}
-
-}  // namespace apt
-
-extern "C" int apt_synth_grid_barrier(int num_groups, int phases, void* state, void* buf, void* stream) {
-  using namespace apt;
-  APT_REQUIRE(num_groups >= 1 && phases >= 0 && state != nullptr && buf != nullptr, APT_EINVAL,
-              "apt_synth_grid_barrier: bad arguments");
-  int dev = 0, cus = 0, per_cu = 0;
-  APT_HIP(hipGetDevice(&dev));
-  APT_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  APT_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, grid_barrier_probe_kernel, kSynBlock, 0));
-  // every workgroup must be resident at once, with room to spare for whatever else runs
-  APT_REQUIRE(static_cast<int64_t>(num_groups) * 2 <= static_cast<int64_t>(cus) * per_cu, APT_ELIMIT,
-              "apt_synth_grid_barrier: %d workgroups cannot be resident together on %d CUs", num_groups, cus);
-  hipLaunchKernelGGL(grid_barrier_probe_kernel, dim3(static_cast<unsigned>(num_groups)), dim3(kSynBlock), 0,
-                     static_cast<hipStream_t>(stream), static_cast<unsigned*>(state), static_cast<uint32_t*>(buf), phases);
-  APT_LAUNCH_CHECK("grid_barrier_probe_kernel");
-  return APT_OK;
-}
-
-extern "C" int apt_synth_empty_launches(int count, void* buf, void* stream) {
-  using namespace apt;
-  APT_REQUIRE(count >= 0 && buf != nullptr, APT_EINVAL, "apt_synth_empty_launches: bad arguments");
-  for (int i = 0; i < count; ++i) {
-    hipLaunchKernelGGL(empty_probe_kernel, dim3(64), dim3(kSynBlock), 0, static_cast<hipStream_t>(stream),
-                       static_cast<uint32_t*>(buf));
-    APT_LAUNCH_CHECK("empty_probe_kernel");
-  }
-  return APT_OK;
-}
-
 extern "C" int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream) {
   using namespace apt;
   APT_REQUIRE(bytes >= 0 && bytes % 16 == 0, APT_EINVAL, "apt_synth_copy: bytes must be a multiple of 16");
@@ -267,3 +229,26 @@ extern "C" int apt_synth_rmat_fill(const int64_t* indptr, int64_t num_rows, int6
   APT_LAUNCH_CHECK("rmat_fill_kernel");
   return APT_OK;
 }
+
+extern "C" int apt_synth_symmetrize_fill(const int64_t* fwd_indptr, const int64_t* fwd_indices, int64_t num_nodes,
+                                         int64_t num_fwd_edges, const int64_t* indptr, void* cursor,
+                                         int64_t* out, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_nodes > 0 && num_fwd_edges >= 0, APT_EINVAL, "apt_synth_symmetrize_fill: bad sizes");
+  APT_REQUIRE(fwd_indptr != nullptr && indptr != nullptr && cursor != nullptr && out != nullptr &&
+                  (fwd_indices != nullptr || num_fwd_edges == 0),
+              APT_EINVAL, "apt_synth_symmetrize_fill: a pointer is NULL");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const unsigned row_blocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_nodes, kSynBlock), 16384));
+  hipLaunchKernelGGL(self_loop_kernel, dim3(row_blocks), dim3(kSynBlock), 0, st, indptr, num_nodes, out);
+  APT_LAUNCH_CHECK("self_loop_kernel");
+  if (num_fwd_edges == 0) return APT_OK;
+  const int64_t blocks = ceil_div(num_fwd_edges, kSynEdgesPerBlock);
+  APT_REQUIRE(blocks <= 0x7fffffffLL, APT_ELIMIT, "apt_synth_symmetrize_fill: too many edges");
+  hipLaunchKernelGGL(symmetrize_fill_kernel, dim3(static_cast<unsigned>(blocks)), dim3(kSynBlock), 0, st, fwd_indptr,
+                     fwd_indices, num_nodes, num_fwd_edges, indptr, static_cast<uint32_t*>(cursor), out);
+  APT_LAUNCH_CHECK("symmetrize_fill_kernel");
+  return APT_OK;
+}
+
+extern "C" const char* apt_synth_last_error(void) { return apt::last_error_buf(); }

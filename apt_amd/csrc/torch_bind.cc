@@ -45,15 +45,16 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   Tensor rank_table, mb_workspace;
   int64_t mb_batch = -1;
   std::vector<int64_t> mb_fanouts;
-  // sample_blocks' output buffers (upper-bound sized), handed out in turn: what call k returned stays
-  // untouched until call k + ring; ring 0 = fresh tensors on every call
+  // sample_blocks' output buffers (upper-bound sized).  Ring 0 (the default) = fresh tensors on every call,
+  // as the reference's operators return them; set_block_buffer_ring(n) hands out n registry-owned sets in
+  // turn instead: what call k returned is then overwritten by call k + n
   struct BlockBuffers {
     Tensor nodes, sizes, format_ws;
     std::vector<Tensor> nb, rl, ct, row, col, csc;
     bool formats = false;
   };
   std::vector<BlockBuffers> mb_ring;
-  int64_t mb_ring_size = 2, mb_ring_pos = 0;
+  int64_t mb_ring_size = 0, mb_ring_pos = 0;
 };
 
 State& S() {
@@ -102,7 +103,11 @@ void SetRngSeed(IdType seed) {
 
 void SetStrict(bool strict) { S().strict = strict; }
 
-// How many sets of output buffers sample_blocks hands out in turn (0 = fresh tensors on every call).
+// How many registry-owned sets of output buffers sample_blocks hands out in turn.  0 (the default) = fresh
+// tensors on every call.  With n > 0 a call costs less (no allocation), but what call k returned is
+// overwritten by call k + n whatever stream or consumer still holds it.
+IdType BlockBufferRing() { return S().mb_ring_size; }
+
 void SetBlockBufferRing(IdType sets) {
   TORCH_CHECK(sets >= 0 && sets <= 64, "npc: set_block_buffer_ring: 0..64 sets");
   S().mb_ring_size = sets;
@@ -743,7 +748,8 @@ TORCH_LIBRARY(npc, m) {
       .def("set_topology", &SetTopology)
       .def("set_rng_seed", &SetRngSeed)
       .def("set_strict", &SetStrict)
-      .def("set_block_buffer_ring", &SetBlockBufferRing);
+      .def("set_block_buffer_ring", &SetBlockBufferRing)
+      .def("block_buffer_ring", &BlockBufferRing);
 }
 
 }  // namespace npc

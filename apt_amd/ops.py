@@ -65,9 +65,14 @@ def set_strict(strict: bool) -> None:
 
 
 def set_block_buffer_ring(sets: int) -> None:
-    """sample_blocks hands out `sets` sets of output buffers in turn (default 2): the tensors of call k
-    are overwritten by call k + sets.  0 = fresh tensors on every call."""
+    """0 (default): sample_blocks returns fresh tensors on every call, as the reference's operators do.
+    n > 0: it hands out n registry-owned sets of output buffers in turn, which saves the allocations, but
+    the tensors of call k are overwritten by call k + n, whoever still holds them."""
     _npc.set_block_buffer_ring(int(sets))
+
+
+def block_buffer_ring() -> int:
+    return int(_npc.block_buffer_ring())
 
 
 # ---------------------------------------------------------------- hot path

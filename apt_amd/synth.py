@@ -140,6 +140,81 @@ def rmat_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B
     return indptr, indices
 
 
+def symmetrize_csr_numpy(indptr, indices):
+    """Small graphs on the CPU: the simple, bidirected graph with a self-loop on every node that the
+    reference trains on (scripts/load_data.py:13-17: remove_self_loop, add_self_loop, to_bidirected).
+    -> (indptr, indices) with sorted rows."""
+    n = len(indptr) - 1
+    row = np.repeat(np.arange(n, dtype=np.int64), np.diff(indptr))
+    col = np.asarray(indices, dtype=np.int64)
+    loops = np.arange(n, dtype=np.int64)
+    key = np.unique(np.concatenate([row * n + col, col * n + row, loops * n + loops]))
+    return csr_from_edges(n, key // n, key % n)
+
+
+def rmat_symmetric_csr_gpu(num_nodes, num_edges, seed, device="cuda:0", a=RMAT_A, b=RMAT_B, c=RMAT_C,
+                           chunk_edges=1 << 27, stats=None):
+    """Large R-MAT graph of the kind the reference trains on (scripts/load_data.py:13-17): simple,
+    bidirected, a self-loop on every node, built on the GPU.
+
+    num_edges // 2 forward edges are drawn as rmat_csr_gpu draws them; every edge is stored in both
+    directions (in-degrees counted with one atomic per edge, reverse copies placed by tickets), every
+    node gets a self-loop, then the rows are sorted and repeated entries merged, a range of rows at a
+    time (keys (row << bits) | neighbour, torch.sort).  The result does not depend on scheduling.
+    stats (dict, optional) receives forward_edges, entries_before_merge, merged_fraction.
+
+    -> (indptr int64[num_nodes + 1], indices int64[E'], rows sorted by id, no repeats)
+    """
+    import math
+
+    import torch
+
+    from . import capi
+
+    N = int(num_nodes)
+    fwd_indptr, fwd_indices = rmat_csr_gpu(N, num_edges // 2, seed, device, a, b, c)
+    in_deg = torch.zeros(N, dtype=torch.int64, device=device)
+    capi.count_ids(fwd_indices, in_deg)
+    indptr = torch.zeros(N + 1, dtype=torch.int64, device=device)
+    torch.cumsum(fwd_indptr[1:] - fwd_indptr[:-1] + in_deg + 1, 0, out=indptr[1:])
+    del in_deg
+    total = int(indptr[-1].item())
+    out = torch.empty(total, dtype=torch.int64, device=device)
+    capi.synth_symmetrize_fill(fwd_indptr, fwd_indices, indptr, out)
+    n_fwd = int(fwd_indices.numel())
+    del fwd_indptr, fwd_indices
+    # ranges of rows holding about chunk_edges entries each
+    marks = torch.arange(0, total, int(chunk_edges), dtype=torch.int64, device=device)
+    rows = torch.unique(torch.clamp(torch.searchsorted(indptr, marks, right=True) - 1, min=0))
+    rows = torch.cat([rows, torch.tensor([N], dtype=torch.int64, device=device)])
+    rows[0] = 0
+    rows_h = rows.cpu().tolist()
+    offs_h = indptr[rows].cpu().tolist()
+    bits = max(1, int(math.ceil(math.log2(max(N, 2)))))
+    mask = (1 << bits) - 1
+    new_deg = torch.empty(N, dtype=torch.int64, device=device)
+    w = 0
+    for (r0, r1), (e0, e1) in zip(zip(rows_h[:-1], rows_h[1:]), zip(offs_h[:-1], offs_h[1:])):
+        if r1 == r0:
+            continue
+        local = torch.repeat_interleave(torch.arange(r1 - r0, dtype=torch.int64, device=device),
+                                        indptr[r0 + 1:r1 + 1] - indptr[r0:r1], output_size=e1 - e0)
+        key = torch.sort((local << bits) | out[e0:e1]).values
+        del local
+        keep = torch.ones(e1 - e0, dtype=torch.bool, device=device)
+        keep[1:] = key[1:] != key[:-1]
+        key = key[keep]
+        del keep
+        new_deg[r0:r1] = torch.bincount(key >> bits, minlength=r1 - r0)
+        out[w:w + key.numel()] = key & mask            # w <= e0: only entries already read are overwritten
+        w += int(key.numel())
+        del key
+    torch.cumsum(new_deg, 0, out=indptr[1:])
+    if stats is not None:
+        stats.update(forward_edges=n_fwd, entries_before_merge=total, merged_fraction=1.0 - w / max(total, 1))
+    return indptr, out[:w]
+
+
 def random_features(num_rows, dim, dtype, seed, device="cuda:0"):
     """~N(0,1) feature table generated on the GPU in chunks."""
     import torch
@@ -154,20 +229,31 @@ def random_features(num_rows, dim, dtype, seed, device="cuda:0"):
     return out
 
 
-def partition_share(num_nodes, num_edges, parts, part, dim, dtype, cache_ratio, seed, device="cuda:0"):
+def partition_share(num_nodes, num_edges, parts, part, dim, dtype, cache_ratio, seed, device="cuda:0",
+                    full_graph=None):
     """One GPU's share of a graph split into `parts` contiguous id ranges (the reference's partitioned
     layout: python/npc/utils/utils.py load_partition, src/cache_feats.cc:14-61, src/core.cc:102-125):
     the CSR rows of range `part` (neighbour ids stay global), the feature rows of that range, a cache
     of the `cache_ratio` hottest remote rows (largest expected degree; ties by id), the position map
     over all ids (-(i)-2 local row i, >= 0 cache row, -1 absent), the range bounds `min_vids` and the
     owner -> request-bucket map (bucket 0 = this GPU, the other owners 1.. in id order).
+    full_graph: (indptr, indices) of the whole graph on the device; the share is then its rows [lo, hi)
+    and the cache holds the remote rows of largest actual degree.  Without it the share's rows of the
+    directed multigraph generator are drawn and the cache goes by expected degree.
     -> dict(lo, hi, indptr, indices, feats, cache, hot, pos_map, min_vids, remote_worker_map)"""
     import torch
 
     lo, hi = num_nodes * part // parts, num_nodes * (part + 1) // parts
-    indptr, indices = rmat_csr_gpu(num_nodes, num_edges, seed, device, row_begin=lo, num_rows=hi - lo)
+    if full_graph is not None:
+        g_indptr, g_indices = full_graph
+        e0, e1 = int(g_indptr[lo].item()), int(g_indptr[hi].item())
+        indptr = (g_indptr[lo:hi + 1] - e0).contiguous()
+        indices = g_indices[e0:e1].clone()
+        exp_deg = (g_indptr[1:] - g_indptr[:-1]).to(torch.float32)
+    else:
+        indptr, indices = rmat_csr_gpu(num_nodes, num_edges, seed, device, row_begin=lo, num_rows=hi - lo)
+        exp_deg = rmat_expected_degree(num_nodes, num_edges, device)
     feats = random_features(hi - lo, dim, dtype, seed + 1, device)
-    exp_deg = rmat_expected_degree(num_nodes, num_edges, device)
     exp_deg[lo:hi] = -1.0
     n_cache = int((num_nodes - (hi - lo)) * cache_ratio)
     hot = torch.sort(exp_deg, descending=True, stable=True).indices[:n_cache].contiguous()

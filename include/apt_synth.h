@@ -1,7 +1,10 @@
 /*
- * apt_synth.h — synthetic-input helpers of libapt_hip.so (benchmark and test
- * support; no counterpart in the reference, which loads OGB datasets through
- * DGL, scripts/preprocess_dataset.py).
+ * apt_synth.h — libapt_bench.so: synthetic inputs and measurement helpers for
+ * the benchmark and the tests.  A library of its own, not part of the product
+ * ABI (libapt_hip.so, apt_amd.h); no counterpart in the reference, which loads
+ * OGB datasets through DGL (scripts/preprocess_dataset.py, scripts/load_data.py).
+ * Every function returns 0 or an error code whose text apt_synth_last_error()
+ * gives.
  */
 #ifndef APT_SYNTH_H_
 #define APT_SYNTH_H_
@@ -44,20 +47,22 @@ int apt_synth_copy(const void* src, void* dst, int64_t bytes, void* stream);
 int apt_synth_random_access(int mode, void* table, int64_t table_bytes, int64_t num_accesses,
                             uint32_t salt, void* sink, void* stream);
 
-/* What a step between two dependent phases costs, two ways.
- * apt_synth_grid_barrier: one kernel of num_groups workgroups (256 threads) that
- *   run `phases` phases separated by a grid-wide barrier (arrival counter and
- *   generation word in device memory); in every phase a thread writes a word
- *   that another workgroup reads after the barrier.  The spin is bounded: if a
- *   workgroup gives up, state[128] counts it and the kernel ends.
- *   state  device uint32[192], all zero before the first call (arrivals at word
- *          0, generation at 64, failures at 128)
- *   buf    device uint32[num_groups * 256]
- *   num_groups is limited to half of what can be resident at once.
- * apt_synth_empty_launches: `count` launches of an empty kernel, each dependent
- *   on the one before by stream order. */
-int apt_synth_grid_barrier(int num_groups, int phases, void* state, void* buf, void* stream);
-int apt_synth_empty_launches(int count, void* buf, void* stream);
+/* Turns a forward CSR (fwd_indptr int64[num_nodes + 1], fwd_indices) into the rows
+ * of its symmetrised form with a self-loop per node, unsorted and with repeats:
+ * row u = [u, the forward neighbours of u, every w with a forward edge w -> u]
+ * (what dgl.add_self_loop + dgl.to_bidirected give before parallel edges are
+ * merged; reference scripts/load_data.py:13-17).  The caller sizes the rows:
+ *   indptr   device int64[num_nodes + 1], row u holding 1 + out-degree + in-degree
+ *   cursor   device uint32[num_nodes], all zero (tickets of the reverse copies)
+ *   out      device int64[indptr[num_nodes]]
+ * The order of the reverse copies inside a row depends on scheduling; sort the
+ * rows (and drop repeats) afterwards. */
+int apt_synth_symmetrize_fill(const int64_t* fwd_indptr, const int64_t* fwd_indices, int64_t num_nodes,
+                              int64_t num_fwd_edges, const int64_t* indptr, void* cursor, int64_t* out,
+                              void* stream);
+
+/* Text of the last error of this library on the calling thread. */
+const char* apt_synth_last_error(void);
 
 #ifdef __cplusplus
 }

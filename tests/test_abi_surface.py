@@ -10,24 +10,36 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_functions():
-    names = []
-    for hdr in ("apt_amd.h", "apt_synth.h"):
-        text = open(os.path.join(ROOT, "include", hdr)).read()
-        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names += re.findall(r"\b(apt_[a-z0-9_]+)\s*\(", text)
-    return sorted(set(names))
+def _declared_functions(hdr):
+    text = open(os.path.join(ROOT, "include", hdr)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(apt_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_symbols_are_exported_and_bound():
     from apt_amd import capi
-    lib = ctypes.CDLL(capi.LIB_PATH)
-    declared = _declared_functions()
-    assert len(declared) >= 15
-    for name in declared:
-        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
-        assert name in capi.SYMBOLS, f"{name} has no ctypes prototype in capi.SYMBOLS"
+    for hdr, path, table, least in (("apt_amd.h", capi.LIB_PATH, capi.SYMBOLS, 15),
+                                    ("apt_synth.h", capi.BENCH_LIB_PATH, capi.BENCH_SYMBOLS, 4)):
+        lib = ctypes.CDLL(path)
+        declared = _declared_functions(hdr)
+        assert len(declared) >= least
+        for name in declared:
+            assert hasattr(lib, name), f"{name} declared in include/{hdr} but not exported by {path}"
+            assert name in table, f"{name} has no ctypes prototype in capi"
+        assert sorted(table) == declared, f"capi binds symbols that include/{hdr} does not declare"
     assert capi.lib().apt_abi_version() == 1
+    capi.bench_lib()
+
+
+def test_product_library_exports_the_product_abi_only():
+    """Benchmark inputs and probes live in libapt_bench.so: the product library exports what
+    include/apt_amd.h declares and nothing named apt_synth_*."""
+    import subprocess
+
+    from apt_amd import capi
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line and line.split()[-1].startswith("apt_")}
+    assert exported == set(_declared_functions("apt_amd.h")), exported ^ set(_declared_functions("apt_amd.h"))
 
 
 def test_argument_checks_need_no_gpu():
@@ -131,3 +143,18 @@ def test_peer_operators_raise():
         torch.ops.npc.np_sample_and_shuffle(torch.arange(4), 3)
     with pytest.raises(RuntimeError, match="other GPUs"):
         torch.ops.npc.nccl_get_unique_id()
+
+
+def test_sample_blocks_returns_fresh_tensors_by_default():
+    """The registry-owned output ring of sample_blocks is opt-in: by default the operator allocates its
+    outputs on every call, like the reference's operators (a result is never overwritten by a later call)."""
+    import torch
+
+    import apt_amd
+    assert torch.ops.npc.block_buffer_ring() == 0
+    apt_amd.ops.set_block_buffer_ring(3)
+    assert apt_amd.ops.block_buffer_ring() == 3
+    apt_amd.ops.set_block_buffer_ring(0)
+    assert torch.ops.npc.block_buffer_ring() == 0
+    with pytest.raises(RuntimeError, match="0..64"):
+        apt_amd.ops.set_block_buffer_ring(-1)

@@ -33,5 +33,5 @@ def test_build_from_sources_only(tmp_path):
     r = subprocess.run([sys.executable, "-c", code], cwd=tree, env=env, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-4000:]
     assert "built" in r.stdout
-    for so in ("apt_amd/libapt_hip.so", "apt_amd/libnpc.so", "oracle/liborc.so"):
+    for so in ("apt_amd/libapt_hip.so", "apt_amd/libapt_bench.so", "apt_amd/libnpc.so", "oracle/liborc.so"):
         assert (tree / so).exists(), so

@@ -2,12 +2,15 @@
 
 medium (2.4 M nodes / 62 M edges): the graph is copied to the host and the
 whole batch is compared with the oracle, bit for bit.
-full (111 M nodes / 3.2 B edges, 128 x bf16): too big to hand to the CPU oracle
-in a test, so the batch is checked through properties that do not depend on
-size: counts = min(fanout, degree), sampled ids are true neighbours, the node
-list has no duplicates and starts with the seeds, nodes[relabeled] gives the
-sampled ids back, the gathered rows equal torch's own index_select, and the
-same rng key reproduces the batch.
+full (111 M nodes, 1.6 B R-MAT edges stored in both directions plus a self-loop
+per node, 128 x bf16): the graph (27 GB) is copied to the host once and whole
+batches of 4096 seeds are compared with the oracle bit for bit, with and
+without replacement; the gathered rows are compared with torch's own
+index_select of the same ids (the 28 GB feature table stays on the GPU).  The
+properties that hold at any size are checked as well: counts = min(fanout,
+degree), sampled ids are true neighbours, the node list has no duplicates and
+starts with the seeds, nodes[relabeled] gives the sampled ids back, and the same
+rng key reproduces the batch.
 """
 import numpy as np
 import pytest
@@ -91,7 +94,7 @@ def test_medium_scale_vs_oracle(orc, capi):
     from apt_amd import synth
     from apt_amd.pipeline import MiniBatchPipeline
     N, E, D = 2_449_029, 62_000_000, 100
-    indptr, indices = synth.rmat_csr_gpu(N, E, 1, DEV)
+    indptr, indices = synth.rmat_symmetric_csr_gpu(N, E, 1, DEV)
     feats = synth.random_features(N, D, torch.float32, 2, DEV)
     graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
     hops = [5, 10, 15]
@@ -115,14 +118,108 @@ def test_medium_scale_vs_oracle(orc, capi):
     orc.set_threads(1)
 
 
-@pytest.mark.parametrize("replace", [False, True])
-def test_full_scale_properties(capi, replace):
+FULL_N, FULL_E, FULL_D = 111_059_956, 3_200_000_000, 128
+
+
+@pytest.fixture(scope="module")
+def full(capi):
+    """The full-scale graph and feature table, built once for this module and freed after it."""
     from apt_amd import synth
+    stats = {}
+    indptr, indices = synth.rmat_symmetric_csr_gpu(FULL_N, FULL_E, 1, DEV, stats=stats)
+    feats = synth.random_features(FULL_N, FULL_D, torch.bfloat16, 2, DEV)
+    box = dict(indptr=indptr, indices=indices, feats=feats, stats=stats)
+    yield box
+    box.clear()
+    del indptr, indices, feats
+    torch.cuda.empty_cache()
+
+
+def test_full_scale_graph_is_simple_symmetric_with_self_loops(full):
+    """What the generator promises (the kind of graph the reference trains on, scripts/load_data.py:13-17),
+    checked at full size with size-independent properties and on sampled rows."""
+    indptr, indices, st = full["indptr"], full["indices"], full["stats"]
+    N = FULL_N
+    assert indptr.numel() == N + 1 and int(indptr[0]) == 0 and int(indptr[-1]) == indices.numel()
+    assert st["forward_edges"] > 1_550_000_000 and st["entries_before_merge"] == 2 * st["forward_edges"] + N
+    assert indices.numel() > 2_800_000_000                           # what is left after merging repeats
+    deg = indptr[1:] - indptr[:-1]
+    assert int(deg.min()) >= 1                                       # every node has at least its self-loop
+    assert int(indices.min()) >= 0 and int(indices.max()) < N
+    # rows strictly increasing (sorted, no repeats): a decrease is only allowed where a new row starts
+    step = 1 << 28
+    row_start = torch.zeros(indices.numel(), dtype=torch.bool, device=DEV)
+    row_start[indptr[:-1]] = True
+    for s in range(0, indices.numel() - 1, step):
+        e = min(s + step, indices.numel() - 1)
+        assert bool(((indices[s + 1:e + 1] > indices[s:e]) | row_start[s + 1:e + 1]).all())
+    del row_start
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(1)
+    rows = torch.cat([torch.randint(0, N, (300,), generator=gen, device=DEV), torch.topk(deg, 3).indices]).tolist()
+    for u in rows:
+        row = indices[int(indptr[u]):int(indptr[u + 1])]
+        assert bool((row == u).any())                                # the self-loop
+        for v in row[torch.randperm(row.numel(), device=DEV)[:20]].tolist():   # symmetry: u in row v
+            rv = indices[int(indptr[v]):int(indptr[v + 1])]
+            k = int(torch.searchsorted(rv, torch.tensor(u, device=DEV)))
+            assert k < rv.numel() and int(rv[k]) == u
+    # every entry (u, v) has its mirror image (v, u): then the sum of u * v^2 over all entries equals the sum
+    # of v * u^2 (64-bit wrap-around, an odd multiplier mixed in); over the entries with both ends among the
+    # first million nodes, which hold the hubs
+    M = 1 << 20
+    src = torch.repeat_interleave(torch.arange(M, device=DEV), deg[:M])
+    sub = indices[:src.numel()]
+    inside = sub < M
+    a, b = src[inside], sub[inside]
+    assert a.numel() > 10_000_000
+    h = 0x9E3779B97F4A7C15 - (1 << 64)
+    assert int((a * (b * b * h)).sum()) == int((b * (a * a * h)).sum())
+    assert int((a * (b * b * h)).sum()) != int(((a + 1) * (b * b * h)).sum())
+
+
+def test_full_scale_vs_oracle(orc, capi, full):
+    """Whole batches of 4096 seeds on the full-scale graph against the CPU oracle, bit for bit: the node list
+    and every hop's sampled ids, compact ids and counts, without and with replacement, fused driver and
+    per-hop driver; gathered rows against index_select."""
     from apt_amd.pipeline import MiniBatchPipeline
-    N, E, D = 111_059_956, 3_200_000_000, 128
-    indptr, indices = synth.rmat_csr_gpu(N, E, 1, DEV)
-    assert indices.numel() > 3_000_000_000 and int(indptr[-1]) == indices.numel()
-    feats = synth.random_features(N, D, torch.bfloat16, 2, DEV)
+    indptr, indices, feats = full["indptr"], full["indices"], full["feats"]
+    graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
+    og = orc.Graph(indptr.cpu().numpy(), indices.cpu().numpy())
+    orc.set_threads(16)
+    hops = [5, 10, 15]
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(11)
+    try:
+        for replace in (False, True):
+            pipes = [MiniBatchPipeline(graph, store, 4096, hops, replace=replace),
+                     MiniBatchPipeline(graph, None, 4096, hops, replace=replace, gather=False, fused=False)]
+            for batch in range(2):
+                seeds = torch.randperm(FULL_N, generator=gen, device=DEV)[:4096].contiguous()
+                key = 31337 + 10 * batch + int(replace)
+                want_in, want_blocks = orc.sample_blocks(og, seeds.cpu().numpy(), hops, replace, key)
+                assert sum(int(b["counts"].sum()) for b in want_blocks) > 500_000
+                for pipe in pipes[:1 if batch else 2]:
+                    pipe.run(seeds, key)
+                    res = pipe.result()
+                    assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
+                    for got, want in zip(res["blocks"], want_blocks):
+                        for k in ("neighbors", "relabeled", "counts"):
+                            assert np.array_equal(got[k].cpu().numpy(), want[k]), (k, replace, batch)
+                    if res["features"] is not None:
+                        ids = torch.from_numpy(want_in).to(DEV)
+                        assert torch.equal(res["features"].view(torch.int16), feats.index_select(0, ids).view(torch.int16))
+            del pipes
+    finally:
+        orc.set_threads(1)
+        del og
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_full_scale_properties(capi, full, replace):
+    from apt_amd.pipeline import MiniBatchPipeline
+    N = FULL_N
+    indptr, indices, feats = full["indptr"], full["indices"], full["feats"]
     graph, store = capi.Graph(indptr, indices), capi.FeatStore(feats)
     hops = [5, 10, 15]
     pipe = MiniBatchPipeline(graph, store, 4096, hops, replace=replace, formats=True)
@@ -187,7 +284,7 @@ def test_full_scale_properties(capi, replace):
             assert torch.equal(want["features"].view(torch.int16), feats_i), i
             assert torch.equal(want["blocks"][0]["relabeled"], rel_i), i
         del loader, kept
-    del pipe, feats, indices, indptr
+    del pipe
     torch.cuda.empty_cache()
 
 

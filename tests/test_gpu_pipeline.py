@@ -398,20 +398,25 @@ def test_operator_layer_fused_sampler(orc, capi):
     assert sizes[:2] == [50, len(want_in)] and np.array_equal(nodes.cpu().numpy(), want_in)
     assert np.array_equal(hops[0][0].cpu().numpy(), want_blocks[0]["neighbors"])
     assert np.array_equal(hops[0][2].cpu().numpy(), want_blocks[0]["counts"])
-    nodes, hops = nodes.clone(), [tuple(t.clone() for t in hops[0])]      # the ring below overwrites the originals
-    # output buffers come from a ring of two sets: a call's tensors stay untouched during the next call and
-    # are overwritten by the one after; with a ring of 0 every call gets fresh tensors
+    # by default every call returns fresh tensors, as the reference's operators do: three results in a row
+    # are three sets of buffers and a held result is never overwritten
+    assert npc.ops.block_buffer_ring() == 0
+    outs = [npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10 + k) for k in range(3)]
+    keep = (outs[0][1].clone(), outs[0][2][0][1].clone())
+    assert len({o[1].data_ptr() for o in outs}) == 3 and len({o[2][0][1].data_ptr() for o in outs}) == 3
+    again = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10)
+    assert torch.equal(outs[0][1], keep[0]) and torch.equal(outs[0][2][0][1], keep[1])   # untouched by later calls
+    assert torch.equal(again[1], keep[0]) and torch.equal(again[2][0][1], keep[1])       # same key, same batch
+    # opt-in: a ring of two registry-owned sets: a call's tensors stay untouched during the next call and are
+    # overwritten by the one after
+    npc.ops.set_block_buffer_ring(2)
+    assert npc.ops.block_buffer_ring() == 2
     s1, n1, h1 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10)
-    keep = (n1.clone(), h1[0][1].clone())
     s2, n2, h2 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 11)
     assert n2.data_ptr() != n1.data_ptr() and torch.equal(n1, keep[0]) and torch.equal(h1[0][1], keep[1])
     s3, n3, h3 = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 12)
     assert n3.data_ptr() == n1.data_ptr() and h3[0][1].data_ptr() == h1[0][1].data_ptr()
     npc.ops.set_block_buffer_ring(0)
-    outs = [npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 10 + k) for k in range(3)]
-    assert len({o[1].data_ptr() for o in outs}) == 3
-    assert torch.equal(outs[0][1], keep[0]) and torch.equal(outs[0][2][0][1], keep[1])   # same key, same batch
-    npc.ops.set_block_buffer_ring(2)
     # the same call with the blocks' COO + CSC emitted before its one wait
     sizes_f, nodes_f, hops_f, fmts = npc.ops.sample_blocks(dev(np.arange(50)), [4], False, 9, formats=True)
     assert sizes_f == sizes and torch.equal(nodes_f, nodes) and torch.equal(hops_f[0][1], hops[0][1])

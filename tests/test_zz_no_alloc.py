@@ -31,22 +31,45 @@ def test_static_relabel_matches_workspace_relabel(orc, capi):
     rng = np.random.default_rng(17)
     limit = capi.lib().apt_relabel_static_max_items()
     assert limit == 1 << 21
-    # two calls in a row, the second smaller (then a few more shapes, all sharing the one array)
-    for ns, nn, id_range in [(67_584, 1_013_760, 111_000_000), (1024, 5120, 3000), (0, 0, 10), (5, 0, 10),
-                             (6144, 61_440, 50_000), (1 << 20, 1 << 20, 1 << 40), (1, 3, 2)]:
-        seeds, nbr = _case(rng, ns, nn, id_range)
-        want_u, want_r, want_n = capi.relabel(seeds, nbr)
-        before = torch.cuda.memory_allocated()
-        uniq, rel, cnt = _static(capi, seeds, nbr)
-        n = int(cnt.item())
-        assert n == int(want_n)
-        assert torch.equal(uniq[:n], want_u[:n]) and torch.equal(rel, want_r)
-        assert bool((uniq[n:] == -7).all())                     # nothing written past the count
-        if ns + nn <= 200_000:                                  # and both against the oracle
-            ou, orl = orc.relabel(seeds.cpu().numpy(), nbr.cpu().numpy())
-            assert np.array_equal(uniq[:n].cpu().numpy(), ou) and np.array_equal(rel.cpu().numpy(), orl)
-        del uniq, rel, cnt
-        assert torch.cuda.memory_allocated() == before          # torch's allocator saw nothing new
+    # Two calls in a row, the second smaller (then a few more shapes, all sharing the one array).  Small inputs
+    # normally take the single-workgroup kernel with its table in LDS, which never touches the shared array:
+    # that path is switched off here, so that every call below runs its passes over the array and would show
+    # what an earlier, larger call left in it.
+    _static(capi, *_case(rng, 2000, 30_000, 1 << 30))           # first use resolves the array's address
+    torch.cuda.synchronize()
+    capi.set_tuning("relabel_lds", 0)
+    try:
+        for ns, nn, id_range in [(67_584, 1_013_760, 111_000_000), (1024, 5120, 3000), (0, 0, 10), (5, 0, 10),
+                                 (6144, 61_440, 50_000), (1 << 20, 1 << 20, 1 << 40), (1, 3, 2)]:
+            seeds, nbr = _case(rng, ns, nn, id_range)
+            want_u, want_r, want_n = capi.relabel(seeds, nbr)
+            uniq = torch.full((ns + nn,), -7, dtype=torch.int64, device=DEV)
+            rel = torch.full((nn,), -7, dtype=torch.int64, device=DEV)
+            cnt = torch.full((1,), -7, dtype=torch.int64, device=DEV)
+            torch.cuda.synchronize()
+            # free device memory as the driver reports it (hipMemGetInfo): sees a hipMalloc made behind
+            # torch's back, which torch.cuda.memory_allocated() would not
+            free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+            capi.check(capi.lib().apt_relabel_static(capi._ptr(seeds), ns, None, capi._ptr(nbr), nn, 0, capi._ptr(uniq),
+                                                     capi._ptr(rel), capi._ptr(cnt), capi._stream()))
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+            n = int(cnt.item())
+            assert n == int(want_n)
+            assert torch.equal(uniq[:n], want_u[:n]) and torch.equal(rel, want_r)
+            assert bool((uniq[n:] == -7).all())                     # nothing written past the count
+            if ns + nn <= 200_000:                                  # and both against the oracle
+                ou, orl = orc.relabel(seeds.cpu().numpy(), nbr.cpu().numpy())
+                assert np.array_equal(uniq[:n].cpu().numpy(), ou) and np.array_equal(rel.cpu().numpy(), orl)
+            del uniq, rel, cnt
+    finally:
+        capi.set_tuning("relabel_lds", 1)
+    # the LDS path (small inputs, default setting) gives the same answer and allocates nothing either
+    seeds, nbr = _case(rng, 1024, 5120, 3000)
+    want_u, want_r, want_n = capi.relabel(seeds, nbr)
+    uniq, rel, cnt = _static(capi, seeds, nbr)
+    n = int(cnt.item())
+    assert n == int(want_n) and torch.equal(uniq[:n], want_u[:n]) and torch.equal(rel, want_r)
     # device-side seed count (the frontier of a later hop): only the first n * stride neighbours count
     seeds, nbr = _case(rng, 4000, 4000 * 10, 20_000)
     ns_dev = torch.tensor([2500], dtype=torch.int64, device=DEV)
