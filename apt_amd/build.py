@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libapt_hip.so")
 NPC_LIB = os.path.join(HERE, "libnpc.so")
 BENCH_LIB = os.path.join(HERE, "libapt_bench.so")
-SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "minibatch.hip", "spmm.hip", "cache.hip", "block.hip"]
+SOURCES = ["lib.hip", "sample.hip", "relabel.hip", "gather.hip", "bucket.hip", "minibatch.hip", "spmm.hip", "cache.hip", "block.hip", "epoch.hip"]
 BENCH_SOURCES = ["synth.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

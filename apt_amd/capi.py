@@ -36,6 +36,32 @@ class CFeatStore(C.Structure):
                 ("out_dim", C.c_int64), ("elem_size", C.c_int)]
 
 
+MAX_HOPS, MAX_SLOTS = 8, 16
+
+
+class CBatchSlot(C.Structure):       # apt_batch_slot
+    _fields_ = [("stream", C.c_void_p), ("nodes", C.c_void_p),
+                ("neighbors", C.c_void_p * MAX_HOPS), ("relabeled", C.c_void_p * MAX_HOPS),
+                ("counts", C.c_void_p * MAX_HOPS), ("sizes", C.c_void_p), ("rank_table", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("features", C.c_void_p),
+                ("miss_count", C.c_void_p), ("request_sizes", C.c_void_p), ("request_offsets", C.c_void_p),
+                ("request_ids", C.c_void_p), ("request_perm", C.c_void_p), ("request_workspace", C.c_void_p),
+                ("request_workspace_bytes", C.c_size_t)]
+
+
+class CEpochDesc(C.Structure):       # apt_epoch_desc
+    _fields_ = [("graph", CGraph), ("store", CFeatStore), ("batch", C.c_int64), ("num_hops", C.c_int),
+                ("hop_fanouts", C.c_int * MAX_HOPS), ("replace", C.c_int), ("rank_table_len", C.c_int64),
+                ("has_requests", C.c_int), ("request_pos_map", C.c_void_p), ("request_num_total_nodes", C.c_int64),
+                ("remote_worker_map", C.c_void_p), ("min_vids", C.c_void_p), ("world_size", C.c_int),
+                ("num_remote_workers", C.c_int), ("num_slots", C.c_int), ("slots", CBatchSlot * MAX_SLOTS)]
+
+
+class CEpochCost(C.Structure):       # apt_epoch_cost
+    _fields_ = [("batches", C.c_int64), ("enqueue_seconds", C.c_double), ("wait_enqueue_seconds", C.c_double),
+                ("wait_gpu_seconds", C.c_double), ("release_seconds", C.c_double)]
+
+
 # every symbol include/apt_amd.h declares: name -> (restype, argtypes)
 _P, _I64, _I, _U64, _SZ = C.c_void_p, C.c_int64, C.c_int, C.c_uint64, C.c_size_t
 SYMBOLS = {
@@ -84,6 +110,13 @@ SYMBOLS = {
     "apt_gat_block_backward": (_I, [_P, _I64, _I, _P, _I64, _I, _I64, _I, _P, _P, C.c_float, _P, _P, _P, _P, _P, _P, _P]),
     "apt_spmm_heads": (_I, [_P, _P, _I64, _P, _I64, _P, _P, _I, _I64, _I, _I, _P, _I64, _P, _P, _P, _P]),
     "apt_time_next_sample": (_I, [_I, _P, _P]),
+    "apt_epoch_create": (_I, [C.POINTER(CEpochDesc), C.POINTER(_P)]),
+    "apt_epoch_begin": (_I, [_P, _P, _I64, _U64, _P]),
+    "apt_epoch_next": (_I, [_P, C.POINTER(_I), _P, _P]),
+    "apt_epoch_release": (_I, [_P, _P]),
+    "apt_epoch_end": (_I, [_P]),
+    "apt_epoch_destroy": (_I, [_P]),
+    "apt_epoch_host_cost": (_I, [_P, C.POINTER(CEpochCost)]),
 }
 
 # every symbol include/apt_synth.h declares (libapt_bench.so: inputs and probes of the benchmark and the tests)
@@ -506,6 +539,94 @@ class MinibatchPlan:
             self.pending.open = True
         else:
             check(lib().apt_minibatch_sample(*args))
+
+
+class EpochDriver:
+    """apt_epoch over the buffers of a list of MiniBatchPipeline objects (one slot each, fused driver, no
+    formats) and their streams.  The pipelines keep owning the buffers; this object must not outlive them."""
+
+    def __init__(self, pipes, streams):
+        p0 = pipes[0]
+        H = len(p0.fanouts)
+        if len(pipes) > MAX_SLOTS or H > MAX_HOPS:
+            raise AptError(f"epoch driver: at most {MAX_SLOTS} slots and {MAX_HOPS} hops")
+        d = CEpochDesc()
+        d.graph = p0.graph.c
+        if p0.feat is not None:
+            d.store = p0.feat.c
+        d.batch, d.num_hops, d.replace = p0.plan.batch, H, int(p0.replace)
+        for h, f in enumerate(p0.fanouts):
+            d.hop_fanouts[h] = f
+        d.rank_table_len = p0.plan.table_len
+        rq = p0.requests
+        if rq is not None:
+            d.has_requests = 1
+            d.request_pos_map = rq["feat_pos_map"].data_ptr()
+            d.request_num_total_nodes = rq["feat_pos_map"].numel()
+            d.remote_worker_map, d.min_vids = rq["remote_worker_map"].data_ptr(), rq["min_vids"].data_ptr()
+            d.world_size, d.num_remote_workers = int(rq["world_size"]), int(rq["num_remote_workers"])
+        d.num_slots = len(pipes)
+        for k, (p, st) in enumerate(zip(pipes, streams)):
+            s = d.slots[k]
+            s.stream = st.cuda_stream
+            s.nodes, s.sizes = p.plan.nodes.data_ptr(), p.plan.sizes.data_ptr()
+            for h in range(H):
+                s.neighbors[h], s.relabeled[h] = p.plan.neighbors[h].data_ptr(), p.plan.relabeled[h].data_ptr()
+                s.counts[h] = p.plan.counts[h].data_ptr() if p.plan.counts is not None else None
+            s.rank_table, s.workspace = p.plan.table.data_ptr(), p.plan.workspace.data_ptr()
+            s.workspace_bytes = p.plan.workspace.numel()
+            s.features = p.features.data_ptr() if p.features is not None else None
+            s.miss_count = p.misses.data_ptr()
+            if rq is not None:
+                s.request_sizes, s.request_offsets = p.request_sizes.data_ptr(), p.request_offsets.data_ptr()
+                s.request_ids, s.request_perm = p.request_ids.data_ptr(), p.request_perm.data_ptr()
+                s.request_workspace, s.request_workspace_bytes = p.request_ws.data_ptr(), p.request_ws.numel()
+        self._desc, self._keep = d, (pipes, streams)
+        self.num_hops = H
+        self.num_requests = d.num_remote_workers if rq is not None else 0
+        self.handle = C.c_void_p()
+        check(lib().apt_epoch_create(C.byref(d), C.byref(self.handle)))
+        self._slot = C.c_int()
+        self._sizes = (C.c_int64 * (H + 2))()
+        self._req = (C.c_int64 * max(self.num_requests, 1))()
+
+    def begin(self, seeds, num_batches, rng_seed0, ready_event=None):
+        seeds = _dev_i64(seeds, "seeds")
+        if seeds.numel() < num_batches * self._desc.batch:
+            raise AptError("epoch driver: fewer seeds than num_batches * batch")
+        self._seeds = seeds                                  # stays alive for the epoch
+        self._ready = ready_event
+        check(lib().apt_epoch_begin(self.handle, _ptr(seeds), int(num_batches), int(rng_seed0) & 0xFFFFFFFFFFFFFFFF,
+                                    C.c_void_p(ready_event.cuda_event) if ready_event is not None else None))
+
+    def next(self):
+        """Blocks until the next batch is complete -> (slot, sizes list, request sizes list or None)."""
+        check(lib().apt_epoch_next(self.handle, C.byref(self._slot), self._sizes,
+                                   self._req if self.num_requests else None))
+        return self._slot.value, list(self._sizes), (list(self._req)[:self.num_requests] if self.num_requests else None)
+
+    def release(self):
+        check(lib().apt_epoch_release(self.handle, _stream()))
+
+    def end(self):
+        check(lib().apt_epoch_end(self.handle))
+
+    def host_cost(self):
+        """-> dict(batches, enqueue_seconds, wait_enqueue_seconds, wait_gpu_seconds) since the driver was created."""
+        c = CEpochCost()
+        check(lib().apt_epoch_host_cost(self.handle, C.byref(c)))
+        return {k: getattr(c, k) for k, _ in CEpochCost._fields_}
+
+    def close(self):
+        if self.handle:
+            lib().apt_epoch_destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def synth_copy(src, dst):

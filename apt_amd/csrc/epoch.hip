@@ -1,0 +1,365 @@
+// Epoch driver: the host side of a trainer's data loader, in C.
+//
+// The reference's trainer iterates a dgl DataLoader whose sampler is
+// MixedPSNeighborSampler and then calls load_subtensor (examples/train.py:84-94,
+// 139; python/npc/utils/utils.py:425): per batch that is a Python loop over the
+// hops, two operator calls per hop, each with a stream synchronisation, and a
+// third for the features.  Here a batch is enqueued by a worker thread of this
+// library -- fused sampling + relabel, the gather (or, for a partitioned feature
+// store, the bucketing of the requests and the gather of the rows present here),
+// the copy of the batch's sizes to pinned host memory and the event that marks
+// it complete -- on one of a few "slots" (a set of device buffers and a HIP
+// stream each), so that several batches are in flight and the consumer's thread
+// does nothing per batch but wait for the next one and say when it is done with
+// it.  No device memory is allocated here: the slots' buffers come from the
+// caller.
+#include "common.hpp"
+
+#include <chrono>
+#include <condition_variable>
+#include <cstring>
+#include <deque>
+#include <mutex>
+#include <new>
+#include <thread>
+
+namespace apt {
+
+constexpr int kPinnedPerSlot = APT_MAX_HOPS + 2 + APT_MAX_BUCKETS;  // int64 words of pinned memory per slot
+
+// The batch's sizes (and request bucket sizes) go to pinned host memory by a one-workgroup kernel: a
+// hipMemcpyAsync of 40 bytes would put a copy-engine transfer and its two queue hand-overs between every batch
+// and the next one on the stream (25 us per batch at batch 1024).
+__global__ void publish_sizes_kernel(const int64_t* __restrict__ sizes, int n, const int64_t* __restrict__ req,
+                                     int r, int64_t* __restrict__ host_words) {
+  const int t = threadIdx.x;
+  if (t < n) host_words[t] = sizes[t];
+  if (t < r) host_words[APT_MAX_HOPS + 2 + t] = req[t];
+}
+
+struct EpochWork {
+  int64_t batch;
+  int slot;
+  hipEvent_t after;  // the slot's stream waits for it first (may be NULL)
+};
+
+}  // namespace apt
+
+struct apt_epoch {
+  apt_epoch_desc d;
+  int device = 0;
+  std::thread worker;
+  std::mutex mu;
+  std::condition_variable cv_work, cv_done;
+  std::deque<apt::EpochWork> queue;
+  bool stop = false;
+  bool busy = false;  // the worker is enqueueing a batch
+  // the current epoch
+  bool active = false;
+  const int64_t* seeds = nullptr;
+  int64_t num_batches = 0;
+  uint64_t rng0 = 0;
+  int64_t handed_out = 0;  // batches returned by apt_epoch_next so far
+  int64_t enqueued = 0;    // batches [0, enqueued) are on their streams
+  bool last_released = true;
+  int error = 0;
+  char error_text[512] = {0};
+  hipEvent_t done[APT_MAX_SLOTS] = {};
+  hipEvent_t released[APT_MAX_SLOTS] = {};
+  int64_t* pinned = nullptr;      // host address of the pinned size words
+  int64_t* pinned_dev = nullptr;  // the same memory as the GPU addresses it
+  apt_pending_lookup pending[APT_MAX_SLOTS];
+  // what the worker thread spent enqueueing (host time), since the handle was created
+  double enqueue_seconds = 0.0;
+  int64_t enqueued_total = 0;
+  // what apt_epoch_next spent waiting: for the worker to have enqueued the batch, then for the GPU
+  double wait_enqueue_seconds = 0.0, wait_gpu_seconds = 0.0, release_seconds = 0.0;
+};
+
+namespace apt {
+
+static int enqueue_batch(apt_epoch* ep, const EpochWork& w) {
+  const apt_epoch_desc& d = ep->d;
+  const apt_batch_slot& s = d.slots[w.slot];
+  hipStream_t st = static_cast<hipStream_t>(s.stream);
+  const int H = d.num_hops;
+  if (w.after != nullptr) APT_HIP(hipStreamWaitEvent(st, w.after, 0));
+  const int64_t* seeds = ep->seeds + w.batch * d.batch;
+  const uint64_t rng = ep->rng0 + static_cast<uint64_t>(w.batch);
+  int64_t* const* counts = s.counts[0] != nullptr ? s.counts : nullptr;
+  int rc;
+  if (s.features != nullptr && d.has_requests == 0) {
+    // the relabel's last pass rides in the gather's launch
+    rc = apt_minibatch_sample_deferred(&d.graph, seeds, d.batch, d.hop_fanouts, H, d.replace, rng, nullptr,
+                                       s.rank_table, d.rank_table_len, s.nodes, s.neighbors, s.relabeled, counts,
+                                       s.sizes, s.workspace, s.workspace_bytes, st, &ep->pending[w.slot]);
+    if (rc != APT_OK) return rc;
+    const int64_t cap = apt_minibatch_capacity(d.batch, d.hop_fanouts, H, H);
+    rc = apt_gather_rows_with_lookup(&d.store, s.nodes, cap, s.sizes + H, s.features, s.miss_count,
+                                     &ep->pending[w.slot], st);
+    if (rc != APT_OK) return rc;
+  } else {
+    rc = apt_minibatch_sample(&d.graph, seeds, d.batch, d.hop_fanouts, H, d.replace, rng, nullptr, s.rank_table,
+                              d.rank_table_len, s.nodes, s.neighbors, s.relabeled, counts, s.sizes, s.workspace,
+                              s.workspace_bytes, st);
+    if (rc != APT_OK) return rc;
+    if (d.has_requests != 0) {
+      const int64_t cap = apt_minibatch_capacity(d.batch, d.hop_fanouts, H, H);
+      rc = apt_cluster_reqs(s.nodes, cap, s.sizes + H, d.request_pos_map, d.request_num_total_nodes,
+                            d.remote_worker_map, d.min_vids, d.world_size, d.num_remote_workers, s.request_sizes,
+                            s.request_offsets, s.request_ids, s.request_perm, s.request_workspace,
+                            s.request_workspace_bytes, st);
+      if (rc != APT_OK) return rc;
+      if (s.features != nullptr) {
+        // rows that are here: features[k] belongs to request_ids[k], k < request_sizes[0]
+        rc = apt_gather_rows(&d.store, s.request_ids, cap, s.request_sizes, s.features, s.miss_count, st);
+        if (rc != APT_OK) return rc;
+      }
+    }
+  }
+  static_assert(APT_MAX_HOPS + 2 <= 64 && APT_MAX_BUCKETS <= 64, "publish_sizes_kernel runs one wavefront");
+  hipLaunchKernelGGL(publish_sizes_kernel, dim3(1), dim3(64), 0, st, s.sizes, H + 2,
+                     d.has_requests != 0 ? s.request_sizes : nullptr, d.has_requests != 0 ? d.num_remote_workers : 0,
+                     ep->pinned_dev + static_cast<size_t>(w.slot) * kPinnedPerSlot);
+  APT_LAUNCH_CHECK("publish_sizes_kernel");
+  APT_HIP(hipEventRecord(ep->done[w.slot], st));
+  return APT_OK;
+}
+
+static void worker_main(apt_epoch* ep) {
+  (void)hipSetDevice(ep->device);
+  for (;;) {
+    EpochWork w;
+    {
+      std::unique_lock<std::mutex> lk(ep->mu);
+      ep->cv_work.wait(lk, [ep] { return ep->stop || !ep->queue.empty(); });
+      if (ep->queue.empty()) return;  // stop
+      w = ep->queue.front();
+      ep->queue.pop_front();
+      ep->busy = true;
+    }
+    const auto t0 = std::chrono::steady_clock::now();
+    const int rc = ep->error == 0 ? enqueue_batch(ep, w) : APT_OK;
+    const double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    {
+      std::lock_guard<std::mutex> lk(ep->mu);
+      ep->enqueue_seconds += dt;
+      ep->enqueued_total += 1;
+      if (rc != APT_OK && ep->error == 0) {
+        ep->error = rc;
+        std::strncpy(ep->error_text, apt_last_error(), sizeof(ep->error_text) - 1);
+      }
+      ep->enqueued = w.batch + 1;
+      ep->busy = false;
+    }
+    ep->cv_done.notify_all();
+  }
+}
+
+static int check_desc(const apt_epoch_desc* d) {
+  APT_REQUIRE(d != nullptr, APT_EINVAL, "apt_epoch_create: desc is NULL");
+  APT_REQUIRE(d->batch > 0, APT_EINVAL, "apt_epoch_create: batch %lld must be > 0", (long long)d->batch);
+  APT_REQUIRE(d->num_hops >= 1 && d->num_hops <= APT_MAX_HOPS, APT_ELIMIT, "apt_epoch_create: num_hops %d outside [1, %d]",
+              d->num_hops, APT_MAX_HOPS);
+  APT_REQUIRE(d->num_slots >= 1 && d->num_slots <= APT_MAX_SLOTS, APT_ELIMIT,
+              "apt_epoch_create: num_slots %d outside [1, %d]", d->num_slots, APT_MAX_SLOTS);
+  APT_REQUIRE(apt_minibatch_capacity(d->batch, d->hop_fanouts, d->num_hops, d->num_hops) > 0, APT_ELIMIT,
+              "apt_epoch_create: unsupported batch / fanouts");
+  const size_t need = apt_minibatch_workspace_bytes(d->batch, d->hop_fanouts, d->num_hops);
+  if (d->has_requests != 0) {
+    APT_REQUIRE(d->request_pos_map != nullptr && d->remote_worker_map != nullptr && d->min_vids != nullptr &&
+                    d->world_size >= 1 && d->num_remote_workers >= 1 && d->num_remote_workers <= APT_MAX_BUCKETS,
+                APT_EINVAL, "apt_epoch_create: incomplete request description");
+  }
+  for (int k = 0; k < d->num_slots; ++k) {
+    const apt_batch_slot& s = d->slots[k];
+    APT_REQUIRE(s.nodes != nullptr && s.sizes != nullptr && s.rank_table != nullptr && s.workspace != nullptr,
+                APT_EINVAL, "apt_epoch_create: slot %d: nodes / sizes / rank_table / workspace is NULL", k);
+    APT_REQUIRE(s.workspace_bytes >= need, APT_EWORKSPACE, "apt_epoch_create: slot %d: workspace of %zu bytes, %zu needed",
+                k, s.workspace_bytes, need);
+    for (int h = 0; h < d->num_hops; ++h)
+      APT_REQUIRE(s.neighbors[h] != nullptr && s.relabeled[h] != nullptr, APT_EINVAL,
+                  "apt_epoch_create: slot %d: neighbors[%d] / relabeled[%d] is NULL", k, h, h);
+    if (d->has_requests != 0)
+      APT_REQUIRE(s.request_sizes != nullptr && s.request_ids != nullptr && s.request_perm != nullptr &&
+                      s.request_workspace != nullptr,
+                  APT_EINVAL, "apt_epoch_create: slot %d: request buffers missing", k);
+  }
+  return APT_OK;
+}
+
+}  // namespace apt
+
+extern "C" int apt_epoch_create(const apt_epoch_desc* desc, apt_epoch** out) {
+  using namespace apt;
+  APT_REQUIRE(out != nullptr, APT_EINVAL, "apt_epoch_create: out is NULL");
+  *out = nullptr;
+  if (const int rc = check_desc(desc)) return rc;
+  apt_epoch* ep = new (std::nothrow) apt_epoch();
+  APT_REQUIRE(ep != nullptr, APT_EINVAL, "apt_epoch_create: out of host memory");
+  ep->d = *desc;
+  auto fail_create = [ep](int code) {
+    for (int k = 0; k < APT_MAX_SLOTS; ++k) {
+      if (ep->done[k] != nullptr) (void)hipEventDestroy(ep->done[k]);
+      if (ep->released[k] != nullptr) (void)hipEventDestroy(ep->released[k]);
+    }
+    if (ep->pinned != nullptr) (void)hipHostFree(ep->pinned);
+    delete ep;
+    return code;
+  };
+  if (hipGetDevice(&ep->device) != hipSuccess) return fail_create(fail(APT_EHIP, "apt_epoch_create: hipGetDevice failed"));
+  for (int k = 0; k < ep->d.num_slots; ++k) {
+    // done[k] makes a kernel's stores to host memory visible to the host that waits for it
+    if (hipEventCreateWithFlags(&ep->done[k], hipEventDisableTiming | hipEventReleaseToSystem) != hipSuccess ||
+        hipEventCreateWithFlags(&ep->released[k], hipEventDisableTiming) != hipSuccess)
+      return fail_create(fail(APT_EHIP, "apt_epoch_create: hipEventCreate failed"));
+  }
+  if (hipHostMalloc(reinterpret_cast<void**>(&ep->pinned),
+                    sizeof(int64_t) * kPinnedPerSlot * static_cast<size_t>(ep->d.num_slots),
+                    hipHostMallocMapped | hipHostMallocCoherent) != hipSuccess ||
+      hipHostGetDevicePointer(reinterpret_cast<void**>(&ep->pinned_dev), ep->pinned, 0) != hipSuccess)
+    return fail_create(fail(APT_EHIP, "apt_epoch_create: pinned, device-visible host memory for the sizes is not available"));
+  std::memset(ep->pinned, 0, sizeof(int64_t) * kPinnedPerSlot * static_cast<size_t>(ep->d.num_slots));
+  ep->worker = std::thread(worker_main, ep);
+  *out = ep;
+  return APT_OK;
+}
+
+// Ends the current epoch (if any): batches not yet on a stream are dropped, the
+// one being enqueued is waited for, and the slots' streams are synchronised, so
+// that the caller may reuse or free every buffer afterwards.
+extern "C" int apt_epoch_end(apt_epoch* ep) {
+  using namespace apt;
+  APT_REQUIRE(ep != nullptr, APT_EINVAL, "apt_epoch_end: epoch is NULL");
+  {
+    std::unique_lock<std::mutex> lk(ep->mu);
+    ep->queue.clear();
+    ep->cv_done.wait(lk, [ep] { return !ep->busy; });
+    ep->active = false;
+  }
+  for (int k = 0; k < ep->d.num_slots; ++k)
+    APT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(ep->d.slots[k].stream)));
+  return APT_OK;
+}
+
+extern "C" int apt_epoch_destroy(apt_epoch* ep) {
+  if (ep == nullptr) return APT_OK;
+  const int rc = apt_epoch_end(ep);
+  {
+    std::lock_guard<std::mutex> lk(ep->mu);
+    ep->stop = true;
+  }
+  ep->cv_work.notify_all();
+  if (ep->worker.joinable()) ep->worker.join();
+  for (int k = 0; k < ep->d.num_slots; ++k) {
+    (void)hipEventDestroy(ep->done[k]);
+    (void)hipEventDestroy(ep->released[k]);
+  }
+  (void)hipHostFree(ep->pinned);
+  delete ep;
+  return rc;
+}
+
+extern "C" int apt_epoch_begin(apt_epoch* ep, const int64_t* seeds, int64_t num_batches, uint64_t rng_seed0,
+                               void* ready_event) {
+  using namespace apt;
+  APT_REQUIRE(ep != nullptr, APT_EINVAL, "apt_epoch_begin: epoch is NULL");
+  APT_REQUIRE(num_batches >= 0 && (seeds != nullptr || num_batches == 0), APT_EINVAL,
+              "apt_epoch_begin: seeds is NULL or num_batches < 0");
+  if (ep->active)
+    if (const int rc = apt_epoch_end(ep)) return rc;
+  std::lock_guard<std::mutex> lk(ep->mu);
+  ep->seeds = seeds;
+  ep->num_batches = num_batches;
+  ep->rng0 = rng_seed0;
+  ep->handed_out = 0;
+  ep->enqueued = 0;
+  ep->last_released = true;
+  ep->error = 0;
+  ep->error_text[0] = 0;
+  ep->active = true;
+  const int64_t first = std::min<int64_t>(num_batches, ep->d.num_slots);
+  for (int64_t i = 0; i < first; ++i)
+    ep->queue.push_back(EpochWork{i, static_cast<int>(i), static_cast<hipEvent_t>(ready_event)});
+  ep->cv_work.notify_all();
+  return APT_OK;
+}
+
+extern "C" int apt_epoch_next(apt_epoch* ep, int* slot, int64_t* sizes_host, int64_t* request_sizes_host) {
+  using namespace apt;
+  APT_REQUIRE(ep != nullptr && slot != nullptr && sizes_host != nullptr, APT_EINVAL,
+              "apt_epoch_next: epoch / slot / sizes_host is NULL");
+  int64_t i;
+  {
+    std::unique_lock<std::mutex> lk(ep->mu);
+    APT_REQUIRE(ep->active, APT_EINVAL, "apt_epoch_next: no epoch has been begun");
+    APT_REQUIRE(ep->handed_out < ep->num_batches, APT_EINVAL, "apt_epoch_next: the epoch has no batch left");
+    APT_REQUIRE(ep->last_released, APT_EINVAL, "apt_epoch_next: the previous batch has not been released");
+    i = ep->handed_out;
+    const auto t0 = std::chrono::steady_clock::now();
+    ep->cv_done.wait(lk, [ep, i] { return ep->enqueued > i; });
+    ep->wait_enqueue_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (ep->error != 0) return fail(ep->error, "apt_epoch_next: batch could not be enqueued: %s", ep->error_text);
+  }
+  const int k = static_cast<int>(i % ep->d.num_slots);
+  const auto t1 = std::chrono::steady_clock::now();
+  APT_HIP(hipEventSynchronize(ep->done[k]));
+  const double gpu_wait = std::chrono::duration<double>(std::chrono::steady_clock::now() - t1).count();
+  const int64_t* pin = ep->pinned + static_cast<size_t>(k) * kPinnedPerSlot;
+  for (int j = 0; j < ep->d.num_hops + 2; ++j) sizes_host[j] = pin[j];
+  if (request_sizes_host != nullptr && ep->d.has_requests != 0)
+    for (int j = 0; j < ep->d.num_remote_workers; ++j) request_sizes_host[j] = pin[APT_MAX_HOPS + 2 + j];
+  {
+    std::lock_guard<std::mutex> lk(ep->mu);
+    ep->handed_out = i + 1;
+    ep->last_released = false;
+    ep->wait_gpu_seconds += gpu_wait;
+  }
+  *slot = k;
+  return APT_OK;
+}
+
+extern "C" int apt_epoch_release(apt_epoch* ep, void* consumer_stream) {
+  using namespace apt;
+  APT_REQUIRE(ep != nullptr, APT_EINVAL, "apt_epoch_release: epoch is NULL");
+  std::unique_lock<std::mutex> lk(ep->mu);
+  APT_REQUIRE(ep->active && !ep->last_released, APT_EINVAL, "apt_epoch_release: no batch is held");
+  ep->last_released = true;
+  const int64_t i = ep->handed_out - 1;
+  const int64_t next = i + ep->d.num_slots;
+  if (next >= ep->num_batches) return APT_OK;
+  const int k = static_cast<int>(i % ep->d.num_slots);
+  lk.unlock();
+  // Whatever the consumer enqueued on its stream for batch i runs before the slot's buffers are reused.  When
+  // that stream has nothing pending there is nothing to wait for, and no event is recorded: a marker in the
+  // consumer's stream may share a hardware queue with one of the slots' streams (there are few hardware queues)
+  // and would then complete only after that stream's queued batches, stalling the slot for no reason.
+  hipEvent_t after = nullptr;
+  const auto t0 = std::chrono::steady_clock::now();
+  const hipError_t idle = hipStreamQuery(static_cast<hipStream_t>(consumer_stream));
+  if (idle == hipErrorNotReady) {
+    APT_HIP(hipEventRecord(ep->released[k], static_cast<hipStream_t>(consumer_stream)));
+    after = ep->released[k];
+  } else if (idle != hipSuccess) {
+    return fail(APT_EHIP, "apt_epoch_release: hipStreamQuery failed: %s", hipGetErrorString(idle));
+  }
+  lk.lock();
+  ep->release_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  if (ep->active) {
+    ep->queue.push_back(EpochWork{next, k, after});
+    ep->cv_work.notify_all();
+  }
+  return APT_OK;
+}
+
+extern "C" int apt_epoch_host_cost(apt_epoch* ep, apt_epoch_cost* cost) {
+  using namespace apt;
+  APT_REQUIRE(ep != nullptr && cost != nullptr, APT_EINVAL, "apt_epoch_host_cost: a pointer is NULL");
+  std::lock_guard<std::mutex> lk(ep->mu);
+  cost->batches = ep->enqueued_total;
+  cost->enqueue_seconds = ep->enqueue_seconds;
+  cost->wait_enqueue_seconds = ep->wait_enqueue_seconds;
+  cost->wait_gpu_seconds = ep->wait_gpu_seconds;
+  cost->release_seconds = ep->release_seconds;
+  return APT_OK;
+}

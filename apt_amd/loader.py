@@ -7,6 +7,12 @@ idle, the last hop is bound by random memory transactions and the gather by
 bandwidth, so batches on different streams overlap well: `in_flight` pipelines
 (own buffers and rank table each) run on streams of their own, and the consumer
 receives batch i while batches i+1 .. i+in_flight-1 are being built.
+
+The per-batch host work (a dozen kernel launches, the copy of the sizes, the
+events) is done by a thread of the C library (apt_epoch_*, capi.EpochDriver):
+the Python thread only waits for the next batch and narrows its buffers.  With
+block formats or graph replay requested the batches are enqueued from Python
+instead (driver="python" forces that path).
 """
 import torch
 
@@ -15,7 +21,8 @@ from .pipeline import MiniBatchPipeline
 
 class MiniBatchLoader:
     def __init__(self, graph, feat, indices, batch_size, hop_fanouts, in_flight=4, shuffle=True, drop_last=True,
-                 replace=False, seed=0, formats=False, requests=None, use_graph=False, as_blocks=False):
+                 replace=False, seed=0, formats=False, requests=None, use_graph=False, as_blocks=False,
+                 driver="auto"):
         """indices: node ids to draw seeds from (the training ids).  hop_fanouts
         start from the seeds.  Yields MiniBatchPipeline.result() dicts with
         `output_nodes` (the batch's seeds) added.  A yielded batch lives in its
@@ -24,7 +31,9 @@ class MiniBatchLoader:
         waited for before the buffers are reused.  use_graph: every pipeline
         replays a captured HIP graph, which costs the host less per batch (worth it
         for small batches, where the host's launch calls are the limit).  as_blocks:
-        batch["blocks"] are sampler.Block objects, ready for apt_amd.layers."""
+        batch["blocks"] are sampler.Block objects, ready for apt_amd.layers.
+        driver: "c" = batches are enqueued by the C library's epoch thread (not with formats or use_graph),
+        "python" = from this thread, "auto" = "c" where it applies."""
         if in_flight < 1:
             raise ValueError("in_flight must be >= 1")
         dev = graph.device
@@ -46,9 +55,26 @@ class MiniBatchLoader:
         self.tail_pipe = self._make(self.tail) if self.tail else None     # the short last batch has buffers of its own
         self.as_blocks = bool(as_blocks)
         self.epoch = 0
+        if driver not in ("auto", "c", "python"):
+            raise ValueError("driver must be 'auto', 'c' or 'python'")
+        c_ok = not formats and not use_graph
+        if driver == "c" and not c_ok:
+            raise ValueError("the C epoch driver does not emit block formats or replay graphs: use driver='python'")
+        self._c_driver = None
+        self._use_c = c_ok and driver != "python"
+        # The C driver enqueues batch i + F behind batch i on the same stream without waiting for the consumer,
+        # so that no stream runs dry between a batch's completion and the consumer's release of it: that takes a
+        # second set of buffers per stream (the two sets of a stream share its rank table).
+        self._spare = ([MiniBatchPipeline(graph, feat, self.batch_size, hop_fanouts, table=p.plan.table, **kw)
+                        for p in self.pipes] if self._use_c else [])
 
     def __len__(self):
         return self.num_full + (1 if self.tail else 0)
+
+    def host_cost(self):
+        """What the C driver's thread has spent enqueueing and what the consumer has spent waiting, in seconds,
+        since the loader's first epoch (capi.EpochDriver.host_cost); None on the Python path."""
+        return self._c_driver.host_cost() if self._c_driver is not None else None
 
     def _launch(self, k, pipe, seeds, rng_seed, after):
         st = self.streams[k]
@@ -74,6 +100,9 @@ class MiniBatchLoader:
         F = len(self.pipes)
         ready = torch.cuda.Event()
         ready.record(cur)                                  # the seeds above were produced on the consumer's stream
+        if self._use_c:
+            yield from self._iter_c(full, batches, rng0, ready)
+            return
 
         def launch(i, after):
             k = i % F
@@ -97,3 +126,35 @@ class MiniBatchLoader:
                 cur = torch.cuda.current_stream(self.device)
                 self.released[k].record(cur)
                 owner[i + F] = launch(i + F, self.released[k])
+
+    def _iter_c(self, full, batches, rng0, ready):
+        """The epoch through the C library's driver: its thread enqueues batch i on pipeline i % F; this
+        thread waits for batches in order.  The short last batch (drop_last=False) has buffers of its own and
+        is run from here after the others."""
+        from . import capi
+        slots = self.pipes + self._spare
+        if self._c_driver is None:
+            self._c_driver = capi.EpochDriver(slots, self.streams + self.streams)
+        drv = self._c_driver
+        if self.num_full:
+            drv.begin(full.reshape(-1), self.num_full, rng0, ready)
+            try:
+                for i in range(self.num_full):
+                    k, sizes, rs = drv.next()
+                    pipe = slots[k]
+                    pipe.seeds = batches[i]
+                    out = pipe.result(as_blocks=self.as_blocks, sizes=sizes, request_sizes=rs)
+                    out["output_nodes"] = batches[i]
+                    yield out
+                    drv.release()
+            finally:
+                drv.end()
+        if self.tail:
+            cur = torch.cuda.current_stream(self.device)
+            self.released[0].record(cur)
+            self._launch(0, self.tail_pipe, batches[-1], rng0 + self.num_full, self.released[0])
+            cur.wait_event(self.done[0])
+            self.done[0].synchronize()
+            out = self.tail_pipe.result(staged=True, as_blocks=self.as_blocks)
+            out["output_nodes"] = batches[-1]
+            yield out

@@ -22,7 +22,7 @@ from . import capi
 
 class MiniBatchPipeline:
     def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
-                 use_graph=False, requests=None, formats=False, defer_lookup=False):
+                 use_graph=False, requests=None, formats=False, defer_lookup=False, table=None):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
         --fan_out list reversed).
 
@@ -39,6 +39,9 @@ class MiniBatchPipeline:
         batch, while that launch gets 2-3 us longer (it is no longer the gather alone).  Only where the gather
         is what follows the sampling (fused driver, features gathered, no requests, no formats).
 
+        table: the rank table of another pipeline (fused driver) whose batches run on the same stream as this
+        one's: batches that follow each other on one stream can share a table (444 MB at 111 M nodes).
+
         formats: True or "csc" also emits every hop's block as COO + CSC (+ CSR
         with True), what DGL derives from (row, col) in the reference
         (python/npc/sampler.py:59-69); result() then carries them per block."""
@@ -51,7 +54,7 @@ class MiniBatchPipeline:
         H = len(self.fanouts)
         i64 = dict(dtype=torch.int64, device=dev)
         if self.fused:
-            self.plan = capi.MinibatchPlan(graph, batch_size, self.fanouts, replace=replace)
+            self.plan = capi.MinibatchPlan(graph, batch_size, self.fanouts, replace=replace, table=table)
             self.caps = self.plan.caps
             self.sizes = self.plan.sizes
             self.neighbors, self.relabeled, self.counts = (self.plan.neighbors, self.plan.relabeled,
@@ -231,17 +234,20 @@ class MiniBatchPipeline:
                 self.format_edges_host = torch.empty(len(self.fanouts), dtype=torch.int64, pin_memory=True)
             self.format_edges_host.copy_(self.format_edges, non_blocking=True)
 
-    def result(self, staged=False, as_blocks=False):
+    def result(self, staged=False, as_blocks=False, sizes=None, request_sizes=None):
         """Waits for the batch and narrows the buffers to their real sizes ->
         dict(input_nodes, blocks (outermost first), features, num_edges).
         staged: the sizes were copied by stage_sizes() and that copy has finished.
+        sizes (and request_sizes): the batch's sizes as host lists, when the caller already has them (the
+        epoch driver reads them from pinned memory); nothing is waited for then.
         as_blocks: the blocks come as sampler.Block objects (what the layers of
         apt_amd.layers take) instead of dicts; they live in this pipeline's buffers
         like everything else, so a training step must finish with them before the
         pipeline runs its next batch."""
         if self.fused and self.plan.pending.open:      # sampled with the last pass deferred and never gathered
             self.plan.pending.run()
-        sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
+        if sizes is None:
+            sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
         fmt_edges = None
         if self.formats is not None:
             fmt_edges = self.format_edges_host.tolist() if staged else self.format_edges.cpu().tolist()
@@ -268,7 +274,8 @@ class MiniBatchPipeline:
         out = dict(input_nodes=inp, blocks=blocks, features=feats, num_edges=sizes[-1],
                    sizes=sizes[:-1])
         if self.requests is not None:
-            rs = self.request_sizes_host.tolist() if staged else self.request_sizes.cpu().tolist()
+            rs = request_sizes if request_sizes is not None else (
+                self.request_sizes_host.tolist() if staged else self.request_sizes.cpu().tolist())
             out.update(request_sizes=rs, request_ids=self.request_ids[:sizes[H]],
                        request_perm=self.request_perm[:sizes[H]],
                        features=None if self.features is None else self.features[:rs[0]])

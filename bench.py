@@ -139,11 +139,21 @@ class KernelEvents:
         self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
         self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
         self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
 
     def pair(self):
         a, b = ctypes.c_void_p(), ctypes.c_void_p()
         assert self.hip.hipEventCreate(ctypes.byref(a)) == 0 and self.hip.hipEventCreate(ctypes.byref(b)) == 0
         return a, b
+
+    def record(self, event, stream):
+        """Records `event` on a torch stream."""
+        rc = self.hip.hipEventRecord(event, ctypes.c_void_p(stream.cuda_stream))
+        assert rc == 0, f"hipEventRecord -> {rc}"
+
+    def destroy(self, pair):
+        self.hip.hipEventDestroy(pair[0])
+        self.hip.hipEventDestroy(pair[1])
 
     def ms(self, pair, destroy=True):
         ms = ctypes.c_float()
@@ -483,17 +493,11 @@ def stage_target_shape(args, ctx, wl, hops, store_of):
         if args.driver == "fused" and args.inflight > 1:
             loader = MiniBatchLoader(wl.graph, store, torch.cat(sets), B, hops, in_flight=args.inflight,
                                      shuffle=False, replace=args.replace, seed=args.seed)
-            it = iter(loader)
-            for _ in range(Wt):
-                next(it)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            l_edges = sum(batch["num_edges"] for batch in it)
-            torch.cuda.synchronize()
-            t_ld = time.perf_counter() - t0
+            t_ld, l_edges, gaps = time_loader(torch, loader, Wt)
             loader_fig = {"batches_in_flight": args.inflight, "ms_per_step": t_ld / Kt * 1e3,
-                          "edges_per_s": l_edges / t_ld}
-            del loader, it
+                          "edges_per_s": l_edges / t_ld, "ms_between_batches": gaps,
+                          "host_us_per_batch": loader_cost_per_batch(loader)}
+            del loader
         q_us, q_frac = quantiles(us), quantiles(frac)
         tr = MEASURED_GATHER_TRAFFIC_PER_ROW.get(("target", wl.graph_kind, name, store.out_dim, B), (None, None))
         out[name] = {
@@ -514,6 +518,42 @@ def stage_target_shape(args, ctx, wl, hops, store_of):
         }
         del log, sets, pool
     return out
+
+
+def quiet_gc():
+    """Python's cycle collector walks every container object of the process when it runs a full collection
+    (tens of milliseconds with torch imported), and the loops below allocate enough small objects per batch to
+    set one off inside a timed region now and then.  Everything alive after set-up is moved out of its reach;
+    the garbage of the timed loops themselves is still collected."""
+    import gc
+    gc.collect()
+    gc.freeze()
+
+
+def time_loader(torch, loader, warm):
+    """One epoch of `loader` after `warm` untimed batches -> (seconds, sampled edges, quantiles of the time
+    between consecutive batches in ms)."""
+    it = iter(loader)
+    for _ in range(warm):
+        next(it)
+    torch.cuda.synchronize()
+    stamps = [time.perf_counter()]
+    edges = 0
+    for batch in it:
+        edges += batch["num_edges"]
+        stamps.append(time.perf_counter())
+    torch.cuda.synchronize()
+    stamps[-1] = time.perf_counter()
+    return stamps[-1] - stamps[0], edges, quantiles([(b - a) * 1e3 for a, b in zip(stamps, stamps[1:])])
+
+
+def loader_cost_per_batch(loader):
+    """What a batch costs the host through the loader's C driver, in us: the driver thread's enqueue calls, and
+    the consumer's waits for that thread and for the GPU."""
+    c = loader.host_cost()
+    if not c or not c["batches"]:
+        return None
+    return {k.replace("_seconds", ""): v / c["batches"] * 1e6 for k, v in c.items() if k != "batches"}
 
 
 def stage_ceilings(ctx, N):
@@ -681,6 +721,7 @@ def stage_config(args, ctx, name, full_graph=None, with_aggregation=False):
     torch = ctx.torch
     w = dict(WORKLOADS[name])
     wl = build_workload(args, name, w, ctx, full_graph=full_graph)
+    quiet_gc()
     hops = list(reversed(w["fan_out"]))
     K, W = args.config_steps, 10
     m = measure(args, ctx, wl, w["batch"], hops, K, W, event_steps=16, per_step=False)
@@ -706,16 +747,10 @@ def stage_config(args, ctx, name, full_graph=None, with_aggregation=False):
         from apt_amd.loader import MiniBatchLoader
         loader = MiniBatchLoader(wl.graph, wl.store, torch.cat(m.seed_sets), m.B, hops, in_flight=args.inflight,
                                  shuffle=False, replace=args.replace, seed=args.seed, requests=wl.requests)
-        it = iter(loader)
-        for _ in range(W):
-            next(it)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        l_edges = sum(batch["num_edges"] for batch in it)
-        torch.cuda.synchronize()
-        t_ld = time.perf_counter() - t0
-        out["loader"] = {"batches_in_flight": args.inflight, "ms_per_step": t_ld / K * 1e3, "edges_per_s": l_edges / t_ld}
-        del loader, it
+        t_ld, l_edges, gaps = time_loader(torch, loader, W)
+        out["loader"] = {"batches_in_flight": args.inflight, "ms_per_step": t_ld / K * 1e3, "edges_per_s": l_edges / t_ld,
+                         "ms_between_batches": gaps, "host_us_per_batch": loader_cost_per_batch(loader)}
+        del loader
     if args.cpu_seconds > 0:
         # feature tables of the partition are 17 GB: its rows are compared in tests/test_gpu_configs.py, not here
         h = host_copies(ctx, wl, with_features=wl.requests is None)
@@ -769,6 +804,7 @@ def main():
     H = len(hops)
 
     wl = build_workload(args, args.workload, w, ctx)
+    quiet_gc()
     m = measure(args, ctx, wl, B, hops, K, W, args.event_steps)
     pipe, stage_pipe, seed_sets = m.pipe, m.stage_pipe, m.seed_sets
     edges, rows = m.edges, m.rows
@@ -830,6 +866,9 @@ def main():
         assert all(int(p.misses.item()) == 0 for p in pipes)
         in_flight = {"batches_in_flight": len(pipes), "ms_per_step": t_fl / K * 1e3,
                      "edges_per_s": edges / t_fl}
+        if args.driver == "fused" and wl.requests is None:
+            in_flight["timeline"] = extra.stage_in_flight_timeline(args, capi, kev, torch, pipes, streams, seed_sets,
+                                                                   W, K, hops)
         del pipes[1:]
         # the same through the epoch loader a trainer would use (MiniBatchLoader): the consumer receives
         # every batch narrowed to its sizes, which costs one host read-back per batch
@@ -837,16 +876,10 @@ def main():
             from apt_amd.loader import MiniBatchLoader
             loader = MiniBatchLoader(wl.graph, wl.store, torch.cat(seed_sets), B, hops, in_flight=args.inflight,
                                      shuffle=False, replace=args.replace, seed=args.seed, requests=wl.requests)
-            it = iter(loader)
-            for _ in range(W):
-                next(it)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            loader_edges = sum(batch["num_edges"] for batch in it)
-            torch.cuda.synchronize()
-            t_ld = time.perf_counter() - t0
-            in_flight["loader"] = {"ms_per_step": t_ld / K * 1e3, "edges_per_s": loader_edges / t_ld}
-            del loader, it
+            t_ld, loader_edges, gaps = time_loader(torch, loader, W)
+            in_flight["loader"] = {"ms_per_step": t_ld / K * 1e3, "edges_per_s": loader_edges / t_ld,
+                                   "ms_between_batches": gaps, "host_us_per_batch": loader_cost_per_batch(loader)}
+            del loader
 
     agg = None
     if args.aggregation:

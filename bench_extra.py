@@ -361,3 +361,82 @@ def stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, see
             "gather_us_median": st.median(r["gather_us"]),
             "last_hop_sample_us_median": st.median(r["sample_us"]) if args.driver == "fused" else None})
     return out
+
+
+def interval_union(iv):
+    """Total length covered by a list of (start, end) intervals."""
+    tot, cs, ce = 0.0, None, None
+    for s_, e_ in sorted(iv):
+        if cs is None:
+            cs, ce = s_, e_
+        elif s_ > ce:
+            tot += ce - cs
+            cs, ce = s_, e_
+        else:
+            ce = max(ce, e_)
+    return tot + (ce - cs if cs is not None else 0.0)
+
+
+def covered_at_least(iv, k):
+    """Total time during which at least k of the intervals are open."""
+    pts = sorted([(s_, 1) for s_, _ in iv] + [(e_, -1) for _, e_ in iv])
+    tot, open_, last = 0.0, 0, None
+    for t, d in pts:
+        if last is not None and open_ >= k:
+            tot += t - last
+        open_ += d
+        last = t
+    return tot
+
+
+def stage_in_flight_timeline(args, capi, kev, torch, pipes, streams, seed_sets, first, count, hops):
+    """Where the time of the batches-in-flight arrangement goes, without a profiler in the way: every batch's
+    last-hop sampling kernel and gather kernel carry HIP events on their dispatches; read against one base
+    event they give each kernel's begin and end on the GPU's clock, across streams.  -> how much of the
+    region has a gather running, a last-hop sampler running, two of a kind at once, one of each at once, or
+    neither (only the short kernels of hops 1-2 and the relabel passes), and how the two kernels stretch when
+    they share the GPU."""
+    H = len(hops)
+    base = kev.pair()
+    gp, sp = [], []
+    torch.cuda.synchronize()
+    kev.record(base[0], streams[0])
+    for i in range(count):
+        k = i % len(pipes)
+        with torch.cuda.stream(streams[k]):
+            g, s_ = kev.pair(), kev.pair()
+            capi.check(capi.lib().apt_time_next_sample(H - 1, s_[0], s_[1]))
+            pipes[k].sample(seed_sets[first + i], args.seed + 100 + first + i, defer_lookup=True)
+            capi.check(capi.lib().apt_time_next_gather(g[0], g[1]))
+            pipes[k].gather()
+            gp.append(g)
+            sp.append(s_)
+    torch.cuda.synchronize()
+    at = lambda ev: kev.ms((base[0], ev), destroy=False) * 1e3
+    gat = [(at(a), at(b)) for a, b in gp]
+    sam = [(at(a), at(b)) for a, b in sp]
+    for pr in gp + sp + [base]:
+        kev.destroy(pr)
+    # leave the ramp-up and the drain out: the middle 80 % of the batches
+    lo, hi = count // 10, count - count // 10
+    gat_m, sam_m = gat[lo:hi], sam[lo:hi]
+    t0, t1 = min(s_ for s_, _ in sam_m), max(e_ for _, e_ in gat_m)
+    clip = lambda iv: [(max(a, t0), min(b, t1)) for a, b in iv if b > t0 and a < t1]
+    g_all, s_all = clip(gat), clip(sam)
+    span = t1 - t0
+    both = interval_union(g_all) + interval_union(s_all) - interval_union(g_all + s_all)
+    return {
+        "batches": hi - lo, "us_per_batch": span / (hi - lo),
+        "gather_us_mean": sum(b - a for a, b in gat_m) / len(gat_m),
+        "last_hop_sample_us_mean": sum(b - a for a, b in sam_m) / len(sam_m),
+        "fraction_of_time": {
+            "a_gather_running": interval_union(g_all) / span,
+            "a_last_hop_sampler_running": interval_union(s_all) / span,
+            "either_running": interval_union(g_all + s_all) / span,
+            "a_gather_and_a_sampler_running": both / span,
+            "two_or_more_gathers_running": covered_at_least(g_all, 2) / span,
+            "two_or_more_samplers_running": covered_at_least(s_all, 2) / span,
+            "neither_running": 1.0 - interval_union(g_all + s_all) / span,
+        },
+        "timing": "HIP events carried by every batch's two largest dispatches, read against one base event",
+    }

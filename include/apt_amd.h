@@ -383,6 +383,115 @@ int apt_gather_rows_with_lookup(const apt_feat_store* store, const int64_t* inde
                                 int64_t* miss_count, const apt_pending_lookup* pending,
                                 void* stream);
 
+/* Epoch driver: what a trainer's data loader does around the sampler, with the
+ * per-batch host work done by a thread of this library instead of the caller's.
+ * Replaces the loop `for input_nodes, output_nodes, blocks in dataloader:` +
+ * load_subtensor of the reference's trainer (examples/train.py:84-94,139; the
+ * dgl DataLoader is built in python/npc/utils/utils.py with batch size :425),
+ * DP strategy: per batch MixedPSNeighborSampler.sample
+ * (python/npc/sampler.py:187-203,358-364) and load_subtensor
+ * (python/npc/ops.py:598-600).
+ *
+ * The caller provides num_slots sets of device buffers ("slots", what
+ * apt_minibatch_sample and apt_gather_rows take, plus a HIP stream each) and,
+ * per epoch, the seeds of all batches as one device array.  The driver's thread
+ * enqueues batch i on slot i % num_slots: apt_minibatch_sample_deferred +
+ * apt_gather_rows_with_lookup (no features: apt_minibatch_sample alone; a
+ * partitioned store: apt_minibatch_sample, apt_cluster_reqs on the input nodes,
+ * apt_gather_rows of bucket 0), then copies the batch's sizes to pinned host
+ * memory and records an event.  num_slots batches are in flight at any time.
+ * Batch i is built from seeds[i * batch, (i + 1) * batch) with rng seed
+ * rng_seed0 + i and is bit-identical to what those calls give on their own.
+ * Nothing here allocates device memory; pinned host memory for the sizes, the
+ * events and the thread belong to the handle. */
+#define APT_MAX_SLOTS 16
+typedef struct apt_batch_slot {
+  void* stream;                       /* hipStream_t of this slot (not the default stream) */
+  int64_t* nodes;                     /* as in apt_minibatch_sample, sized by apt_minibatch_capacity */
+  int64_t* neighbors[APT_MAX_HOPS];
+  int64_t* relabeled[APT_MAX_HOPS];
+  int64_t* counts[APT_MAX_HOPS];      /* counts[0] == NULL: no counts */
+  int64_t* sizes;                     /* device int64[num_hops + 2] */
+  void* rank_table;                   /* a table per slot (apt_rank_table_init) */
+  void* workspace;                    /* apt_minibatch_workspace_bytes, initialised once */
+  size_t workspace_bytes;
+  void* features;                     /* [capacity(num_hops), out_dim] elements, or NULL for no gather */
+  int64_t* miss_count;                /* optional device int64[1], see apt_gather_rows */
+  /* partitioned feature store only (apt_epoch_desc.has_requests), as in apt_cluster_reqs: */
+  int64_t* request_sizes;             /* device int64[num_remote_workers] */
+  int64_t* request_offsets;           /* optional */
+  int64_t* request_ids;               /* device int64[capacity(num_hops)] */
+  int64_t* request_perm;              /* device int64[capacity(num_hops)] */
+  void* request_workspace;            /* apt_bucket_workspace_bytes(capacity(num_hops), num_remote_workers) */
+  size_t request_workspace_bytes;
+} apt_batch_slot;
+
+typedef struct apt_epoch_desc {
+  apt_graph graph;
+  apt_feat_store store;               /* read only when the slots have feature buffers */
+  int64_t batch;
+  int num_hops;
+  int hop_fanouts[APT_MAX_HOPS];      /* from the seeds outward */
+  int replace;
+  int64_t rank_table_len;
+  int has_requests;                   /* != 0: bucket the input nodes (apt_cluster_reqs), gather bucket 0 */
+  const int64_t* request_pos_map;     /* feat_pos_map of apt_cluster_reqs */
+  int64_t request_num_total_nodes;
+  const int64_t* remote_worker_map;
+  const int64_t* min_vids;
+  int world_size;
+  int num_remote_workers;
+  int num_slots;
+  apt_batch_slot slots[APT_MAX_SLOTS];
+} apt_epoch_desc;
+
+typedef struct apt_epoch apt_epoch;   /* opaque */
+
+/* apt_epoch_create   copies *desc (the buffers it points to stay the caller's and
+ *                    must outlive the handle), creates events, pinned memory and
+ *                    the thread, for the GPU that is current.
+ * apt_epoch_begin    starts an epoch of num_batches batches over seeds (device
+ *                    int64[num_batches * batch], must stay valid until the epoch
+ *                    ends); the slots' streams first wait for ready_event
+ *                    (hipEvent_t, may be NULL: the seeds are already complete).
+ *                    An epoch still in progress is ended first.
+ * apt_epoch_next     blocks until the next batch (they come in order) is
+ *                    complete on the GPU; *slot = the slot that holds it,
+ *                    sizes_host[num_hops + 2] = its sizes as apt_minibatch_sample
+ *                    defines them, request_sizes_host[num_remote_workers]
+ *                    (optional) the request buckets.  The slot's buffers are
+ *                    the caller's to read until apt_epoch_release.
+ * apt_epoch_release  the caller is done with the batch apt_epoch_next returned
+ *                    last: work it has enqueued on consumer_stream so far is
+ *                    waited for (by the slot's stream, not the host) before the
+ *                    slot is reused for batch i + num_slots.  Must be called
+ *                    before the next apt_epoch_next.
+ * apt_epoch_end      drops what has not been enqueued, synchronises the slots'
+ *                    streams; after it every buffer is quiescent.  Optional
+ *                    after the last batch.
+ * apt_epoch_destroy  apt_epoch_end, then stops the thread and frees the handle.
+ * One consumer thread per handle.  A batch that could not be enqueued makes
+ * apt_epoch_next return its error. */
+int apt_epoch_create(const apt_epoch_desc* desc, apt_epoch** out);
+int apt_epoch_begin(apt_epoch* epoch, const int64_t* seeds, int64_t num_batches, uint64_t rng_seed0,
+                    void* ready_event);
+int apt_epoch_next(apt_epoch* epoch, int* slot, int64_t* sizes_host, int64_t* request_sizes_host);
+int apt_epoch_release(apt_epoch* epoch, void* consumer_stream);
+int apt_epoch_end(apt_epoch* epoch);
+int apt_epoch_destroy(apt_epoch* epoch);
+/* Where the host's time went since the handle was created: what the driver's
+ * thread spent enqueueing batches (what a batch costs the host), and what
+ * apt_epoch_next spent waiting, first for the batch to be on its stream, then
+ * for the GPU to finish it. */
+typedef struct apt_epoch_cost {
+  int64_t batches;              /* batches enqueued so far */
+  double enqueue_seconds;       /* driver thread, inside the enqueue calls */
+  double wait_enqueue_seconds;  /* apt_epoch_next, waiting for the driver thread */
+  double wait_gpu_seconds;      /* apt_epoch_next, waiting for the batch's completion event */
+  double release_seconds;       /* apt_epoch_release, asking the consumer's stream whether it is idle */
+} apt_epoch_cost;
+int apt_epoch_host_cost(apt_epoch* epoch, apt_epoch_cost* cost);
+
 /* Cache construction (the callers of the registries).
  *   apt_count_ids        freq[ids[i]] += 1 for ids in [0, num_total_nodes): the
  *                        access counting of a dry run (examples/dryrun.py:86-92,

@@ -158,3 +158,49 @@ def test_sample_blocks_returns_fresh_tensors_by_default():
     assert torch.ops.npc.block_buffer_ring() == 0
     with pytest.raises(RuntimeError, match="0..64"):
         apt_amd.ops.set_block_buffer_ring(-1)
+
+
+def test_ctypes_structs_match_the_header(tmp_path):
+    """The ctypes mirrors of the ABI's structs have the size and field offsets the C compiler gives them."""
+    import subprocess
+
+    from apt_amd import capi
+    src = tmp_path / "sizes.c"
+    fields = [("apt_graph", capi.CGraph, ["indptr", "adj_pos_map", "num_total_nodes"]),
+              ("apt_feat_store", capi.CFeatStore, ["pos_map", "out_dim", "elem_size"]),
+              ("apt_batch_slot", capi.CBatchSlot, ["counts", "workspace_bytes", "features", "request_workspace_bytes"]),
+              ("apt_epoch_desc", capi.CEpochDesc, ["store", "hop_fanouts", "rank_table_len", "request_pos_map",
+                                                   "num_remote_workers", "num_slots", "slots"])]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "apt_amd.h"', "int main(void) {"]
+    for name, _, fs in fields:
+        lines.append(f'  printf("%zu\\n", sizeof({name}));')
+        lines += [f'  printf("%zu\\n", offsetof({name}, {f}));' for f in fs]
+    lines += ['  printf("%zu %d %d %d\\n", sizeof(apt_pending_lookup), APT_MAX_HOPS, APT_MAX_SLOTS, APT_MAX_BUCKETS);',
+              "  return 0;", "}"]
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()
+    it = iter(out)
+    for name, ct, fs in fields:
+        assert int(next(it)) == ctypes.sizeof(ct), name
+        for f in fs:
+            assert int(next(it)) == getattr(ct, f).offset, (name, f)
+    assert [int(x) for x in it] == [512, capi.MAX_HOPS, capi.MAX_SLOTS, 64]
+
+
+def test_epoch_driver_argument_checks_need_no_gpu():
+    from apt_amd import capi
+    L = capi.lib()
+    h = ctypes.c_void_p()
+    d = capi.CEpochDesc()
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"batch" in L.apt_last_error()
+    d.batch, d.num_hops, d.num_slots = 64, 2, 1
+    d.hop_fanouts[0], d.hop_fanouts[1] = 5, 5
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"slot 0" in L.apt_last_error()
+    d.num_slots = 17
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"num_slots" in L.apt_last_error()
+    assert not h.value
+    assert L.apt_epoch_next(None, None, None, None) != 0 and L.apt_epoch_release(None, None) != 0
+    assert L.apt_epoch_begin(None, None, 0, 0, None) != 0 and L.apt_epoch_end(None) != 0
+    assert L.apt_epoch_destroy(None) == 0

@@ -65,6 +65,70 @@ def test_loader_matches_single_pipeline(capi, in_flight, drop_last, formats, use
     assert not torch.equal(first, got)                   # epochs are shuffled differently
 
 
+def test_loader_c_and_python_drivers_agree(capi):
+    """The C library's epoch thread and the Python enqueue path build the same batches; the C path is what a
+    loader without formats uses by default."""
+    import torch
+
+    from apt_amd.loader import MiniBatchLoader
+    g, store, table = _setup(capi)
+    ids = torch.arange(3000, 3000 + 2100).cuda()
+    kw = dict(in_flight=3, shuffle=True, drop_last=False, seed=11)
+    a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", **kw)
+    b = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="python", **kw)
+    assert a._use_c and not b._use_c and MiniBatchLoader(g, store, ids, 200, [4], **kw)._use_c
+    with pytest.raises(ValueError):
+        MiniBatchLoader(g, store, ids, 200, [4], driver="c", formats=True)
+    for epoch in range(2):
+        n = 0
+        for x, y in zip(a, b):
+            assert torch.equal(x["output_nodes"], y["output_nodes"]) and x["sizes"] == y["sizes"]
+            assert torch.equal(x["input_nodes"], y["input_nodes"]) and torch.equal(x["features"], y["features"])
+            assert x["num_edges"] == y["num_edges"]
+            for p, q in zip(x["blocks"], y["blocks"]):
+                for k in ("seeds", "neighbors", "relabeled", "counts", "unique"):
+                    assert torch.equal(p[k], q[k]), k
+            n += 1
+        assert n == 11
+
+
+def test_loader_with_partitioned_store(capi):
+    """A partitioned feature store through the loader: request lists and the rows held here are what a lone
+    pipeline produces for the same seeds and key."""
+    import torch
+
+    from apt_amd import synth
+    from apt_amd.loader import MiniBatchLoader
+    from apt_amd.pipeline import MiniBatchPipeline
+    n, lo, hi, dim, P = 30000, 10000, 20000, 16, 4
+    indptr, indices = synth.rmat_csr_gpu(n, 12 * n, seed=9)
+    g = capi.Graph((indptr[lo:hi + 1] - indptr[lo]).contiguous(), indices[int(indptr[lo]):int(indptr[hi])].clone(),
+                   row_begin=lo, num_total_nodes=n)
+    local = synth.random_features(hi - lo, dim, torch.float32, seed=4)
+    hot = torch.cat([torch.arange(0, 3000), torch.arange(25000, 26000)]).cuda()
+    cache = synth.random_features(hot.numel(), dim, torch.float32, seed=5)
+    pos = torch.full((n,), -1, dtype=torch.int64, device="cuda")
+    pos[lo:hi] = -torch.arange(hi - lo, device="cuda") - 2
+    pos[hot] = torch.arange(hot.numel(), device="cuda")
+    store = capi.FeatStore(local, cache, pos)
+    rq = dict(feat_pos_map=pos, remote_worker_map=torch.tensor([1, 0, 2, 3], device="cuda"),
+              min_vids=torch.tensor([0, 10000, 20000, 25000, 30000], device="cuda"), world_size=P, num_remote_workers=P)
+    ids = torch.arange(lo, lo + 1280).cuda()
+    lone = MiniBatchPipeline(g, store, 128, [4, 4], requests=rq)
+    for driver in ("c", "python"):
+        loader = MiniBatchLoader(g, store, ids, 128, [4, 4], in_flight=3, shuffle=False, seed=2, requests=rq,
+                                 driver=driver)
+        for i, batch in enumerate(loader):
+            lone.run(ids[i * 128:(i + 1) * 128], 2 * 7919 * 10 + i)
+            want = lone.result()
+            assert batch["request_sizes"] == want["request_sizes"] and sum(batch["request_sizes"]) == want["sizes"][-1]
+            assert batch["request_sizes"][0] > 0 and sum(batch["request_sizes"][1:]) > 0
+            assert torch.equal(batch["request_ids"], want["request_ids"])
+            assert torch.equal(batch["request_perm"], want["request_perm"])
+            assert torch.equal(batch["features"], want["features"]) and torch.equal(batch["input_nodes"], want["input_nodes"])
+        assert i == 9
+
+
 def test_loader_without_shuffle_and_early_exit(capi):
     import torch
 
