@@ -71,6 +71,9 @@ SYMBOLS = {
     "apt_sample_neighbors": (_I, [C.POINTER(CGraph), _P, _I64, _P, _I, _I, _U64, _I, _P, _P, _P, _P]),
     "apt_relabel_workspace_bytes": (_SZ, [_I64]),
     "apt_relabel": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_relabel_ranked_max_items": (_I64, []),
+    "apt_relabel_ranked_workspace_bytes": (_SZ, [_I64]),
+    "apt_relabel_ranked": (_I, [_P, _I64, _P, _P, _I64, _I64, _I, _P, _I64, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "apt_relabel_static_max_items": (_I64, []),
     "apt_relabel_static": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P]),
     "apt_gather_rows": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P]),
@@ -319,6 +322,65 @@ def relabel(seeds, neighbors, num_seeds_dev=None, neighbor_stride=0, unique=None
     if sync:
         return unique[:host.value], relabeled, int(host.value)
     return unique, relabeled, num_unique_dev
+
+
+class RankedRelabel:
+    """apt_relabel_ranked with its rank table and workspace: relabel calls for ids below num_total_nodes.
+    relabel(seeds, neighbors) -> (unique, relabeled, num_unique) like capi.relabel(sync=True); a call whose seeds
+    are the tensor the previous call returned as `unique` continues that batch (the table still holds its ids)."""
+
+    def __init__(self, num_total_nodes, device):
+        self.table = rank_table(num_total_nodes, device)
+        self.table_len = int(num_total_nodes)
+        self.workspace = None
+        self.counts = torch.zeros(2, dtype=torch.int64, device=device)
+        # the unique list the last call returned (kept alive, so that its address cannot be given to another
+        # tensor) and its (data_ptr, numel, version): seeds with the same identity continue that batch
+        self._last, self._last_tensor = None, None
+        torch.cuda.current_stream().synchronize()
+
+    def _workspace_for(self, items, device):
+        need = int(lib().apt_relabel_ranked_workspace_bytes(items))
+        if need == 0:
+            raise AptError(f"relabel_ranked: {items} items exceed the supported maximum")
+        if self.workspace is None or self.workspace.numel() < need:
+            self.workspace = torch.empty(max(need, 256) * 2, dtype=torch.uint8, device=device)
+            check(lib().apt_minibatch_workspace_init(_ptr(self.workspace), self.workspace.numel(), _stream()))
+
+    def enqueue(self, seeds, neighbors, continued, unique, relabeled, num_unique_dev, num_outside_dev,
+                num_seeds_dev=None, neighbor_stride=0):
+        """Asynchronous form with the caller's buffers and device-side sizes (as capi.relabel(sync=False)):
+        num_unique_dev receives the count, num_outside_dev is incremented per id outside the table (device
+        int64[1] each; the caller clears the second)."""
+        seeds, neighbors = _dev_i64(seeds, "seeds"), _dev_i64(neighbors, "neighbors")
+        self._workspace_for(seeds.numel() + neighbors.numel(), seeds.device)
+        self._last = self._last_tensor = None
+        check(lib().apt_relabel_ranked(_ptr(seeds), seeds.numel(), _ptr(num_seeds_dev), _ptr(neighbors),
+                                       neighbors.numel(), int(neighbor_stride), int(bool(continued)), _ptr(self.table),
+                                       self.table_len, _ptr(unique), _ptr(relabeled), _ptr(num_unique_dev),
+                                       _ptr(num_outside_dev), None, _ptr(self.workspace), self.workspace.numel(),
+                                       _stream()))
+
+    def relabel(self, seeds, neighbors, continued=None):
+        seeds, neighbors = _dev_i64(seeds, "seeds"), _dev_i64(neighbors, "neighbors")
+        ns, nn = seeds.numel(), neighbors.numel()
+        self._workspace_for(ns + nn, seeds.device)
+        if continued is None:
+            continued = self._last == (seeds.data_ptr(), ns, seeds._version)
+        unique = torch.empty(ns + nn, dtype=torch.int64, device=seeds.device)
+        relabeled = torch.empty(nn, dtype=torch.int64, device=seeds.device)
+        host = (C.c_int64 * 2)(-1, -1)
+        self._last = None
+        self.counts.zero_()
+        check(lib().apt_relabel_ranked(_ptr(seeds), ns, None, _ptr(neighbors), nn, 0, int(bool(continued)),
+                                       _ptr(self.table), self.table_len, _ptr(unique), _ptr(relabeled),
+                                       _ptr(self.counts[0:1]), _ptr(self.counts[1:2]), host,
+                                       _ptr(self.workspace), self.workspace.numel(), _stream()))
+        if host[1] != 0:
+            raise AptError(f"relabel_ranked: {host[1]} ids are outside [0, {self.table_len})")
+        unique = unique[:host[0]]
+        self._last, self._last_tensor = (unique.data_ptr(), unique.numel(), unique._version), unique
+        return unique, relabeled, int(host[0])
 
 
 def gather_rows(store, index, num_index_dev=None, out=None, miss_count=None, pending=None):

@@ -26,6 +26,8 @@ static int g_sample_max_blocks = 0;
 int tuning_sample_max_blocks() { return g_sample_max_blocks; }
 static int g_sample_min_workgroups = 0;
 int tuning_sample_min_workgroups() { return g_sample_min_workgroups; }
+static int g_sample_direct_rows = 0;
+int tuning_sample_direct_rows() { return g_sample_direct_rows; }
 static int g_gather_vector_bytes = 0;
 int tuning_gather_vector_bytes() { return g_gather_vector_bytes; }
 static int g_gather_store_policy = 0;
@@ -74,6 +76,12 @@ extern "C" int apt_set_tuning(const char* key, int value) {
   if (std::strcmp(key, "sample_min_workgroups") == 0) {
     if (value < 0) return apt::fail(APT_EINVAL, "apt_set_tuning: sample_min_workgroups must be >= 0");
     apt::g_sample_min_workgroups = value;
+    return APT_OK;
+  }
+  if (std::strcmp(key, "sample_direct_rows") == 0) {
+    if (value != 0 && value != 1 && value != 2 && value != 4)
+      return apt::fail(APT_EINVAL, "apt_set_tuning: sample_direct_rows must be 0, 1, 2 or 4");
+    apt::g_sample_direct_rows = value;
     return APT_OK;
   }
   if (std::strcmp(key, "gather_vector_bytes") == 0) {

@@ -78,6 +78,10 @@ struct HopParams {
   uint64_t* flags;           // owner bit per item, one word per wavefront-load
   uint32_t* tile_cnt;
   uint8_t* displaced;        // per slot: a smaller bid took the node over (rank_table.hpp)
+  int64_t nn_fixed;          // >= 0: the number of neighbour slots, where it is not rows x fanout (apt_relabel_ranked)
+  int64_t* outside;          // optional: counts the ids that the table cannot hold (>= table_len)
+  int mark_seeds;            // the marking pass of the first hop also lets the seeds bid (no pass of their own)
+  const int64_t* prefix_src; // the marking pass of a later hop also copies these ns ids to the head of `nodes`
 };
 
 struct HopSizes {
@@ -87,7 +91,7 @@ struct HopSizes {
 __device__ __forceinline__ HopSizes hop_sizes(const HopParams& p) {
   HopSizes s;
   s.ns = actual_count(p.ns_cap, p.ns_dev);
-  s.nn = s.ns * p.fanout;
+  s.nn = p.nn_fixed >= 0 ? p.nn_fixed : s.ns * p.fanout;
   return s;
 }
 
@@ -136,9 +140,11 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_seeds_kernel(HopParams p, in
                                                                  int num_sizes) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x;
   if (i < num_sizes) sizes[i] = i == 0 ? p.ns_cap : 0;
-  if (i < p.ns_cap) {
+  if (i < actual_count(p.ns_cap, p.ns_dev)) {
     const int64_t v = p.seeds[i];
     if (in_table(p, v)) atomicMin(&p.table[v], table_base(p.state) + static_cast<uint32_t>(i));
+    else if (p.outside != nullptr && v >= p.table_len)
+      atomicAdd(reinterpret_cast<unsigned long long*>(p.outside), 1ull);
   }
 }
 
@@ -149,9 +155,26 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p
   const HopSizes s = hop_sizes(p);
   const RankEpoch ep = rank_epoch(p.state);
   const RankTable t{p.table, p.table_len, p.state, p.displaced};
-  for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < s.nn;
-       j += static_cast<int64_t>(gridDim.x) * kMbBlock)
-    p.relabeled[j] = rank_table_bid(t, ep, FIRST, p.neighbors[j], s.ns, j);
+  const bool with_rows = FIRST ? p.mark_seeds != 0 : p.prefix_src != nullptr;
+  const int64_t work = with_rows && s.ns > s.nn ? s.ns : s.nn;
+  for (int64_t j = static_cast<int64_t>(blockIdx.x) * kMbBlock + threadIdx.x; j < work;
+       j += static_cast<int64_t>(gridDim.x) * kMbBlock) {
+    if (j < s.nn) {
+      const int64_t v = p.neighbors[j];
+      p.relabeled[j] = rank_table_bid(t, ep, FIRST, v, s.ns, j);
+      if (p.outside != nullptr && v >= p.table_len) atomicAdd(reinterpret_cast<unsigned long long*>(p.outside), 1ull);
+    }
+    if (with_rows && j < s.ns) {
+      if (FIRST) {
+        const int64_t v = p.seeds[j];
+        if (in_table(p, v)) atomicMin(&p.table[v], ep.base + static_cast<uint32_t>(j));
+        else if (p.outside != nullptr && v >= p.table_len)
+          atomicAdd(reinterpret_cast<unsigned long long*>(p.outside), 1ull);
+      } else {
+        p.nodes[j] = p.prefix_src[j];
+      }
+    }
+  }
 }
 
 // Item i of a hop: FIRST -> seeds followed by neighbours (index = bid);
@@ -429,6 +452,10 @@ static int minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_
   }
 
   HopParams hp{};
+  hp.nn_fixed = -1;
+  hp.outside = nullptr;
+  hp.mark_seeds = 0;
+  hp.prefix_src = nullptr;
   hp.table = static_cast<uint32_t*>(rank_table);
   hp.table_len = rank_table_len;
   hp.state = state;
@@ -560,5 +587,161 @@ extern "C" int apt_minibatch_lookup(const apt_pending_lookup* pending, void* str
   hipLaunchKernelGGL(mb_lookup_kernel, dim3(q->blocks), dim3(kLookupBlock), 0, static_cast<hipStream_t>(stream),
                      q->lp);
   APT_LAUNCH_CHECK("mb_lookup_kernel");
+  return APT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// apt_relabel_ranked: apt_relabel's result through a node-indexed rank table
+// instead of a hash table, for ids that index a registered graph.  It is one hop
+// of the driver above called on its own (reference python/npc/sampler.py:187-203
+// calls relabel_csc once per hop, src/relabel.cc:9-15):
+//   a fresh call     seeds and neighbours bid with their positions (the first-hop
+//                    path: ownership is read back from the table);
+//   a continued call the seeds are exactly the unique list the previous call
+//                    returned, so the table still holds their ids: a neighbour
+//                    already in the batch costs one load, the others bid with an
+//                    atomicMin that settles ownership (the later-hop path).
+namespace apt {
+constexpr uint32_t kRankedPayloadBits = 24;  // fixed, so that calls of any size share a table without refills
+constexpr int64_t kRankedMaxItems = (int64_t{1} << kRankedPayloadBits) - 2;
+
+struct RankedLayout {
+  size_t flags_off, tile_off, displaced_off, total;
+};
+static RankedLayout ranked_layout(int64_t items) {
+  RankedLayout L;
+  const int64_t tiles = ceil_div(std::max<int64_t>(items, 1), kMbTile);
+  size_t off = 0;
+  L.flags_off = off; off = mb_align(off + sizeof(uint64_t) * tiles * kMbIters * kMbWaves);
+  L.tile_off = off;  off = mb_align(off + sizeof(uint32_t) * tiles);
+  L.displaced_off = off; off = mb_align(off + static_cast<size_t>(std::max<int64_t>(items, 1)));
+  L.total = off;
+  return L;
+}
+}  // namespace apt
+
+extern "C" int64_t apt_relabel_ranked_max_items(void) { return apt::kRankedMaxItems; }
+
+extern "C" size_t apt_relabel_ranked_workspace_bytes(int64_t num_items) {
+  if (num_items < 0 || num_items > apt::kRankedMaxItems) return 0;
+  return apt::ranked_layout(num_items).total;
+}
+
+extern "C" int apt_relabel_ranked(const int64_t* seeds, int64_t num_seeds, const int64_t* num_seeds_dev,
+                                  const int64_t* neighbors, int64_t num_neighbors, int64_t neighbor_stride,
+                                  int continued, void* rank_table, int64_t rank_table_len,
+                                  int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev, int64_t* num_outside_dev,
+                                  int64_t* counts_host, void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(num_seeds >= 0 && num_neighbors >= 0, APT_EINVAL, "apt_relabel_ranked: negative size");
+  APT_REQUIRE(num_seeds_dev == nullptr || (neighbor_stride > 0 && num_seeds <= num_neighbors / neighbor_stride),
+              APT_EINVAL, "apt_relabel_ranked: with num_seeds_dev, neighbors must hold num_seeds * neighbor_stride entries");
+  const int64_t items = num_seeds + num_neighbors;
+  APT_REQUIRE(items <= kRankedMaxItems, APT_ELIMIT, "apt_relabel_ranked: %lld items exceed the supported maximum %lld",
+              (long long)items, (long long)kRankedMaxItems);
+  APT_REQUIRE(rank_table != nullptr && rank_table_len > 0 && rank_table_len < (int64_t{1} << 32) - 1 &&
+                  (reinterpret_cast<uintptr_t>(rank_table) & 255) == 0,
+              APT_EINVAL, "apt_relabel_ranked: rank table missing, misaligned or too long");
+  APT_REQUIRE(num_unique_dev != nullptr && num_outside_dev != nullptr, APT_EINVAL,
+              "apt_relabel_ranked: num_unique_dev / num_outside_dev is NULL");
+  APT_REQUIRE((num_seeds == 0 || seeds != nullptr) && (num_neighbors == 0 || (neighbors != nullptr && relabeled != nullptr)) &&
+                  (items == 0 || unique != nullptr),
+              APT_EINVAL, "apt_relabel_ranked: seeds / neighbors / unique / relabeled is NULL");
+  APT_REQUIRE(workspace != nullptr && workspace_bytes >= ranked_layout(items).total &&
+                  (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
+              APT_EWORKSPACE, "apt_relabel_ranked: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace_bytes,
+              ranked_layout(items).total);
+  // The parts of the workspace are laid out for the largest call it can hold, not for this call: the per-slot
+  // flags must be all zero when a call starts (each call clears the ones it sets), so they must not share
+  // their bytes with another call's tile counts.
+  int64_t lo = items, hi = kRankedMaxItems;
+  while (lo < hi) {
+    const int64_t mid = lo + (hi - lo + 1) / 2;
+    if (ranked_layout(mid).total <= workspace_bytes) lo = mid;
+    else hi = mid - 1;
+  }
+  const RankedLayout L = ranked_layout(lo);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char* ws = static_cast<char*>(workspace);
+  uint32_t* state = reinterpret_cast<uint32_t*>(static_cast<char*>(rank_table) + table_state_offset(rank_table_len));
+  auto grid_for = [](int64_t n, int64_t per_block, int64_t cap) {
+    return dim3(static_cast<unsigned>(std::max<int64_t>(1, std::min<int64_t>(ceil_div(n, per_block), cap))));
+  };
+  HopParams hp{};
+  hp.table = static_cast<uint32_t*>(rank_table);
+  hp.table_len = rank_table_len;
+  hp.state = state;
+  hp.nodes = unique;
+  hp.nodes_cap = items;
+  hp.flags = reinterpret_cast<uint64_t*>(ws + L.flags_off);
+  hp.tile_cnt = reinterpret_cast<uint32_t*>(ws + L.tile_off);
+  hp.displaced = reinterpret_cast<uint8_t*>(ws + L.displaced_off);
+  hp.seeds = seeds;
+  hp.ns_cap = num_seeds;
+  hp.ns_dev = num_seeds_dev;
+  hp.fanout = num_seeds_dev != nullptr ? neighbor_stride : 1;
+  hp.nn_fixed = num_seeds_dev != nullptr ? -1 : num_neighbors;   // device-side count: rows x stride slots
+  hp.neighbors = neighbors;
+  hp.relabeled = relabeled;
+  hp.n_next = num_unique_dev;
+  hp.outside = num_outside_dev;
+  hp.last = 0;
+  hp.mark_seeds = 1;
+  hp.prefix_src = nullptr;
+  const dim3 mark_grid = grid_for(std::max(num_neighbors, num_seeds), kMbBlock, 1 << 16);
+  if (continued == 0) {
+    // a new batch of the table: next epoch (refill when they have run out); *num_unique_dev = num_seeds for now
+    const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
+    hipLaunchKernelGGL(mb_begin_kernel, dim3(kBeginBlocks), dim3(kMbBlock), 0, st, static_cast<uint4*>(rank_table), vecs,
+                       state, kRankedPayloadBits, num_unique_dev, 1, num_seeds);
+    APT_LAUNCH_CHECK("mb_begin_kernel");
+    if (items > 0) {
+      hipLaunchKernelGGL(mb_mark_neighbors_kernel<true>, mark_grid, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+      const dim3 tiles = grid_for(items, kMbTile, int64_t{1} << 30);
+      hipLaunchKernelGGL(mb_count_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_count_kernel");
+      hipLaunchKernelGGL(mb_place_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_place_kernel");
+    }
+  } else {
+    // the seeds hold ids 0 .. num_seeds - 1 in the table's current epoch (the caller vouches for it); the marking
+    // pass also copies them to the head of the unique list
+    hp.prefix_src = unique != seeds ? seeds : nullptr;
+    hipLaunchKernelGGL(mb_mark_neighbors_kernel<false>, mark_grid, dim3(kMbBlock), 0, st, hp);
+    APT_LAUNCH_CHECK("mb_mark_neighbors_kernel");
+    const dim3 tiles = grid_for(num_neighbors, kMbTile, int64_t{1} << 30);
+    hipLaunchKernelGGL(mb_count_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+    APT_LAUNCH_CHECK("mb_count_kernel");
+    hipLaunchKernelGGL(mb_place_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+    APT_LAUNCH_CHECK("mb_place_kernel");
+  }
+  if (num_neighbors > 0) {
+    LookupParams lp{};
+    lp.num_hops = 1;
+    lp.table = static_cast<const uint32_t*>(rank_table);
+    lp.state = state;
+    lp.last_is_bid = 0;
+    lp.block_begin[0] = 0;
+    lp.neighbors[0] = neighbors;
+    lp.relabeled[0] = relabeled;
+    // the pass only needs the number of slots: rows x stride, or num_neighbors x 1
+    lp.ns_dev[0] = num_seeds_dev;
+    lp.ns_cap[0] = num_seeds_dev != nullptr ? num_seeds : num_neighbors;
+    lp.fanout[0] = num_seeds_dev != nullptr ? neighbor_stride : 1;
+    const int64_t nblocks = std::max<int64_t>(1, std::min<int64_t>(ceil_div(num_neighbors, kMbBlock), 2048));
+    lp.block_begin[1] = nblocks;
+    hipLaunchKernelGGL(mb_lookup_kernel, dim3(static_cast<unsigned>(nblocks)), dim3(kLookupBlock), 0, st, lp);
+    APT_LAUNCH_CHECK("mb_lookup_kernel");
+  }
+  if (counts_host != nullptr) {
+    if (num_outside_dev == num_unique_dev + 1) {  // neighbours in memory: one copy
+      APT_HIP(hipMemcpyAsync(counts_host, num_unique_dev, 2 * sizeof(int64_t), hipMemcpyDeviceToHost, st));
+    } else {
+      APT_HIP(hipMemcpyAsync(counts_host, num_unique_dev, sizeof(int64_t), hipMemcpyDeviceToHost, st));
+      APT_HIP(hipMemcpyAsync(counts_host + 1, num_outside_dev, sizeof(int64_t), hipMemcpyDeviceToHost, st));
+    }
+    APT_HIP(hipStreamSynchronize(st));
+  }
   return APT_OK;
 }

@@ -47,6 +47,7 @@ struct SampleParams {
   int64_t* counts;
   int64_t* total;
   int rows_per_group;
+  int direct;  // every lane group resolves its own rows (no staging of the tile in LDS, no workgroup barrier)
   // Optional fusion with the rank-table relabel of the multi-hop driver: every
   // sampled id is looked up / bid for in the rank table right after it is loaded.
   RankTable table;       // entries == NULL: plain sampling
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   // frontier -> (pos_map ->) indptr loads of the whole tile overlap.  With one
   // row per group there is nothing to overlap: every group resolves its own row
   // (its lanes read the same addresses) and no group waits for another.
-  const bool direct = p.rows_per_group == 1 && p.fanout <= LPS;
+  const bool direct = p.direct != 0;
   __syncthreads();
   // The grid may be smaller than the number of tiles (it is capped when the row
   // count is only known on the device): a workgroup strides over the tiles.
@@ -327,6 +328,7 @@ static int launch_sample(const SampleParams& p, bool replace, int64_t blocks, si
 int tuning_sample_lanes();
 int tuning_sample_min_workgroups();  // 0 = default
 int tuning_sample_max_blocks();      // 0 = default
+int tuning_sample_direct_rows();     // 0 / 1 = one row per lane group in the unstaged shape
 
 }  // namespace apt
 
@@ -403,6 +405,15 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
   if (rpg < 1) rpg = 1;
   if (rpg > kMaxRowsPerGroup) rpg = kMaxRowsPerGroup;
   p.rows_per_group = static_cast<int>(rpg);
+  p.direct = rpg == 1 && fanout <= lps;
+  // Several rows per lane group in flight without the staging (knob sample_direct_rows, 2 or 4): the group
+  // issues the dependent loads of its rows back to back, so that the index loads and rank-table reads of one
+  // row overlap the atomics of another inside a group and not only between groups.
+  const int direct_rows = tuning_sample_direct_rows();
+  if (p.direct && (direct_rows == 2 || direct_rows == 4)) {
+    rpg = direct_rows;
+    p.rows_per_group = direct_rows;
+  }
   const int64_t tile = static_cast<int64_t>(groups) * rpg;
   int64_t blocks = ceil_div(num_frontier, tile);
   // With a device-side count num_frontier is an upper bound: a capped grid that

@@ -41,6 +41,13 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   uint64_t rng_seed = 7777777;  // reference src/cuda/npc_kernel.cu:292
   int64_t sample_calls = 0;
   bool strict = true;
+  // relabel_csc on a registered graph: a rank table of its own, a workspace that grows with the largest call, and
+  // the unique list the last call returned (kept alive so that its address cannot be reused) with its version
+  Tensor ranked_table, ranked_ws, ranked_counts, ranked_last;
+  uint32_t ranked_last_version = 0;
+  bool ranked_enabled = true;
+  // pinned host words that the relabel operators read their counts into (a copy to pageable memory is staged)
+  Tensor pinned_counts;
   // fused multi-hop driver: rank table of the registered graph, workspace of the last plan
   Tensor rank_table, mb_workspace;
   int64_t mb_batch = -1;
@@ -83,6 +90,13 @@ const int64_t* i64(const Tensor& t) { return t.defined() && t.numel() ? t.data_p
 
 torch::TensorOptions i64_opts() { return torch::TensorOptions().dtype(torch::kInt64).device(device()); }
 
+int64_t* pinned_counts() {
+  auto& s = S();
+  if (!s.pinned_counts.defined())
+    s.pinned_counts = torch::zeros({4}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+  return s.pinned_counts.data_ptr<int64_t>();
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------- registries
@@ -102,6 +116,13 @@ void SetRngSeed(IdType seed) {
 }
 
 void SetStrict(bool strict) { S().strict = strict; }
+
+// relabel_csc goes through the registered graph's rank table where it can (default) or always through the
+// hash table (false).
+void SetRankedRelabel(bool enabled) {
+  S().ranked_enabled = enabled;
+  S().ranked_last = Tensor();
+}
 
 // How many registry-owned sets of output buffers sample_blocks hands out in turn.  0 (the default) = fresh
 // tensors on every call.  With n > 0 a call costs less (no allocation), but what call k returned is
@@ -181,6 +202,8 @@ void MixCacheGraphs(IdType num_cached_nodes, Tensor cached_node_idx, Tensor cach
   s.graph.num_rows = total;
   s.graph.num_total_nodes = total;
   s.rank_table = Tensor();
+  s.ranked_table = Tensor();
+  s.ranked_last = Tensor();
   s.adj_pos_map = Tensor();
   if (num_cached_nodes > 0) {
     auto idx = ids_on_device(cached_node_idx, "cached_node_idx");
@@ -215,6 +238,8 @@ void RegisterGraphPartition(Tensor indptr, Tensor indices, IdType row_begin, IdT
   s.graph.num_rows = s.indptr.numel() - 1;
   s.graph.num_total_nodes = num_total_nodes;
   s.rank_table = Tensor();
+  s.ranked_table = Tensor();
+  s.ranked_last = Tensor();
   s.has_graph = true;
 }
 
@@ -425,22 +450,78 @@ std::vector<Tensor> LocalSamplingNeibhorsOneLayer(Tensor seeds, IdType fanout) {
   return {f, out};
 }
 
+// relabel_csc through the rank table of the registered graph (apt_relabel_ranked).  The reference's sampler calls
+// relabel_csc once per hop with seeds = the unique list of the hop before (python/npc/sampler.py:187-203): such a
+// call continues the batch, its seeds are already in the table.  -> false when an id does not fit the table (the
+// caller then takes the hash table).
+static bool RelabelRanked(const Tensor& sd, const Tensor& nb, Tensor& unique, Tensor& relabeled) {
+  auto& s = S();
+  const int64_t items = sd.numel() + nb.numel();
+  const int64_t len = s.graph.num_total_nodes;
+  auto u8 = torch::TensorOptions().dtype(torch::kUInt8).device(device());
+  if (!s.ranked_table.defined()) {
+    const size_t bytes = apt_rank_table_bytes(len);
+    if (bytes == 0) return false;
+    s.ranked_table = torch::empty({static_cast<int64_t>(bytes)}, u8);
+    check(apt_rank_table_init(s.ranked_table.data_ptr(), bytes, stream()));
+    s.ranked_counts = torch::zeros({2}, i64_opts());
+    s.ranked_last = Tensor();
+  }
+  const size_t need = apt_relabel_ranked_workspace_bytes(items);
+  if (!s.ranked_ws.defined() || static_cast<size_t>(s.ranked_ws.numel()) < need) {
+    s.ranked_ws = torch::empty({static_cast<int64_t>(std::max<size_t>(need, 256) * 2)}, u8);
+    check(apt_minibatch_workspace_init(s.ranked_ws.data_ptr(), static_cast<size_t>(s.ranked_ws.numel()), stream()));
+  }
+  const bool continued = s.ranked_last.defined() && s.ranked_last.data_ptr() == sd.data_ptr() &&
+                         s.ranked_last.numel() == sd.numel() && s.ranked_last_version == sd._version();
+  s.ranked_last = Tensor();
+  unique = torch::empty({items}, i64_opts());
+  relabeled = torch::empty({nb.numel()}, i64_opts());
+  int64_t* host = pinned_counts();
+  host[0] = host[1] = -1;
+  // ranked_counts[1] counts ids beyond the graph; it is zero unless the previous call found some
+  check(apt_relabel_ranked(i64(sd), sd.numel(), nullptr, i64(nb), nb.numel(), 0, continued ? 1 : 0,
+                           s.ranked_table.data_ptr(), len,
+                           unique.data_ptr<int64_t>(), nb.numel() ? relabeled.data_ptr<int64_t>() : nullptr,
+                           s.ranked_counts.data_ptr<int64_t>(), s.ranked_counts.data_ptr<int64_t>() + 1, host,
+                           s.ranked_ws.data_ptr(),
+                           static_cast<size_t>(s.ranked_ws.numel()), stream()));
+  if (host[1] != 0) {  // ids beyond the graph: not a valid relabel, and the table's batch is not continued
+    s.ranked_counts.zero_();
+    return false;
+  }
+  unique = unique.narrow(0, 0, host[0]);
+  s.ranked_last = unique;
+  s.ranked_last_version = unique._version();
+  return true;
+}
+
 // reference src/relabel.cc:9-15
 std::vector<Tensor> RelabelCSC(Tensor seeds, Tensor neighbors) {
+  auto& s = S();
   auto sd = ids_on_device(seeds, "seeds");
   auto nb = ids_on_device(neighbors, "neighbors");
   const int64_t items = sd.numel() + nb.numel();
+  // Small inputs: one workgroup with its table in LDS (inside apt_relabel).  Larger ones: the rank table of the
+  // registered graph, if there is one and the ids fit it; else the hash table in device memory.
+  if (s.has_graph && s.ranked_enabled && items > 8192 && items <= apt_relabel_ranked_max_items() &&
+      s.graph.num_total_nodes > 0) {
+    Tensor unique, relabeled;
+    if (RelabelRanked(sd, nb, unique, relabeled)) return {unique, relabeled};
+  }
+  s.ranked_last = Tensor();
   const size_t need = apt_relabel_workspace_bytes(items);
   TORCH_CHECK(need > 0, "npc: relabel_csc: ", items, " items exceed the supported maximum");
   auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));
   auto unique = torch::empty({items}, i64_opts());
   auto relabeled = torch::empty({nb.numel()}, i64_opts());
   auto count = torch::empty({1}, i64_opts());
-  int64_t host_count = -1;
+  int64_t* host_count = pinned_counts();
+  *host_count = -1;
   check(apt_relabel(i64(sd), sd.numel(), nullptr, i64(nb), nb.numel(), 0, unique.data_ptr<int64_t>(),
-                    relabeled.data_ptr<int64_t>(), count.data_ptr<int64_t>(), &host_count,
+                    relabeled.data_ptr<int64_t>(), count.data_ptr<int64_t>(), host_count,
                     ws.data_ptr(), need, stream()));
-  return {unique.narrow(0, 0, host_count), relabeled};
+  return {unique.narrow(0, 0, *host_count), relabeled};
 }
 
 // reference src/load_subtensor.cc:19-40
@@ -748,6 +829,7 @@ TORCH_LIBRARY(npc, m) {
       .def("set_topology", &SetTopology)
       .def("set_rng_seed", &SetRngSeed)
       .def("set_strict", &SetStrict)
+      .def("set_ranked_relabel", &SetRankedRelabel)
       .def("set_block_buffer_ring", &SetBlockBufferRing)
       .def("block_buffer_ring", &BlockBufferRing);
 }

@@ -64,6 +64,12 @@ def set_strict(strict: bool) -> None:
     _npc.set_strict(strict)
 
 
+def set_ranked_relabel(enabled: bool) -> None:
+    """True (default): relabel_csc on a registered graph goes through the graph's rank table (and continues the
+    batch when its seeds are the unique list the previous call returned); False: always the hash table."""
+    _npc.set_ranked_relabel(bool(enabled))
+
+
 def set_block_buffer_ring(sets: int) -> None:
     """0 (default): sample_blocks returns fresh tensors on every call, as the reference's operators do.
     n > 0: it hands out n registry-owned sets of output buffers in turn, which saves the allocations, but

@@ -22,7 +22,7 @@ from . import capi
 
 class MiniBatchPipeline:
     def __init__(self, graph, feat, batch_size, hop_fanouts, replace=False, gather=True, fused=True,
-                 use_graph=False, requests=None, formats=False, defer_lookup=False, table=None):
+                 use_graph=False, requests=None, formats=False, defer_lookup=False, table=None, relabel="hash"):
         """hop_fanouts: fanout per hop starting from the seeds (the reference's
         --fan_out list reversed).
 
@@ -38,6 +38,9 @@ class MiniBatchPipeline:
         ride in the launch of the gather that follows it instead of launching it before: 3-5 % less time per
         batch, while that launch gets 2-3 us longer (it is no longer the gather alone).  Only where the gather
         is what follows the sampling (fused driver, features gathered, no requests, no formats).
+
+        relabel (per-hop driver, fused=False): "hash" = apt_relabel's hash table per hop; "ranked" =
+        apt_relabel_ranked, the per-hop calls through a node-indexed rank table, later hops continuing the batch.
 
         table: the rank table of another pipeline (fused driver) whose batches run on the same stream as this
         one's: batches that follow each other on one stream can share a table (444 MB at 111 M nodes).
@@ -70,6 +73,10 @@ class MiniBatchPipeline:
             self.frontier = [None] + [torch.empty(self.caps[h + 1], **i64) for h in range(H)]
             # sizes[h] = rows of the frontier entering hop h; sizes[H] = input nodes; then edges
             self.sizes = torch.zeros(H + 2, **i64)
+            if relabel not in ("hash", "ranked"):
+                raise ValueError("relabel must be 'hash' or 'ranked'")
+            self.ranked = capi.RankedRelabel(graph.num_total_nodes, dev) if relabel == "ranked" else None
+            self.ranked_outside = torch.zeros(1, **i64)    # ids the rank table cannot hold (stays 0 for a valid graph)
             self.workspace = torch.empty(capi.relabel_workspace_bytes(self.caps[-1]), dtype=torch.uint8,
                                          device=dev)
         self.features = None
@@ -124,6 +131,10 @@ class MiniBatchPipeline:
             capi.sample_neighbors(self.graph, self.frontier[h], f, self.replace, rng_seed, h,
                                   num_frontier_dev=n_dev, out_neighbors=self.neighbors[h],
                                   out_counts=self.counts[h], out_total=total)
+            if self.ranked is not None:
+                self.ranked.enqueue(self.frontier[h], self.neighbors[h], h > 0, self.frontier[h + 1], self.relabeled[h],
+                                    self._size(h + 1), self.ranked_outside, num_seeds_dev=n_dev, neighbor_stride=f)
+                continue
             capi.relabel(self.frontier[h], self.neighbors[h], num_seeds_dev=n_dev, neighbor_stride=f,
                          unique=self.frontier[h + 1], relabeled=self.relabeled[h],
                          num_unique_dev=self._size(h + 1), workspace=self.workspace, sync=False)

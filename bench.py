@@ -76,9 +76,11 @@ def parse_args():
                     help="seconds of CPU-oracle work for the cpu_baseline leg (0 = skip, also skips its parity check)")
     ap.add_argument("--cpu_threads", type=int, default=None)
     ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused"],
+    ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused", "unfused_hash"],
                     help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
-                         "unfused: per-hop sample + relabel calls")
+                         "unfused: the reference's call pattern, a sampling call and a relabel call per hop, the "
+                         "relabel through the graph's rank table (apt_relabel_ranked); unfused_hash: the same with the "
+                         "hash-table relabel (apt_relabel)")
     ap.add_argument("--inflight", type=int, default=4,
                     help="after the timed single-stream region, also run the K batches with N of them in "
                          "flight (N pipelines on N HIP streams) and report it under stages.in_flight; 1 = skip")
@@ -231,6 +233,13 @@ def build_workload(args, name, w, ctx, full_graph=None):
     return wl
 
 
+def driver_kw(args):
+    """MiniBatchPipeline arguments of --driver."""
+    if args.driver in ("fused", "graph"):
+        return dict(fused=True)
+    return dict(fused=False, relabel="ranked" if args.driver == "unfused" else "hash")
+
+
 def make_seed_sets(ctx, wl, B, count, seed):
     torch, dev = ctx.torch, ctx.dev
     gen = torch.Generator(device=dev)
@@ -251,8 +260,8 @@ def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True):
     from apt_amd.pipeline import MiniBatchPipeline
 
     def make_pipe(use_graph):
-        return MiniBatchPipeline(wl.graph, wl.store, B, hops, replace=args.replace, fused=args.driver != "unfused",
-                                 use_graph=use_graph, requests=wl.requests, defer_lookup=args.defer_lookup == "on")
+        return MiniBatchPipeline(wl.graph, wl.store, B, hops, replace=args.replace, use_graph=use_graph,
+                                 requests=wl.requests, defer_lookup=args.defer_lookup == "on", **driver_kw(args))
 
     m = SimpleNamespace(make_pipe=make_pipe, B=B, hops=hops, K=K, W=W)
     pipe = m.pipe = make_pipe(args.driver == "graph")
@@ -442,8 +451,8 @@ def stage_target_shape(args, ctx, wl, hops, store_of):
         store = store_of(name)
         esize = store.local_table.element_size()
         moved, spec = gather_bytes_per_row(store.out_dim, esize, store.pos_map is not None)
-        pipe = MiniBatchPipeline(wl.graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused",
-                                 defer_lookup=args.defer_lookup == "on")
+        pipe = MiniBatchPipeline(wl.graph, store, B, hops, replace=args.replace, defer_lookup=args.defer_lookup == "on",
+                                 **driver_kw(args))
         pool = torch.randperm(wl.seed_n, generator=gen, device=dev)[:(Kt + Wt) * B]
         sets = [pool[i * B:(i + 1) * B].contiguous() for i in range(Kt + Wt)]
         log = torch.zeros((Kt, H + 2), dtype=torch.int64, device=dev)

@@ -309,7 +309,8 @@ def stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, see
     touched = sorted({k for _, knobs in settings for k in knobs})
     default_of = lambda k: TUNING_DEFAULTS.get(k, 0)
     H, NB = len(hops), 40
-    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=args.driver != "unfused")
+    pipe = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, fused=not args.driver.startswith("unfused"),
+                             relabel="hash" if args.driver == "unfused_hash" else "ranked")
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.seed + 31)
     pool = seed_lo + torch.randperm(seed_n, generator=gen, device=dev)[:NB * B]

@@ -63,6 +63,8 @@ int apt_abi_version(void);
  *   "sample_lanes_per_row"   8|16|32|64 lanes of a wavefront per frontier row
  *   "sample_min_workgroups"  workgroups a sampling launch must have before a lane
  *                            group is given more than one row
+ *   "sample_direct_rows"     1|2|4 rows a lane group of the sampler has in flight where the launch is
+ *                            too small to give a group several rows through the LDS-staged path
  *   "gather_rows_in_flight"  1|2|4|8 rows a lane group loads before storing
  *   "gather_max_blocks"      cap on the gather grid (rows are strided over)
  *   "gather_vector_bytes"    2|4|8|16: widest load/store a lane of the gather uses
@@ -168,6 +170,45 @@ int apt_relabel(const int64_t* seeds, int64_t num_seeds,
                 int64_t* unique, int64_t* relabeled, int64_t* num_unique_dev,
                 int64_t* num_unique_host, void* workspace,
                 size_t workspace_bytes, void* stream);
+
+/* apt_relabel's result through a node-indexed rank table instead of a hash table,
+ * for callers whose ids index a known range [0, rank_table_len) (the nodes of a
+ * registered graph): no probing, no fill pass per call, and nodes already in the
+ * batch cost one load.  Same reference interface as apt_relabel (relabel_csc,
+ * src/relabel.cc:9-15, called once per hop by python/npc/sampler.py:187-203).
+ *   rank_table    as in apt_minibatch_sample (apt_rank_table_bytes /
+ *                 apt_rank_table_init), but a table of its own: entries are laid
+ *                 out for up to apt_relabel_ranked_max_items() items per call
+ *   num_seeds_dev, neighbor_stride   as in apt_relabel
+ *   continued     0: a fresh relabel of cat(seeds, neighbors).
+ *                 != 0: the caller vouches that seeds[0 .. num_seeds) is exactly
+ *                 the unique list that the previous call on this table wrote
+ *                 (same values, same order, no other call on the table since):
+ *                 the table still holds their ids, so only the neighbours are
+ *                 looked up or bid for.  The result is what a fresh call gives.
+ *   unique        device int64[num_seeds + num_neighbors] capacity
+ *   num_unique_dev   device int64[1], receives the number of unique ids
+ *   num_outside_dev  device int64[1], incremented once per id that the table
+ *                 cannot hold (>= rank_table_len); the caller clears it.  When
+ *                 it is not zero afterwards the outputs are not a valid relabel
+ *                 (such ids were treated as padding) and the caller falls back
+ *                 to apt_relabel
+ *   counts_host   optional host int64[2]; when not NULL the call synchronises
+ *                 the stream and stores the two counters there
+ *   workspace     apt_relabel_ranked_workspace_bytes(num_seeds + num_neighbors)
+ *                 bytes, 16-byte aligned, zeroed once with
+ *                 apt_minibatch_workspace_init (a larger one may be reused for
+ *                 smaller calls; calls leave it ready for the next one)
+ * Negative ids are padding, as in apt_relabel. */
+int64_t apt_relabel_ranked_max_items(void);
+size_t apt_relabel_ranked_workspace_bytes(int64_t num_items);
+int apt_relabel_ranked(const int64_t* seeds, int64_t num_seeds, const int64_t* num_seeds_dev,
+                       const int64_t* neighbors, int64_t num_neighbors, int64_t neighbor_stride,
+                       int continued, void* rank_table,
+                       int64_t rank_table_len, int64_t* unique, int64_t* relabeled,
+                       int64_t* num_unique_dev, int64_t* num_outside_dev,
+                       int64_t* counts_host, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 /* apt_relabel without a workspace argument and without any allocation.
  * No counterpart in the reference.  It is for callers that cannot allocate:

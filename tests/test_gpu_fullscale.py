@@ -290,8 +290,10 @@ def test_full_scale_properties(capi, full, replace):
 
 def test_fused_and_per_hop_drivers_agree_over_many_batches(capi):
     """Three hundred batches on the 2.4 M-node graph: the fused driver (rank table, bids inside
-    the sampling kernel) and the per-hop driver (hash table) are two implementations of the same
-    first-occurrence relabel and must agree bit for bit, whatever the scheduling of a batch was."""
+    the sampling kernel), the per-hop driver with the hash table and the per-hop driver with the rank
+    table (apt_relabel_ranked, later hops continuing the batch; its 8-bit epoch field runs out and the
+    table is refilled on the way) are three implementations of the same first-occurrence relabel and
+    must agree bit for bit, whatever the scheduling of a batch was."""
     from apt_amd import synth
     from apt_amd.pipeline import MiniBatchPipeline
     N = 2_400_000
@@ -300,14 +302,19 @@ def test_fused_and_per_hop_drivers_agree_over_many_batches(capi):
     hops = [5, 10, 15]
     fused = MiniBatchPipeline(graph, None, 1024, hops, gather=False)
     per_hop = MiniBatchPipeline(graph, None, 1024, hops, gather=False, fused=False)
+    ranked = MiniBatchPipeline(graph, None, 1024, hops, gather=False, fused=False, relabel="ranked")
     gen = torch.Generator(device=DEV)
     gen.manual_seed(21)
     for batch in range(300):
         seeds = torch.randint(0, N, (1024,), generator=gen, device=DEV)          # repeated seeds happen
         fused.run(seeds, 9000 + batch)
         per_hop.run(seeds, 9000 + batch)
-        a, b = fused.result(), per_hop.result()
-        assert a["sizes"] == b["sizes"], batch
-        assert torch.equal(a["input_nodes"], b["input_nodes"]), batch
-        for x, y in zip(a["blocks"], b["blocks"]):
-            assert torch.equal(x["relabeled"], y["relabeled"]) and torch.equal(x["neighbors"], y["neighbors"]), batch
+        ranked.run(seeds, 9000 + batch)
+        a = fused.result()
+        for other in (per_hop, ranked):
+            b = other.result()
+            assert a["sizes"] == b["sizes"], batch
+            assert torch.equal(a["input_nodes"], b["input_nodes"]), batch
+            for x, y in zip(a["blocks"], b["blocks"]):
+                assert torch.equal(x["relabeled"], y["relabeled"]) and torch.equal(x["neighbors"], y["neighbors"]), batch
+        assert int(ranked.ranked_outside) == 0

@@ -56,6 +56,36 @@ def test_sampling_random_graph_all_lane_groups(orc, capi, lanes, replace):
         capi.set_tuning("sample_lanes_per_row", 0)
 
 
+@pytest.mark.parametrize("direct_rows", [2, 4])
+def test_sampling_several_unstaged_rows_per_group(orc, capi, direct_rows):
+    """Lane groups that resolve two or four rows themselves (no LDS staging): same rows as one row per group,
+    alone and inside the fused driver with its rank-table bids."""
+    from apt_amd.pipeline import MiniBatchPipeline
+    indptr, indices = small_graph(20000, 30, seed=23)
+    og, dg = _graphs(orc, capi, indptr, indices)
+    frontier = np.random.default_rng(6).integers(0, 20000, size=30011)
+    cnt = torch.tensor([25003], dtype=torch.int64, device=DEV)
+    capi.set_tuning("sample_direct_rows", direct_rows)
+    try:
+        for fanout, replace in [(15, False), (7, True), (5, False)]:
+            want_n, want_c = orc.sample_neighbors(og, frontier[:25003], fanout, replace, 9, 1)
+            got_n, got_c = capi.sample_neighbors(dg, dev(frontier), fanout, replace, 9, 1, num_frontier_dev=cnt)
+            assert np.array_equal(host(got_c)[:25003], want_c)
+            assert np.array_equal(host(got_n)[:25003 * fanout], want_n)
+        pipe = MiniBatchPipeline(dg, None, 512, [5, 10, 15], gather=False)
+        for batch in range(3):
+            seeds = np.random.default_rng(batch).integers(0, 20000, size=512)
+            pipe.run(dev(seeds), 40 + batch)
+            res = pipe.result()
+            want_in, want_blocks = orc.sample_blocks(og, seeds, [5, 10, 15], False, 40 + batch)
+            assert np.array_equal(host(res["input_nodes"]), want_in)
+            for got, want in zip(res["blocks"], want_blocks):
+                for k in ("neighbors", "relabeled", "counts"):
+                    assert np.array_equal(host(got[k]), want[k]), k
+    finally:
+        capi.set_tuning("sample_direct_rows", 0)
+
+
 @pytest.mark.parametrize("min_wg,max_blocks", [(0, 7), (1, 5), (3, 0), (1, 0)])
 def test_sampling_launch_shapes(orc, capi, min_wg, max_blocks):
     """A small grid striding over many tiles, several rows per lane group (rows
@@ -181,6 +211,77 @@ def test_relabel_specials(orc, capi):
     hubs = rng.integers(0, 50, size=300000)
     tail = rng.integers(0, 5_000_000, size=300000)
     _relabel_case(orc, capi, rng.permutation(5_000_000)[:4096], rng.permutation(np.concatenate([hubs, tail])))
+
+
+def test_relabel_ranked_fresh_and_continued(orc, capi):
+    """apt_relabel_ranked (node-indexed rank table) against the oracle: fresh calls with repeated seeds, padding,
+    heavy duplication, ids at the table's end; chains of calls where each call's seeds are the unique list of the
+    one before (the reference's per-hop pattern), which continue the batch in the table; ids beyond the table."""
+    rng = np.random.default_rng(3)
+    N = 2_000_000
+    rr = capi.RankedRelabel(N, DEV)
+    e = np.array([], dtype=np.int64)
+    cases = [(np.array([5, 9, 7]), e), (e, np.array([3, 3, 1, 3])), (e, e), (np.array([4]), np.full(5000, 4)),
+             (np.array([2, 2, 8, 2]), np.array([8, 1, 2, 1])), (np.array([3, 1]), np.array([1, -1, 7, -1, 3])),
+             (np.array([N - 1, 0, N - 2]), rng.integers(N - 50, N, 640)),
+             (rng.permutation(N)[:4096], rng.permutation(np.concatenate([rng.integers(0, 50, 300000),
+                                                                         rng.integers(0, N, 300000)]))),
+             (rng.integers(0, 1000, 3000), np.where(rng.random(50000) < 0.2, -1, rng.integers(0, 3000, 50000)))]
+    for seeds, nbrs in cases + cases[:3]:                        # again: the table is reused without clearing
+        seeds, nbrs = np.asarray(seeds, np.int64), np.asarray(nbrs, np.int64)
+        u, r, n = rr.relabel(dev(seeds), dev(nbrs))
+        want_u, want_r = orc.relabel(seeds, nbrs)
+        assert n == len(want_u) and np.array_equal(host(u), want_u) and np.array_equal(host(r), want_r)
+    # chains: hop h's seeds are hop h-1's unique list
+    for chain in range(4):
+        frontier = dev(rng.integers(0, N, 700))                  # repeated seeds happen
+        first = True
+        for f in (5, 10, 15):
+            nbrs = np.where(rng.random(frontier.numel() * f) < 0.1, -1, rng.integers(0, N if chain % 2 else 30000,
+                                                                                      frontier.numel() * f))
+            want_u, want_r = orc.relabel(host(frontier), nbrs)
+            assert first or rr._last == (frontier.data_ptr(), frontier.numel(), frontier._version)
+            u, r, n = rr.relabel(frontier, dev(nbrs))
+            assert n == len(want_u) and np.array_equal(host(u), want_u) and np.array_equal(host(r), want_r)
+            frontier, first = u, False
+    # a seeds tensor that was modified in place, or is another tensor with the same values, starts afresh
+    u, r, n = rr.relabel(dev(np.arange(100, 9100)), dev(rng.integers(0, N, 40000)))
+    v = u.clone()
+    nbrs = rng.integers(0, N, 60000)
+    want_u, want_r = orc.relabel(host(v), nbrs)
+    u2, r2, _ = rr.relabel(v, dev(nbrs))
+    assert np.array_equal(host(u2), want_u) and np.array_equal(host(r2), want_r)
+    u2[5:7] = u2[5:7].flip(0)                                    # in-place edit: the version changes
+    assert rr._last != (u2.data_ptr(), u2.numel(), u2._version)
+    want_u, want_r = orc.relabel(host(u2), nbrs)
+    u3, r3, _ = rr.relabel(u2, dev(nbrs))
+    assert np.array_equal(host(u3), want_u) and np.array_equal(host(r3), want_r)
+    # an id the table cannot hold is reported, not mislabelled
+    with pytest.raises(capi.AptError, match="outside"):
+        rr.relabel(dev(np.array([1, 2, N])), dev(np.array([3, 4])))
+    with pytest.raises(capi.AptError, match="outside"):
+        rr.relabel(dev(np.array([1, 2])), dev(np.array([3, N + 7, 4])))
+    u, r, n = rr.relabel(dev(np.array([1, 2])), dev(np.array([3, 2, 4])))     # and the table is usable afterwards
+    assert host(u).tolist() == [1, 2, 3, 4] and host(r).tolist() == [2, 1, 3]
+    # device-side count and stride (the per-hop driver's form), fresh and continued
+    cap, f, real = 5000, 5, 3210
+    seeds, nbrs = rng.permutation(100000)[:cap], rng.integers(0, 100000, size=cap * f)
+    cnt = torch.tensor([real], dtype=torch.int64, device=DEV)
+    uq = torch.full((cap * (f + 1),), -7, dtype=torch.int64, device=DEV)
+    rl = torch.full((cap * f,), -7, dtype=torch.int64, device=DEV)
+    counts = torch.zeros(2, dtype=torch.int64, device=DEV)
+    rr.enqueue(dev(seeds), dev(nbrs), False, uq, rl, counts[0:1], counts[1:2], num_seeds_dev=cnt, neighbor_stride=f)
+    want_u, want_r = orc.relabel(seeds[:real], nbrs[:real * f])
+    assert host(counts).tolist() == [len(want_u), 0]
+    assert np.array_equal(host(uq)[:len(want_u)], want_u) and np.array_equal(host(rl)[:real * f], want_r)
+    nb2 = rng.integers(0, 100000, size=uq.numel() * 3)
+    uq2 = torch.full((uq.numel() * 4,), -7, dtype=torch.int64, device=DEV)
+    rl2 = torch.full((uq.numel() * 3,), -7, dtype=torch.int64, device=DEV)
+    n1 = counts[0:1].clone()
+    rr.enqueue(uq, dev(nb2), True, uq2, rl2, counts[0:1], counts[1:2], num_seeds_dev=n1, neighbor_stride=3)
+    want_u2, want_r2 = orc.relabel(want_u, nb2[:len(want_u) * 3])
+    assert host(counts).tolist() == [len(want_u2), 0]
+    assert np.array_equal(host(uq2)[:len(want_u2)], want_u2) and np.array_equal(host(rl2)[:len(want_u) * 3], want_r2)
 
 
 def test_relabel_device_side_count(orc, capi):

@@ -109,6 +109,34 @@ def test_operator_layer_dp_sampler(orc, capi):
     assert np.array_equal(u.cpu().numpy(), seeds)
 
 
+def test_operator_relabel_csc_uses_the_rank_table_and_falls_back(orc, capi):
+    """relabel_csc on a registered graph: calls above the LDS size go through the graph's rank table, a call
+    whose seeds are the unique list of the call before continues that batch, ids the graph does not have make
+    the call take the hash table; all give the oracle's answer, as does the operator with the table switched off."""
+    import apt_amd as npc
+    indptr, indices, feats = _setup(orc, capi, n=50_000, dim=8, seed=6)
+    n = len(indptr) - 1
+    npc.set_topology(0, 1)
+    e = torch.empty(0, dtype=torch.int64)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
+    rng = np.random.default_rng(4)
+    try:
+        for ranked in (True, False, True):
+            npc.ops.set_ranked_relabel(ranked)
+            for chain in range(3):
+                frontier = dev(rng.integers(0, n, 3000))
+                for f in (4, 6, 5):
+                    nbrs = np.where(rng.random(frontier.numel() * f) < 0.05, -1, rng.integers(0, n, frontier.numel() * f))
+                    if chain == 2 and f == 6:
+                        nbrs[17] = n + 123                           # an id the registered graph does not have
+                    want_u, want_r = orc.relabel(frontier.cpu().numpy(), nbrs)
+                    u, r = npc.ops.tensor_relabel_csc(frontier, dev(nbrs))
+                    assert np.array_equal(u.cpu().numpy(), want_u) and np.array_equal(r.cpu().numpy(), want_r), (ranked, chain, f)
+                    frontier = u
+    finally:
+        npc.ops.set_ranked_relabel(True)
+
+
 def test_cpu_load_subtensor_rejects_ids_without_a_local_row(orc, capi):
     """Ids are checked on the host before anything is enqueued: a node outside the map, or one
     that has no local row (map entry -1, or a cache-only node), raises IndexError."""
