@@ -7,10 +7,14 @@
 // C ABI of libapt_hip.so (include/apt_amd.h) on the current HIP stream.
 // Operators whose reference implementation exchanges data with other GPUs
 // over NCCL are registered too, and raise.
+#include <ATen/hip/HIPEvent.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 #include <torch/torch.h>
 
+#include <deque>
+#include <memory>
+#include <string>
 #include <tuple>
 #include <vector>
 
@@ -40,7 +44,20 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   // sampling
   uint64_t rng_seed = 7777777;  // reference src/cuda/npc_kernel.cu:292
   int64_t sample_calls = 0;
-  bool strict = true;
+  // How load_subtensor reports requested nodes that have no row here (the reference reads out of bounds):
+  //   0 not at all (rows are zero-filled), 1 deferred (default): the miss counter travels to pinned host memory
+  //   behind the gather and is looked at by the next operator call or by check_errors(), so no call waits for
+  //   the GPU; 2 immediate: the call waits for its own counter and raises itself.
+  int miss_check = 1;
+  bool strict = true;   // feat_shuffle's pack checks permutations it did not produce itself
+  struct PendingCheck {
+    Tensor dev, host;
+    std::shared_ptr<at::cuda::CUDAEvent> done;
+  };
+  std::deque<PendingCheck> pending_checks;
+  // permutations handed out by shuffle_seeds / cluster_and_permute (kept alive, with their versions): bijections
+  // by construction, which feat_shuffle's pack need not check
+  std::deque<std::pair<Tensor, uint32_t>> own_permutations;
   // relabel_csc on a registered graph: a rank table of its own, a workspace that grows with the largest call, and
   // the unique list the last call returned (kept alive so that its address cannot be reused) with its version
   Tensor ranked_table, ranked_ws, ranked_counts, ranked_last;
@@ -115,7 +132,34 @@ void SetRngSeed(IdType seed) {
   S().sample_calls = 0;
 }
 
-void SetStrict(bool strict) { S().strict = strict; }
+// Looks at the miss counters of earlier load_subtensor calls that have arrived (wait: all of them) and raises for
+// the first that is not zero.
+void PollChecks(bool wait) {
+  auto& q = S().pending_checks;
+  while (!q.empty()) {
+    auto& p = q.front();
+    if (wait) p.done->synchronize();
+    else if (!p.done->query()) break;
+    const int64_t m = p.host.data_ptr<int64_t>()[0];
+    q.pop_front();
+    TORCH_CHECK_INDEX(m == 0, "npc: load_subtensor (an earlier call): ", m,
+                      " requested node(s) have no feature row on this GPU; their rows were zero-filled");
+  }
+}
+
+void CheckErrors() { PollChecks(true); }
+
+void SetStrict(bool strict) {
+  S().strict = strict;
+  S().miss_check = strict ? 1 : 0;
+}
+
+void SetMissCheck(std::string mode) {
+  TORCH_CHECK(mode == "off" || mode == "deferred" || mode == "immediate",
+              "npc: set_miss_check: 'off', 'deferred' or 'immediate'");
+  PollChecks(true);
+  S().miss_check = mode == "off" ? 0 : mode == "deferred" ? 1 : 2;
+}
 
 // relabel_csc goes through the registered graph's rank table where it can (default) or always through the
 // hash table (false).
@@ -528,16 +572,30 @@ std::vector<Tensor> RelabelCSC(Tensor seeds, Tensor neighbors) {
 Tensor LoadSubtensor(Tensor node_id) {
   auto& s = S();
   TORCH_CHECK(s.has_feat, "npc: no features registered (cache_feats_shared)");
+  PollChecks(false);
   auto idx = ids_on_device(node_id, "node_id");
   auto out = torch::empty({idx.numel(), s.feat.out_dim}, s.local_feats.options());
   Tensor miss;
-  if (s.strict) miss = torch::zeros({1}, i64_opts());
+  if (s.miss_check != 0) miss = torch::zeros({1}, i64_opts());
   check(apt_gather_rows(&s.feat, i64(idx), idx.numel(), nullptr, out.data_ptr(),
-                        s.strict ? miss.data_ptr<int64_t>() : nullptr, stream()));
-  if (s.strict) {
+                        s.miss_check != 0 ? miss.data_ptr<int64_t>() : nullptr, stream()));
+  if (s.miss_check == 2) {
     const int64_t m = miss.item<int64_t>();
     TORCH_CHECK_INDEX(m == 0, "npc: load_subtensor: ", m,
                       " requested node(s) have no feature row on this GPU");
+  } else if (s.miss_check == 1) {
+    // the counter follows the gather to pinned host memory; nobody waits for it here
+    State::PendingCheck p;
+    p.dev = miss;
+    p.host = torch::empty({1}, torch::TensorOptions().dtype(torch::kInt64).pinned_memory(true));
+    p.host.copy_(miss, /*non_blocking=*/true);
+    p.done = std::make_shared<at::cuda::CUDAEvent>();
+    p.done->record();
+    s.pending_checks.push_back(std::move(p));
+    if (s.pending_checks.size() > 64) {   // a caller that never lets one arrive: wait for the oldest
+      s.pending_checks.front().done->synchronize();
+      PollChecks(false);
+    }
   }
   return out;
 }
@@ -587,6 +645,9 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> ClusterAndPermuteLocal(Tensor seeds) 
                             node_beg + static_cast<int>(s.node_size), size.data_ptr<int64_t>(),
                             offset.data_ptr<int64_t>(), sorted.data_ptr<int64_t>(),
                             perm.data_ptr<int64_t>(), ws.data_ptr(), need, stream()));
+  auto& own = s.own_permutations;
+  own.emplace_back(perm, perm._version());
+  if (own.size() > 8) own.pop_front();
   return {size, offset, sorted, perm};
 }
 
@@ -674,7 +735,11 @@ Tensor FeatShuffle(Tensor inputs, Tensor send_offset, Tensor recv_offset, Tensor
                          torch::TensorOptions().dtype(torch::kUInt8).device(device()));
   check(apt_scatter_rows(x.data_ptr(), i64(perm), perm.numel(), feat_dim, static_cast<int>(x.element_size()),
                          out.data_ptr(), n_out, ws.data_ptr(), static_cast<size_t>(ws.numel()), stream()));
-  if (S().strict) {
+  bool own = false;   // a permutation this library produced is a bijection onto [0, n): nothing to check
+  for (const auto& p : S().own_permutations)
+    own |= p.first.data_ptr() == perm.data_ptr() && p.first.numel() == perm.numel() && p.second == perm._version() &&
+           perm.numel() == n_out;
+  if (S().strict && !own) {
     // The reference's pack is index_select_backward (src/feat_shuffle.cc:14-16): rows named more than once
     // add up.  The scatter keeps one of them, which is the same thing only for a permutation without
     // repeats (what ShuffleSeeds produces).  The flags tell: as many rows named as entries <=> no repeats and
@@ -829,6 +894,8 @@ TORCH_LIBRARY(npc, m) {
       .def("set_topology", &SetTopology)
       .def("set_rng_seed", &SetRngSeed)
       .def("set_strict", &SetStrict)
+      .def("set_miss_check", &SetMissCheck)
+      .def("check_errors", &CheckErrors)
       .def("set_ranked_relabel", &SetRankedRelabel)
       .def("set_block_buffer_ring", &SetBlockBufferRing)
       .def("block_buffer_ring", &BlockBufferRing);

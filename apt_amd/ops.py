@@ -59,9 +59,25 @@ def set_rng_seed(seed: int) -> None:
 
 
 def set_strict(strict: bool) -> None:
-    """strict (default): load_subtensor raises when a requested node has no row here, and the pack
-    direction of feat_shuffle checks its permutation (repeated entries add up, as in the reference)."""
+    """True (default): load_subtensor reports requested nodes that have no row here (see set_miss_check,
+    "deferred"), and the pack direction of feat_shuffle checks a permutation that shuffle_seeds did not produce
+    (repeated entries add up, as in the reference).  False: neither."""
     _npc.set_strict(strict)
+
+
+def set_miss_check(mode: str) -> None:
+    """How load_subtensor reports requested nodes without a feature row on this GPU (their rows are zero-filled;
+    the reference reads out of bounds):
+      "deferred" (default)  no call waits for the GPU: the miss counter follows the gather to pinned host memory
+                            and the next npc operator call, or check_errors(), raises IndexError for it;
+      "immediate"           load_subtensor waits for its own counter and raises itself;
+      "off"                 not reported."""
+    _npc.set_miss_check(mode)
+
+
+def check_errors() -> None:
+    """Waits for the deferred checks of earlier calls and raises IndexError if one of them failed."""
+    _npc.check_errors()
 
 
 def set_ranked_relabel(enabled: bool) -> None:

@@ -100,8 +100,30 @@ def test_operator_layer_dp_sampler(orc, capi):
     host_rows = npc.cpu_load_subtensor(input_nodes.cpu())
     assert host_rows.device.type == "cpu"                      # as the reference's CPU statement returns
     assert np.array_equal(host_rows.numpy(), feats[frontier])
+    # a requested node without a row: reported without a wait by default, that is by the next operator call or
+    # by check_errors(); by the call itself in "immediate" mode; not at all when switched off
+    rows = npc.load_subtensor(torch.tensor([0, n + 5]))
+    assert np.array_equal(rows.cpu().numpy()[0], feats[0]) and not rows[1].any()
+    with pytest.raises(IndexError, match="earlier call"):
+        npc.ops.check_errors()
+    npc.ops.check_errors()                                     # reported once
+    npc.load_subtensor(torch.tensor([n + 5]))
+    torch.cuda.synchronize()
+    with pytest.raises(IndexError, match="earlier call"):
+        npc.load_subtensor(torch.tensor([3]))                  # the next call reports it
+    npc.ops.check_errors()
+    npc.ops.set_miss_check("immediate")
     with pytest.raises(IndexError):
         npc.load_subtensor(torch.tensor([0, n + 5]))
+    npc.ops.set_miss_check("off")
+    npc.load_subtensor(torch.tensor([0, n + 5]))
+    npc.ops.check_errors()
+    npc.ops.set_miss_check("deferred")
+    for _ in range(100):                                       # many calls nobody checks: the queue stays bounded
+        npc.load_subtensor(dev(seeds))
+    npc.ops.check_errors()
+    with pytest.raises(RuntimeError):
+        npc.ops.set_miss_check("sometimes")
     with pytest.raises(RuntimeError):
         npc.np_sample_and_shuffle(dev(seeds), 5)
     # the operators are reachable under the reference's names
@@ -247,7 +269,10 @@ def test_operator_layer_caches_and_buckets(orc, capi):
     fwd = npc.feat_shuffle(h, dev_off, recv_off, perm, 16, 1)
     assert torch.equal(fwd, h[perm])
     bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm, 16, 0)
-    assert torch.equal(bwd, h)                                  # pack undoes unpack
+    assert torch.equal(bwd, h)                                  # pack undoes unpack (shuffle_seeds' own permutation:
+    #                                                             a bijection by construction, taken without a check)
+    bwd = npc.feat_shuffle(fwd, recv_off, dev_off, perm.clone(), 16, 0)
+    assert torch.equal(bwd, h)                                  # the same values in another tensor: checked, same result
     # the pack direction is index_select_backward (reference src/feat_shuffle.cc:14-16): rows that several
     # entries name add up, rows nobody names are zero
     rep = perm.clone()
