@@ -551,6 +551,8 @@ static int minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_
 }
 }  // namespace apt
 
+
+
 extern "C" int apt_minibatch_sample(const apt_graph* graph, const int64_t* seeds, int64_t batch,
                                     const int* hop_fanouts, int num_hops, int replace,
                                     uint64_t rng_seed, const uint64_t* rng_seed_dev,

@@ -233,6 +233,24 @@ def build_workload(args, name, w, ctx, full_graph=None):
     return wl
 
 
+class TraceMarkers:
+    """Phase boundaries that show in a kernel trace: a one-workgroup launch of the plain copy kernel between the
+    benchmark's phases (the GPU idle before and after it), named in launch order in stages.trace_markers, so that
+    a rocprofv3 trace of this command can be cut into the phases the figures of the line come from."""
+
+    def __init__(self, torch, capi, dev):
+        self.torch, self.capi = torch, capi
+        self.a = torch.zeros(16, dtype=torch.uint8, device=dev)
+        self.b = torch.zeros(16, dtype=torch.uint8, device=dev)
+        self.names = []
+
+    def __call__(self, name):
+        self.torch.cuda.synchronize()
+        self.capi.synth_copy(self.a, self.b)
+        self.torch.cuda.synchronize()
+        self.names.append(name)
+
+
 def driver_kw(args):
     """MiniBatchPipeline arguments of --driver."""
     if args.driver in ("fused", "graph"):
@@ -253,7 +271,7 @@ def make_seed_sets(ctx, wl, B, count, seed):
 
 
 # ------------------------------------------------------------------------------------------------ measurement
-def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True):
+def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True, tag=""):
     """W warm-up and exactly K timed batches of workload wl on one stream, then (untimed) the same batches
     again to read their sizes.  -> SimpleNamespace with the pipeline, the seed sets and the figures."""
     torch, capi, kev = ctx.torch, ctx.capi, ctx.kev
@@ -298,7 +316,7 @@ def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True):
     gkevs = {i: kev.pair() for i in timed_steps}
     skevs = {i: kev.pair() for i in timed_steps} if args.driver == "fused" else {}
     start, stop = ev(), ev()
-    torch.cuda.synchronize()
+    ctx.mark(f"{tag}timed region: {K} batches on one stream")
     t0 = time.perf_counter()
     start.record()
     for i in range(K):
@@ -306,6 +324,7 @@ def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True):
     stop.record()
     torch.cuda.synchronize()
     m.elapsed = time.perf_counter() - t0
+    ctx.mark(f"{tag}end of the timed region")
     m.sample_us = None
     if staged:
         m.gather_ms_by_step = [kev.ms(gkevs[i]) for i in timed_steps]
@@ -488,7 +507,9 @@ def stage_target_shape(args, ctx, wl, hops, store_of):
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) / Kt
 
+        ctx.mark(f"target shape {name}: {Kt} batches of 1024, every gather dispatch with events")
         us, rows, frac, step_ms = timed_pass(False)
+        ctx.mark(f"end of target shape {name}")
         edges = log[:, H + 1].cpu().tolist()
         wall_alone = wall_pass(False)
         riding = None
@@ -733,7 +754,7 @@ def stage_config(args, ctx, name, full_graph=None, with_aggregation=False):
     quiet_gc()
     hops = list(reversed(w["fan_out"]))
     K, W = args.config_steps, 10
-    m = measure(args, ctx, wl, w["batch"], hops, K, W, event_steps=16, per_step=False)
+    m = measure(args, ctx, wl, w["batch"], hops, K, W, event_steps=16, per_step=False, tag=f"{name}: ")
     tr = traffic_entry(MEASURED_GATHER_TRAFFIC_PER_ROW, args, wl, m.B)
     gq = quantiles([t * 1e3 for t in m.gather_ms]) if m.staged else None
     out = {
@@ -798,7 +819,8 @@ def main():
         capi.set_tuning(key, int(val))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    ctx = SimpleNamespace(torch=torch, capi=capi, synth=synth, dev=dev, kev=KernelEvents())
+    ctx = SimpleNamespace(torch=torch, capi=capi, synth=synth, dev=dev, kev=KernelEvents(),
+                          mark=TraceMarkers(torch, capi, dev))
     kev = ctx.kev
 
     w = dict(WORKLOADS[args.workload])
@@ -867,11 +889,12 @@ def main():
                     pipes[k].run(seed_sets[first + i], args.seed + 100 + first + i)
 
         run_batches(0, W)
-        torch.cuda.synchronize()
+        ctx.mark(f"{K} batches, {len(pipes)} in flight on {len(pipes)} streams")
         t0 = time.perf_counter()
         run_batches(W, K)
         torch.cuda.synchronize()
         t_fl = time.perf_counter() - t0
+        ctx.mark("end of the batches in flight")
         assert all(int(p.misses.item()) == 0 for p in pipes)
         in_flight = {"batches_in_flight": len(pipes), "ms_per_step": t_fl / K * 1e3,
                      "edges_per_s": edges / t_fl}
@@ -885,7 +908,9 @@ def main():
             from apt_amd.loader import MiniBatchLoader
             loader = MiniBatchLoader(wl.graph, wl.store, torch.cat(seed_sets), B, hops, in_flight=args.inflight,
                                      shuffle=False, replace=args.replace, seed=args.seed, requests=wl.requests)
+            ctx.mark(f"epoch loader: {W} + {K} batches, {args.inflight} streams")
             t_ld, loader_edges, gaps = time_loader(torch, loader, W)
+            ctx.mark("end of the epoch loader")
             in_flight["loader"] = {"ms_per_step": t_ld / K * 1e3, "edges_per_s": loader_edges / t_ld,
                                    "ms_between_batches": gaps, "host_us_per_batch": loader_cost_per_batch(loader)}
             del loader
@@ -992,6 +1017,7 @@ def main():
             "frontier_sizes_last_step": m.hop_sizes[-1],
             "request_bucket_sizes_last_step": m.request_sizes,
             "setup_s": wl.setup_s,
+            "trace_markers": ctx.mark.names,
             "configs": None,
         },
     }
