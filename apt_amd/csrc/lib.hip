@@ -19,11 +19,18 @@ static int g_payload_bits = 0;
 
 int tuning_sample_lanes() { return g_sample_lanes; }
 int tuning_gather_rows() { return g_gather_rows; }
-int tuning_gather_max_blocks() { return g_gather_max_blocks; }
+// Launch caps of the calling thread (the epoch driver's thread shapes its launches for co-residency); a
+// process-wide knob, when set, wins.
+static thread_local int t_sample_max_blocks = 0, t_gather_max_blocks = 0;
+void set_thread_launch_caps(int sample_blocks, int gather_blocks) {
+  t_sample_max_blocks = sample_blocks;
+  t_gather_max_blocks = gather_blocks;
+}
+int tuning_gather_max_blocks() { return g_gather_max_blocks != 0 ? g_gather_max_blocks : t_gather_max_blocks; }
 int tuning_fuse_mark() { return g_fuse_mark; }
 int tuning_payload_bits() { return g_payload_bits; }
 static int g_sample_max_blocks = 0;
-int tuning_sample_max_blocks() { return g_sample_max_blocks; }
+int tuning_sample_max_blocks() { return g_sample_max_blocks != 0 ? g_sample_max_blocks : t_sample_max_blocks; }
 static int g_sample_min_workgroups = 0;
 int tuning_sample_min_workgroups() { return g_sample_min_workgroups; }
 static int g_sample_direct_rows = 0;

@@ -60,13 +60,18 @@ class MiniBatchLoader:
         c_ok = not formats and not use_graph
         if driver == "c" and not c_ok:
             raise ValueError("the C epoch driver does not emit block formats or replay graphs: use driver='python'")
+        from . import capi
+        if len(self.pipes) > capi.MAX_SLOTS:
+            if driver == "c":
+                raise ValueError(f"the C epoch driver takes at most {capi.MAX_SLOTS} batches in flight")
+            c_ok = False
         self._c_driver = None
         self._use_c = c_ok and driver != "python"
         # The C driver enqueues batch i + F behind batch i on the same stream without waiting for the consumer,
         # so that no stream runs dry between a batch's completion and the consumer's release of it: that takes a
         # second set of buffers per stream (the two sets of a stream share its rank table).
         self._spare = ([MiniBatchPipeline(graph, feat, self.batch_size, hop_fanouts, table=p.plan.table, **kw)
-                        for p in self.pipes] if self._use_c else [])
+                        for p in self.pipes] if self._use_c and 2 * len(self.pipes) <= capi.MAX_SLOTS else [])
 
     def __len__(self):
         return self.num_full + (1 if self.tail else 0)
@@ -134,7 +139,7 @@ class MiniBatchLoader:
         from . import capi
         slots = self.pipes + self._spare
         if self._c_driver is None:
-            self._c_driver = capi.EpochDriver(slots, self.streams + self.streams)
+            self._c_driver = capi.EpochDriver(slots, (self.streams + self.streams)[:len(slots)])
         drv = self._c_driver
         if self.num_full:
             drv.begin(full.reshape(-1), self.num_full, rng0, ready)
