@@ -32,9 +32,21 @@ from bench_extra import HBM_PEAK_GBPS, gather_bytes_per_row, quantiles
 # figure depends on, (workload, graph kind, feature dtype, feature dim, batch); a run with any other combination
 # reports traffic null.  Each entry names the profiles/ file that holds the counter readings.
 MEASURED_GATHER_TRAFFIC_PER_ROW = {
+    ("full", "symmetric", "bf16", 128, 4096): (520.4, "profiles/gather_kernel_full_pmc.txt"),
+    ("target", "symmetric", "bf16", 128, 1024): (519.5, "profiles/gather_kernel_target_bf16_pmc.txt"),
+    ("target", "symmetric", "fp32", 128, 1024): (1030.7, "profiles/gather_kernel_target_fp32_pmc.txt"),
+    ("medium", "symmetric", "fp32", 100, 1024): (916.5, "profiles/gather_kernel_medium_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (1169.4, "profiles/gather_kernel_partition_pmc.txt"),
+    ("small", "directed", "fp32", 128, 1024): (1036.1, "profiles/gather_kernel_small_pmc.txt"),
 }
 # The same for the last hop's sampling kernel (rank-table bids included): HBM bytes per sampled edge.
 MEASURED_SAMPLE_TRAFFIC_PER_EDGE = {
+    ("full", "symmetric", "bf16", 128, 4096): (258.4, "profiles/gather_kernel_full_pmc.txt"),
+    ("target", "symmetric", "bf16", 128, 1024): (270.6, "profiles/gather_kernel_target_bf16_pmc.txt"),
+    ("target", "symmetric", "fp32", 128, 1024): (270.5, "profiles/gather_kernel_target_fp32_pmc.txt"),
+    ("medium", "symmetric", "fp32", 100, 1024): (214.0, "profiles/gather_kernel_medium_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (429.6, "profiles/gather_kernel_partition_pmc.txt"),
+    ("small", "directed", "fp32", 128, 1024): (207.3, "profiles/gather_kernel_small_pmc.txt"),
 }
 
 WORKLOADS = {
@@ -380,8 +392,8 @@ def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True, tag=""):
 
 
 def traffic_entry(table, args, wl, B):
-    if args.fan_out or args.replace:
-        return None
+    if args.fan_out or args.replace or args.tune:
+        return None           # counters were read with the shipped kernels on the workload's own shape
     return table.get((wl.name, wl.graph_kind, wl.w["dtype"], wl.w["dim"], B))
 
 
