@@ -115,11 +115,23 @@ template <int V, int LPR, int R>
 __device__ __forceinline__ void gather_rows_of_block(const GatherParams& p, int64_t block, int64_t num_blocks) {
   using Vec = typename VecT<V>::type;
   constexpr int kGroups = kGatherBlock / LPR;
-  const int64_t n = actual_count(p.n, p.n_dev);
   const int grp = threadIdx.x / LPR;
   const int l = threadIdx.x % LPR;
   const int64_t vec_per_row = p.out_row_bytes / V;
   const int64_t rows_per_block = static_cast<int64_t>(kGroups) * R;
+  const int64_t stride = num_blocks * rows_per_block;
+  int64_t base = block * rows_per_block;
+  // The ids of a group's first rows are asked for before the device-side count has arrived: index[] has p.n
+  // entries whatever the count says, so the two round trips overlap instead of following each other (a launch
+  // of a few hundred thousand rows is a handful of iterations per group, and its first one starts on a cold
+  // path).  Later iterations fetch their ids at the end of the iteration before.
+  int64_t id[R];
+#pragma unroll
+  for (int k = 0; k < R; ++k) {
+    const int64_t r = base + static_cast<int64_t>(k) * kGroups + grp;
+    id[k] = r < p.n ? p.index[r] : -1;
+  }
+  const int64_t n = actual_count(p.n, p.n_dev);
   int launch_policy = p.store_policy;
   // rows from wt_from on are stored write-through: everything when the output is small, else the part the kernel
   // writes last
@@ -129,7 +141,7 @@ __device__ __forceinline__ void gather_rows_of_block(const GatherParams& p, int6
     wt_from = n * p.out_row_bytes <= kWriteThroughMaxBytes ? 0 : n - p.wt_tail_bytes / p.out_row_bytes;
   }
   int64_t misses = 0;
-  for (int64_t base = block * rows_per_block; base < n; base += num_blocks * rows_per_block) {
+  while (base < n) {
     const int policy = base >= wt_from ? kStoreWriteThrough : launch_policy;
     const char* src[R];
     char* dst[R];
@@ -139,7 +151,7 @@ __device__ __forceinline__ void gather_rows_of_block(const GatherParams& p, int6
       src[k] = nullptr;
       dst[k] = nullptr;
       if (r < n) {
-        const int64_t v = p.index[r];
+        const int64_t v = id[k];
         if (p.scatter) {
           // pack: row r of the input goes to row index[r] of the output
           if (v >= 0 && v < p.num_out_rows) {
@@ -167,6 +179,12 @@ __device__ __forceinline__ void gather_rows_of_block(const GatherParams& p, int6
         if (dst[k] != nullptr) store_row_vec<V>(val[k], reinterpret_cast<Vec*>(dst[k]) + c, policy);
       }
     }
+    base += stride;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+      const int64_t r = base + static_cast<int64_t>(k) * kGroups + grp;
+      if (r < n) id[k] = p.index[r];
+    }
   }
   if (p.miss_count != nullptr && misses != 0)
     atomicAdd(reinterpret_cast<unsigned long long*>(p.miss_count),
@@ -181,9 +199,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(GatherParams p) {
 // The gather with a batch's pending relabel lookups in its grid (16-byte vectors, two rows in flight): the
 // grid's first workgroups do the lookup pass, whose dependent reads are then on their way while the rest stream
 // rows.  The lookup blocks are numbered after the gather's and the workgroup ids rotated, rather than numbering
-// them first and subtracting: written that way the row loop came out at 42 VGPRs instead of 40, and the 2048
-// workgroups that the grid of a small launch is capped at no longer ran together (27 instead of 22 us for
-// 235 k rows).
+// them first and subtracting: written that way a launch of 235 k rows took 27 instead of 22 us.
 template <int LPR>
 __global__ __launch_bounds__(kGatherBlock) void gather_with_lookup_kernel(GatherParams p, LookupParams lp) {
   static_assert(kGatherBlock == kLookupBlock, "the lookup pass runs in workgroups of the gather's size");

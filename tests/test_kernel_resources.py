@@ -1,12 +1,12 @@
 """Resource budgets of the hot kernels, read from the compiler's own remarks
 (-Rpass-analysis=kernel-resource-usage while cross-compiling for gfx950; no GPU needed).
 
-The gather's row loop sits on a register cliff: the grid of a small launch is capped at the 2048
-workgroups the CUs hold at once, which they do at 40 VGPRs per lane (8 waves per SIMD); at 41 or more
-the allocation granule takes the kernel to 48, a fifth of the workgroups no longer run together and a
-launch of 235 k rows takes 27 instead of 22 us.  Nothing in a functional test notices that, so the
-budgets are asserted here: an edit (or a compiler) that adds two registers fails this test instead of
-silently costing the 60 %-of-peak target.
+A launch of the gather is capped at the 2048 workgroups the CUs hold at once (8 waves per SIMD), which they
+only do while the kernel allocates at most 64 VGPRs per lane and no scratch; registers are allocated in
+granules of 8, and the shipped row loop (16-byte vectors, two rows in flight, the ids of the next iteration
+fetched at the end of the one before) uses 44.  Nothing in a functional test notices when an edit or a compiler
+takes a kernel over such a limit or makes it spill, so the budgets are asserted here from the compiler's own
+figures.
 """
 import os
 import re
@@ -59,7 +59,7 @@ def _one(res, prefix):
     return res[hits[0]]
 
 
-def test_gather_kernels_stay_on_the_good_side_of_the_register_cliff(tmp_path):
+def test_gather_kernels_keep_full_occupancy_and_do_not_spill(tmp_path):
     res = _resources("gather.hip", tmp_path)
     # the shipped shapes: 16-byte vectors, two rows per lane group in flight, 16 lanes per row (256-byte rows),
     # 32 (512-byte rows) and 8 (128-byte rows); the variant that carries the relabel's last pass
@@ -67,8 +67,8 @@ def test_gather_kernels_stay_on_the_good_side_of_the_register_cliff(tmp_path):
                  "void apt::gather_kernel<16, 8, 2>(", "void apt::gather_with_lookup_kernel<16>(",
                  "void apt::gather_with_lookup_kernel<32>("):
         k = _one(res, name)
-        assert k["VGPRs"] <= 40, (name, k)                       # 8 waves per SIMD: 2048 co-resident workgroups
-        assert k["Occupancy"] >= 8, (name, k)
+        assert k["VGPRs"] <= 48, (name, k)                       # measured at 44; 8 waves per SIMD need <= 64
+        assert k["Occupancy"] >= 8, (name, k)                    # 8 waves per SIMD: 2048 co-resident workgroups
         assert k["ScratchSize"] == 0 and k["VGPRs Spill"] == 0 and k["SGPRs Spill"] == 0, (name, k)
         assert k["LDS Size"] == 0, (name, k)
     # no gather variant may spill, whatever its shape
