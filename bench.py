@@ -114,6 +114,8 @@ def parse_args():
     ap.add_argument("--cache_build", action="store_true",
                     help="also time the cache-construction kernels (access counting, cached CSR of the hottest rows, "
                          "cached feature table) and one step of the all-strategies dry run")
+    ap.add_argument("--operators", action="store_true",
+                    help="also time the batch through the operator layer (per-hop calls and sample_blocks)")
     ap.add_argument("--gather_sizes", action="store_true",
                     help="also time the gather kernel alone on 0 .. 940 k random rows of this workload's table "
                          "(device-side count, every launch with its own events): what a launch costs before it moves a byte")
@@ -322,8 +324,10 @@ def measure(args, ctx, wl, B, hops, K, W, event_steps, per_step=True, tag=""):
     # GPU stamps when the kernel begins and ends (no extra packets on the stream); what is left of the
     # region is sampling + relabel, dispatch gaps included.  Such a dispatch costs the host a little more
     # to enqueue, which would show in launch-bound small workloads, so a limited number of evenly spaced
-    # steps (--event_steps) carry them (and the last hop's sampling kernel of the same steps).
-    every = max(1, -(-K // max(1, event_steps)))
+    # steps (--event_steps) carry them (and the last hop's sampling kernel of the same steps), and never more
+    # than every fourth: a dispatch with events is fenced off from its neighbours on the stream, about 4 us
+    # each, which a short region (--steps 20) would otherwise pay on every step.
+    every = max(min(4, K), -(-K // max(1, event_steps)))
     timed_steps = m.timed_steps = [i for i in range(K) if staged and i % every == 0]
     gkevs = {i: kev.pair() for i in timed_steps}
     skevs = {i: kev.pair() for i in timed_steps} if args.driver == "fused" else {}
@@ -971,6 +975,9 @@ def main():
         torch.cuda.empty_cache()
 
     relabel_small = extra.stage_relabel_small(capi, dev, wl.N, torch) if args.relabel_small else None
+    operators = None
+    if args.operators and wl.requests is None and not args.replace:
+        operators = extra.stage_operators(torch, wl, hops, seed_sets, W, K, args.seed + 5000)
     gather_sizes = None
     if args.gather_sizes and wl.requests is None:
         gather_sizes = extra.stage_gather_sizes(capi, dev, kev, wl.store, wl.N, torch)
@@ -1013,6 +1020,7 @@ def main():
         "cache_build": cache_build,
         "shuffle": shuffle,
         "relabel_small": relabel_small,
+        "operators": operators,
         "alternate": alternate,
         "gather_sizes": gather_sizes,
         "stages": {

@@ -296,6 +296,52 @@ def stage_relabel_small(capi, dev, N, torch):
 TUNING_DEFAULTS = {"minibatch_fuse_mark": 1, "relabel_lds": 1, "block_fused_scan": 1}
 
 
+def stage_operators(torch, wl, hops, seed_sets, W, K, rng_base):
+    """The batch through the operator layer (torch.ops.npc.*), as the reference's sampler calls it
+    (python/npc/sampler.py:187-203): local_sample_one_layer + relabel_csc per hop, with the rank table of the
+    registered graph and with the hash table; then the one operator that runs all hops (sample_blocks), with
+    fresh output tensors per call (the default) and with the ring of two buffer sets.  No gather; every call
+    returns narrowed tensors, i.e. reads its sizes back as the reference's operators do."""
+    import apt_amd as npc
+    empty = torch.empty(0, dtype=torch.int64)
+    npc.set_topology(0, 1)
+    npc.mix_cache_graphs(0, empty, empty, empty, wl.indptr, wl.indices)
+    n = min(K, 60)
+
+    def per_hop(seeds, key):
+        frontier = seeds
+        for h, f in enumerate(hops):
+            nb, _ = npc.ops.sample_neighbors(frontier, f, False, key, h)
+            frontier, _ = npc.ops.tensor_relabel_csc(frontier, nb)
+        return frontier
+
+    def timed(fn):
+        for i in range(min(W, 10)):
+            fn(seed_sets[i], rng_base + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            fn(seed_sets[W + i], rng_base + W + i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    out = {"batches": n}
+    try:
+        npc.ops.set_ranked_relabel(True)
+        out["per_hop_rank_table_ms"] = timed(per_hop)
+        npc.ops.set_ranked_relabel(False)
+        out["per_hop_hash_table_ms"] = timed(per_hop)
+        npc.ops.set_ranked_relabel(True)
+        blocks = lambda seeds, key: npc.ops.sample_blocks(seeds, list(hops), False, key)
+        out["sample_blocks_fresh_tensors_ms"] = timed(blocks)
+        npc.ops.set_block_buffer_ring(2)
+        out["sample_blocks_ring_of_two_ms"] = timed(blocks)
+    finally:
+        npc.ops.set_block_buffer_ring(0)
+        npc.ops.set_ranked_relabel(True)
+    return out
+
+
 def stage_alternate(args, capi, graph, hops, kev, MiniBatchPipeline, seed_n, seed_lo, store, B, torch, dev):
     """Kernel-variant knobs against each other inside one process: six rounds, in each of which every setting
     runs the same 35 batches on one stream (wall time) and 20 more whose gather and last-hop sampling dispatches
