@@ -35,18 +35,18 @@ MEASURED_GATHER_TRAFFIC_PER_ROW = {
     ("full", "symmetric", "bf16", 128, 4096): (520.4, "profiles/gather_kernel_full_pmc.txt"),
     ("target", "symmetric", "bf16", 128, 1024): (519.5, "profiles/gather_kernel_target_bf16_pmc.txt"),
     ("target", "symmetric", "fp32", 128, 1024): (1030.7, "profiles/gather_kernel_target_fp32_pmc.txt"),
-    ("medium", "symmetric", "fp32", 100, 1024): (916.5, "profiles/gather_kernel_medium_pmc.txt"),
-    ("partition", "symmetric", "fp32", 128, 1024): (1169.4, "profiles/gather_kernel_partition_pmc.txt"),
-    ("small", "directed", "fp32", 128, 1024): (1036.1, "profiles/gather_kernel_small_pmc.txt"),
+    ("medium", "symmetric", "fp32", 100, 1024): (916.6, "profiles/gather_kernel_medium_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (1197.7, "profiles/gather_kernel_partition_pmc.txt"),
+    ("small", "directed", "fp32", 128, 1024): (1054.7, "profiles/gather_kernel_small_pmc.txt"),
 }
 # The same for the last hop's sampling kernel (rank-table bids included): HBM bytes per sampled edge.
 MEASURED_SAMPLE_TRAFFIC_PER_EDGE = {
-    ("full", "symmetric", "bf16", 128, 4096): (258.4, "profiles/gather_kernel_full_pmc.txt"),
-    ("target", "symmetric", "bf16", 128, 1024): (270.6, "profiles/gather_kernel_target_bf16_pmc.txt"),
-    ("target", "symmetric", "fp32", 128, 1024): (270.5, "profiles/gather_kernel_target_fp32_pmc.txt"),
-    ("medium", "symmetric", "fp32", 100, 1024): (214.0, "profiles/gather_kernel_medium_pmc.txt"),
-    ("partition", "symmetric", "fp32", 128, 1024): (429.6, "profiles/gather_kernel_partition_pmc.txt"),
-    ("small", "directed", "fp32", 128, 1024): (207.3, "profiles/gather_kernel_small_pmc.txt"),
+    ("full", "symmetric", "bf16", 128, 4096): (258.5, "profiles/gather_kernel_full_pmc.txt"),
+    ("target", "symmetric", "bf16", 128, 1024): (270.3, "profiles/gather_kernel_target_bf16_pmc.txt"),
+    ("target", "symmetric", "fp32", 128, 1024): (270.3, "profiles/gather_kernel_target_fp32_pmc.txt"),
+    ("medium", "symmetric", "fp32", 100, 1024): (213.1, "profiles/gather_kernel_medium_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (429.8, "profiles/gather_kernel_partition_pmc.txt"),
+    ("small", "directed", "fp32", 128, 1024): (204.0, "profiles/gather_kernel_small_pmc.txt"),
 }
 
 WORKLOADS = {
