@@ -577,19 +577,21 @@ def quiet_gc():
 
 
 def time_loader(torch, loader, warm):
-    """One epoch of `loader` after `warm` untimed batches -> (seconds, sampled edges, quantiles of the time
-    between consecutive batches in ms)."""
+    """One epoch of `loader`; the clock starts when the `warm`-th batch has been handed over and stops when the
+    last one has (a batch is complete on the GPU when the loader yields it) -> (seconds, sampled edges of the
+    timed batches, quantiles of the time between consecutive batches in ms).  The pipeline is not drained before
+    the clock starts: the batches the driver has enqueued ahead by then are the steady state, and draining them
+    first would hand the timed part that many finished batches for nothing."""
     it = iter(loader)
+    stamps = [time.perf_counter()]
     for _ in range(warm):
         next(it)
-    torch.cuda.synchronize()
-    stamps = [time.perf_counter()]
+        stamps[0] = time.perf_counter()
     edges = 0
     for batch in it:
         edges += batch["num_edges"]
         stamps.append(time.perf_counter())
     torch.cuda.synchronize()
-    stamps[-1] = time.perf_counter()
     return stamps[-1] - stamps[0], edges, quantiles([(b - a) * 1e3 for a, b in zip(stamps, stamps[1:])])
 
 
