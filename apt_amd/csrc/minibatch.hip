@@ -200,20 +200,66 @@ __device__ __forceinline__ bool mb_is_owner(const HopParams& p, const HopSizes& 
   return p.table[v] == table_base(p.state) + bid;
 }
 
+// Upper bound of a hop's neighbour slots as the host knows it: what the buffers hold whatever the device-side
+// row count says.  Loads of per-slot arrays below this bound are safe before that count has arrived, which
+// takes a memory round trip or two out of the start of the small kernels of a batch (they are chains of three
+// to five such trips and little else).  Only launches of a few hundred workgroups do that: in a large launch
+// the workgroups past the real count would fetch megabytes for nothing, and its many waves hide the trip anyway.
+__device__ __forceinline__ int64_t slot_capacity(const HopParams& p) {
+  return p.nn_fixed >= 0 ? p.nn_fixed : p.ns_cap * p.fanout;
+}
+constexpr unsigned kLoadAheadMaxBlocks = 512;
+
 template <bool FIRST>
 __global__ __launch_bounds__(kMbBlock) void mb_count_kernel(HopParams p) {
-  const HopSizes s = hop_sizes(p);
-  const int64_t items = FIRST ? s.ns + s.nn : s.nn;
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kMbTile;
-  if (base >= items) return;
   __shared__ uint32_t s_wave[kMbWaves];
   const int wave = threadIdx.x / kWave;
   uint32_t c = 0;
+  if (FIRST) {
+    const HopSizes s = hop_sizes(p);
+    const int64_t items = s.ns + s.nn;
+    if (base >= items) return;
 #pragma unroll
-  for (int it = 0; it < kMbIters; ++it) {
-    const uint64_t m = ballot(mb_is_owner<FIRST>(p, s, base + it * kMbBlock + threadIdx.x, items));
-    if (lane_id() == 0) p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + wave] = m;
-    c += __popcll(m);
+    for (int it = 0; it < kMbIters; ++it) {
+      const uint64_t m = ballot(mb_is_owner<FIRST>(p, s, base + it * kMbBlock + threadIdx.x, items));
+      if (lane_id() == 0) p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + wave] = m;
+      c += __popcll(m);
+    }
+  } else {
+    // Later hops: the bidding itself settled ownership (rank_table.hpp): a slot owns its node iff it is
+    // kSlotOwner and was never displaced; the flag is consumed so that the buffer is clean for the next hop.
+    // Both arrays are read under the host's bound, before the row count is known.
+    const bool ahead = gridDim.x <= kLoadAheadMaxBlocks;
+    const int64_t cap = ahead ? slot_capacity(p) : 0;
+    int64_t rel[kMbIters];
+    uint8_t dis[kMbIters];
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it) {
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      rel[it] = i < cap ? p.relabeled[i] : 0;
+      dis[it] = i < cap ? p.displaced[i] : 0;
+    }
+    const HopSizes s = hop_sizes(p);
+    const int64_t items = s.nn;
+    if (base >= items) return;
+    if (!ahead) {
+#pragma unroll
+      for (int it = 0; it < kMbIters; ++it) {
+        const int64_t i = base + it * kMbBlock + threadIdx.x;
+        rel[it] = i < items ? p.relabeled[i] : 0;
+        dis[it] = i < items ? p.displaced[i] : 0;
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it) {
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      const bool bid_in = i < items && rel[it] == kSlotOwner;
+      if (bid_in && dis[it] != 0) p.displaced[i] = 0;
+      const uint64_t m = ballot(bid_in && dis[it] == 0);
+      if (lane_id() == 0) p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + wave] = m;
+      c += __popcll(m);
+    }
   }
   if (lane_id() == 0) s_wave[wave] = c;
   __syncthreads();
@@ -228,6 +274,33 @@ __global__ __launch_bounds__(kMbBlock) void mb_count_kernel(HopParams p) {
 // node list and written into the table.
 template <bool FIRST>
 __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
+  const int64_t base = static_cast<int64_t>(blockIdx.x) * kMbTile;
+  const int wave = threadIdx.x / kWave;
+  const int lane = lane_id();
+  // In a small launch, what does not depend on the hop's row count is requested before it: the owner counts
+  // of the tiles before this one and this tile's owner bits (the count pass wrote both for every tile that has
+  // items, and a tile without items leaves below before using them), and, on later hops, the tile's neighbour
+  // ids.
+  const bool ahead_ok = gridDim.x <= kLoadAheadMaxBlocks;
+  int64_t part = 0;
+  uint64_t mask[kMbIters][kMbWaves];
+  int64_t ahead[kMbIters];
+  auto load_tile = [&](int64_t cap) {
+    for (int64_t b = threadIdx.x; b < blockIdx.x; b += kMbBlock) part += p.tile_cnt[b];
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it)
+#pragma unroll
+      for (int w = 0; w < kMbWaves; ++w)
+        mask[it][w] = p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + w];
+    if (!FIRST) {
+#pragma unroll
+      for (int it = 0; it < kMbIters; ++it) {
+        const int64_t i = base + it * kMbBlock + threadIdx.x;
+        ahead[it] = i < cap ? p.neighbors[i] : -1;
+      }
+    }
+  };
+  if (ahead_ok) load_tile(slot_capacity(p));
   const HopSizes s = hop_sizes(p);
   const int64_t items = FIRST ? s.ns + s.nn : s.nn;
   const int64_t first_id = FIRST ? 0 : s.ns;
@@ -235,23 +308,13 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
     if (blockIdx.x == 0 && threadIdx.x == 0) *p.n_next = first_id;
     return;
   }
-  const int64_t base = static_cast<int64_t>(blockIdx.x) * kMbTile;
   if (base >= items) return;
+  if (!ahead_ok) load_tile(items);
   const int64_t tiles = (items + kMbTile - 1) / kMbTile;
   __shared__ int64_t s_red[kMbWaves];
-  const int wave = threadIdx.x / kWave;
-  const int lane = lane_id();
-  int64_t part = 0;
-  for (int64_t b = threadIdx.x; b < blockIdx.x; b += kMbBlock) part += p.tile_cnt[b];
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_down(part, off, kWave);
   if (lane == 0) s_red[wave] = part;
-  uint64_t mask[kMbIters][kMbWaves];
-#pragma unroll
-  for (int it = 0; it < kMbIters; ++it)
-#pragma unroll
-    for (int w = 0; w < kMbWaves; ++w)
-      mask[it][w] = p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + w];
   __syncthreads();
   int64_t running = first_id;
   for (int w = 0; w < kMbWaves; ++w) running += s_red[w];
@@ -276,7 +339,7 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
         v = i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns];
         if (i >= s.ns) p.relabeled[i - s.ns] = id;
       } else {
-        v = p.neighbors[i];
+        v = ahead[it];
         p.relabeled[i] = id;
       }
       if (id < p.nodes_cap) {

@@ -132,16 +132,26 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   __shared__ unsigned long long s_total;
   extern __shared__ int64_t s_picks[];  // [G][fanout], only when fanout > LPS
 
-  const int64_t n = actual_count(p.n, p.n_dev);
-  const int tile = G * p.rows_per_group;
-  if (static_cast<int64_t>(blockIdx.x) * tile >= n) return;  // block-uniform
-  const uint64_t seed = p.seed_dev != nullptr ? *p.seed_dev : p.seed;
-  RankEpoch ep{0, 0, 0};
-  if (p.table.entries != nullptr) ep = rank_epoch(p.table.state);
-
   const int tid = threadIdx.x;
   const int grp = tid / LPS;
   const int l = tid % LPS;
+  const int tile = G * p.rows_per_group;
+  // What does not depend on the row count is read before it: the rng seed and the table's epoch, and, in a small
+  // launch with a device-side count (the later hops of a batch: a chain of dependent round trips with a single
+  // round of waves to hide them), the frontier entry of the first row this lane will work on, so that the
+  // read that follows the count finds it in the cache.  frontier[] has p.n entries whatever the count says.
+  const uint64_t seed = p.seed_dev != nullptr ? *p.seed_dev : p.seed;
+  RankEpoch ep{0, 0, 0};
+  if (p.table.entries != nullptr) ep = rank_epoch(p.table.state);
+  int64_t touched = 0;
+  if (p.n_dev != nullptr && gridDim.x <= 512) {
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * tile + (p.direct != 0 ? grp : tid);
+    if (first < p.n) touched = p.frontier[first];
+  }
+  const int64_t n = actual_count(p.n, p.n_dev);
+  asm volatile("" ::"v"(touched));  // keeps the early read; nothing uses its value
+  if (static_cast<int64_t>(blockIdx.x) * tile >= n) return;  // block-uniform
+
   const int fanout = p.fanout;
   int64_t my_total = 0;
   if (tid == 0) s_total = 0;

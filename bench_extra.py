@@ -58,7 +58,7 @@ def graph_replay_us(torch, fn, reps=10, replays=5):
 
 
 def stage_aggregation(capi, dev, synth, torch, pipe, seeds, rng_seed, data_seed=1):
-    """The aggregation stage (BASELINE configs[4]) on the outermost block of one batch: GraphSAGE mean SpMM
+    """The aggregation stage on the outermost block of one batch: GraphSAGE mean SpMM
     (hidden 256, fp32 and bf16 rows, fp32 accumulation) and a GAT layer of 4 heads x 64 (logits, then fused
     LeakyReLU + edge softmax + weighted sum), each with the bytes it has to move and its duration."""
     pipe.run(seeds, rng_seed)
