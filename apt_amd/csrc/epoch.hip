@@ -31,8 +31,8 @@ void set_thread_launch_caps(int sample_blocks, int gather_blocks);  // lib.hip
 // takes at most 512 workgroups of 512 threads and a gather at most 1024 of 256, half of the CUs' wave slots
 // either way, so that one batch's gather (bound by bandwidth) and another's last-hop sampler (bound by random
 // transactions) are resident together instead of taking turns at full width.  Measured on the 111 M-node graph
-// with four streams: 0.151-0.155 against 0.160 ms per batch of 4096 seeds, 0.063 against 0.067 ms per batch of
-// 1024; with two or three streams, or a batch alone (0.222 against 0.206 ms), full width is faster.
+// with four streams: 0.151-0.157 against 0.160-0.163 ms per batch of 4096 seeds, 0.064 against 0.067 ms per batch
+// of 1024; with two or three streams, or a batch alone (0.208-0.223 against 0.202 ms), full width is faster.
 constexpr int kCoResidentStreams = 4;
 constexpr int kCoResidentSampleBlocks = 512;
 constexpr int kCoResidentGatherBlocks = 1024;
@@ -316,7 +316,7 @@ extern "C" int apt_epoch_next(apt_epoch* ep, int* slot, int64_t* sizes_host, int
     APT_REQUIRE(ep->last_released, APT_EINVAL, "apt_epoch_next: the previous batch has not been released");
     i = ep->handed_out;
     const auto t0 = std::chrono::steady_clock::now();
-    ep->cv_done.wait(lk, [ep, i] { return ep->enqueued > i; });
+    ep->cv_done.wait(lk, [ep, i] { return ep->enqueued > i || ep->error != 0; });
     ep->wait_enqueue_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     if (ep->error != 0) return fail(ep->error, "apt_epoch_next: batch could not be enqueued: %s", ep->error_text);
   }
@@ -355,15 +355,23 @@ extern "C" int apt_epoch_release(apt_epoch* ep, void* consumer_stream) {
   // and would then complete only after that stream's queued batches, stalling the slot for no reason.
   hipEvent_t after = nullptr;
   const auto t0 = std::chrono::steady_clock::now();
-  const hipError_t idle = hipStreamQuery(static_cast<hipStream_t>(consumer_stream));
-  if (idle == hipErrorNotReady) {
-    APT_HIP(hipEventRecord(ep->released[k], static_cast<hipStream_t>(consumer_stream)));
+  hipError_t err = hipStreamQuery(static_cast<hipStream_t>(consumer_stream));
+  if (err == hipErrorNotReady) {
+    err = hipEventRecord(ep->released[k], static_cast<hipStream_t>(consumer_stream));
     after = ep->released[k];
-  } else if (idle != hipSuccess) {
-    return fail(APT_EHIP, "apt_epoch_release: hipStreamQuery failed: %s", hipGetErrorString(idle));
   }
   lk.lock();
   ep->release_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  if (err != hipSuccess) {
+    // the slot cannot be handed back: the epoch ends here, and apt_epoch_next says why instead of waiting
+    const int rc = fail(APT_EHIP, "apt_epoch_release: the consumer's stream: %s", hipGetErrorString(err));
+    if (ep->error == 0) {
+      ep->error = rc;
+      std::strncpy(ep->error_text, apt_last_error(), sizeof(ep->error_text) - 1);
+    }
+    ep->cv_done.notify_all();
+    return rc;
+  }
   if (ep->active) {
     ep->queue.push_back(EpochWork{next, k, after});
     ep->cv_work.notify_all();
