@@ -22,7 +22,7 @@ from .pipeline import MiniBatchPipeline
 class MiniBatchLoader:
     def __init__(self, graph, feat, indices, batch_size, hop_fanouts, in_flight=4, shuffle=True, drop_last=True,
                  replace=False, seed=0, formats=False, requests=None, use_graph=False, as_blocks=False,
-                 driver="auto"):
+                 driver="auto", streams=None):
         """indices: node ids to draw seeds from (the training ids).  hop_fanouts
         start from the seeds.  Yields MiniBatchPipeline.result() dicts with
         `output_nodes` (the batch's seeds) added.  A yielded batch lives in its
@@ -33,7 +33,11 @@ class MiniBatchLoader:
         for small batches, where the host's launch calls are the limit).  as_blocks:
         batch["blocks"] are sampler.Block objects, ready for apt_amd.layers.
         driver: "c" = batches are enqueued by the C library's epoch thread (not with formats or use_graph),
-        "python" = from this thread, "auto" = "c" where it applies."""
+        "python" = from this thread, "auto" = "c" where it applies.
+        streams: the torch.cuda.Stream objects to build batches on, one per batch in flight (default: new ones;
+        never the consumer's stream).  A process has few hardware queues (HIP's GPU_MAX_HW_QUEUES, 4 by default) and
+        its streams are dealt onto them as they are created, so in a process that has created other streams two of
+        the loader's may share a queue and take turns; a caller that knows better passes its own."""
         if in_flight < 1:
             raise ValueError("in_flight must be >= 1")
         dev = graph.device
@@ -49,7 +53,13 @@ class MiniBatchLoader:
         kw = dict(replace=replace, formats=formats, requests=requests, use_graph=use_graph)
         self._make = lambda b: MiniBatchPipeline(graph, feat, b, hop_fanouts, **kw)
         self.pipes = [self._make(self.batch_size) for _ in range(min(in_flight, max(self.num_full, 1)))]
-        self.streams = [torch.cuda.Stream(device=dev) for _ in self.pipes]
+        if streams is not None:
+            streams = list(streams)
+            if len(streams) < len(self.pipes):
+                raise ValueError(f"{len(streams)} streams for {len(self.pipes)} batches in flight")
+            if any(not isinstance(st, torch.cuda.Stream) or st.cuda_stream == 0 for st in streams):
+                raise ValueError("streams must be torch.cuda.Stream objects other than the default stream")
+        self.streams = streams[:len(self.pipes)] if streams is not None else [torch.cuda.Stream(device=dev) for _ in self.pipes]
         self.done = [torch.cuda.Event() for _ in self.pipes]
         self.released = [torch.cuda.Event() for _ in self.pipes]
         self.tail_pipe = self._make(self.tail) if self.tail else None     # the short last batch has buffers of its own

@@ -79,6 +79,14 @@ def test_loader_c_and_python_drivers_agree(capi):
     assert a._use_c and not b._use_c and MiniBatchLoader(g, store, ids, 200, [4], **kw)._use_c
     with pytest.raises(ValueError):
         MiniBatchLoader(g, store, ids, 200, [4], driver="c", formats=True)
+    # the caller's own streams (one per batch in flight, never the default stream)
+    mine = [torch.cuda.Stream() for _ in range(3)]
+    a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", streams=mine, **kw)
+    assert [st.cuda_stream for st in a.streams] == [st.cuda_stream for st in mine]
+    with pytest.raises(ValueError):
+        MiniBatchLoader(g, store, ids, 200, [4], streams=mine[:2], **kw)
+    with pytest.raises(ValueError):
+        MiniBatchLoader(g, store, ids, 200, [4], streams=[torch.cuda.default_stream()] * 3, **kw)
     for epoch in range(2):
         n = 0
         for x, y in zip(a, b):
