@@ -800,8 +800,7 @@ def stage_config(args, ctx, name, full_graph=None, with_aggregation=False):
                          "ms_between_batches": gaps, "host_us_per_batch": loader_cost_per_batch(loader)}
         del loader
     if args.cpu_seconds > 0:
-        # feature tables of the partition are 17 GB: its rows are compared in tests/test_gpu_configs.py, not here
-        h = host_copies(ctx, wl, with_features=wl.requests is None)
+        h = host_copies(ctx, wl)      # the partition's two feature tables included (17 GB)
         h.orc.set_threads(args.cpu_threads or min(16, h.orc.max_threads()))
         out["parity"] = parity_of_batches(args, ctx, wl, h, m.stage_pipe, m.seed_sets[W:W + 1], [args.seed + 100 + W], hops)
         del h
