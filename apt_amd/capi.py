@@ -74,6 +74,8 @@ SYMBOLS = {
     "apt_relabel_ranked_max_items": (_I64, []),
     "apt_relabel_ranked_workspace_bytes": (_SZ, [_I64]),
     "apt_relabel_ranked": (_I, [_P, _I64, _P, _P, _I64, _I64, _I, _P, _I64, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "apt_sample_neighbors_bidding": (_I, [C.POINTER(CGraph), _P, _I64, _P, _I, _I, _U64, _I, _P, _P, _P, _I, _P, _I64, _P,
+                                          _P, _P, _SZ, _P]),
     "apt_relabel_static_max_items": (_I64, []),
     "apt_relabel_static": (_I, [_P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P]),
     "apt_gather_rows": (_I, [C.POINTER(CFeatStore), _P, _I64, _P, _P, _P, _P]),
@@ -347,16 +349,33 @@ class RankedRelabel:
             self.workspace = torch.empty(max(need, 256) * 2, dtype=torch.uint8, device=device)
             check(lib().apt_minibatch_workspace_init(_ptr(self.workspace), self.workspace.numel(), _stream()))
 
+    def sample_bidding(self, graph, frontier, fanout, replace, rng_seed, hop, continued, out_neighbors, slot_states,
+                       num_frontier_dev=None, out_counts=None, out_total=None, num_outside_dev=None):
+        """apt_sample_neighbors_bidding: one hop of sampling that places the bids of the relabel call that follows
+        (enqueue(..., bids_placed=True) with slot_states as `relabeled`).  fanout <= 64."""
+        frontier = _dev_i64(frontier, "frontier")
+        n = frontier.numel()
+        self._workspace_for(n + n * int(fanout), frontier.device)
+        self._last = self._last_tensor = None
+        check(lib().apt_sample_neighbors_bidding(C.byref(graph.c), _ptr(frontier), n, _ptr(num_frontier_dev), int(fanout),
+                                                 int(bool(replace)), int(rng_seed) & 0xFFFFFFFFFFFFFFFF, int(hop),
+                                                 _ptr(out_neighbors), _ptr(out_counts), _ptr(out_total),
+                                                 int(bool(continued)), _ptr(self.table), self.table_len,
+                                                 _ptr(slot_states), _ptr(num_outside_dev), _ptr(self.workspace),
+                                                 self.workspace.numel(), _stream()))
+
     def enqueue(self, seeds, neighbors, continued, unique, relabeled, num_unique_dev, num_outside_dev,
-                num_seeds_dev=None, neighbor_stride=0):
+                num_seeds_dev=None, neighbor_stride=0, bids_placed=False):
         """Asynchronous form with the caller's buffers and device-side sizes (as capi.relabel(sync=False)):
         num_unique_dev receives the count, num_outside_dev is incremented per id outside the table (device
-        int64[1] each; the caller clears the second)."""
+        int64[1] each; the caller clears the second).  bids_placed: `neighbors` and `relabeled` come from
+        sample_bidding on the same seeds."""
         seeds, neighbors = _dev_i64(seeds, "seeds"), _dev_i64(neighbors, "neighbors")
         self._workspace_for(seeds.numel() + neighbors.numel(), seeds.device)
         self._last = self._last_tensor = None
         check(lib().apt_relabel_ranked(_ptr(seeds), seeds.numel(), _ptr(num_seeds_dev), _ptr(neighbors),
-                                       neighbors.numel(), int(neighbor_stride), int(bool(continued)), _ptr(self.table),
+                                       neighbors.numel(), int(neighbor_stride),
+                                       int(bool(continued)) | (2 if bids_placed else 0), _ptr(self.table),
                                        self.table_len, _ptr(unique), _ptr(relabeled), _ptr(num_unique_dev),
                                        _ptr(num_outside_dev), None, _ptr(self.workspace), self.workspace.numel(),
                                        _stream()))

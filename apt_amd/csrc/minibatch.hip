@@ -41,11 +41,6 @@
 
 namespace apt {
 
-struct SampleMark {  // fused relabel marking inside the sampling kernel (sample.hip)
-  RankTable table;
-  int64_t* relabeled;
-  int first_hop;
-};
 
 int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
                   const int64_t* num_frontier_dev, int fanout, int replace, uint64_t rng_seed,
@@ -692,6 +687,54 @@ extern "C" size_t apt_relabel_ranked_workspace_bytes(int64_t num_items) {
   return apt::ranked_layout(num_items).total;
 }
 
+// apt_sample_neighbors with the bids of the apt_relabel_ranked call that follows placed on the way: the
+// sampling kernel has every id in registers when it loads it, and a bid placed there overlaps with the kernel's
+// own random reads instead of being a pass of its own over the ids.
+extern "C" int apt_sample_neighbors_bidding(const apt_graph* graph, const int64_t* frontier, int64_t num_frontier,
+                                            const int64_t* num_frontier_dev, int fanout, int replace,
+                                            uint64_t rng_seed, int hop, int64_t* out_neighbors, int64_t* out_counts,
+                                            int64_t* out_total, int continued, void* rank_table,
+                                            int64_t rank_table_len, int64_t* slot_states, int64_t* num_outside_dev,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace apt;
+  APT_REQUIRE(fanout >= 1 && fanout <= kWave, APT_ELIMIT, "apt_sample_neighbors_bidding: fanout %d outside [1, %d]",
+              fanout, kWave);
+  APT_REQUIRE(num_frontier >= 0 && slot_states != nullptr, APT_EINVAL,
+              "apt_sample_neighbors_bidding: negative size or slot_states is NULL");
+  const int64_t items = num_frontier + num_frontier * fanout;
+  APT_REQUIRE(items <= kRankedMaxItems, APT_ELIMIT,
+              "apt_sample_neighbors_bidding: %lld items exceed the supported maximum %lld", (long long)items,
+              (long long)kRankedMaxItems);
+  APT_REQUIRE(rank_table != nullptr && rank_table_len > 0 && rank_table_len < (int64_t{1} << 32) - 1 &&
+                  (reinterpret_cast<uintptr_t>(rank_table) & 255) == 0,
+              APT_EINVAL, "apt_sample_neighbors_bidding: rank table missing, misaligned or too long");
+  APT_REQUIRE(workspace != nullptr && workspace_bytes >= ranked_layout(items).total &&
+                  (reinterpret_cast<uintptr_t>(workspace) & 15) == 0,
+              APT_EWORKSPACE, "apt_sample_neighbors_bidding: workspace of %zu bytes, %zu needed (16-byte aligned)",
+              workspace_bytes, ranked_layout(items).total);
+  // the same layout as the apt_relabel_ranked call that will read the flags set here
+  int64_t lo = items, hi = kRankedMaxItems;
+  while (lo < hi) {
+    const int64_t mid = lo + (hi - lo + 1) / 2;
+    if (ranked_layout(mid).total <= workspace_bytes) lo = mid;
+    else hi = mid - 1;
+  }
+  const RankedLayout L = ranked_layout(lo);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t* state = reinterpret_cast<uint32_t*>(static_cast<char*>(rank_table) + table_state_offset(rank_table_len));
+  if (continued == 0) {
+    const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
+    hipLaunchKernelGGL(mb_begin_kernel, dim3(kBeginBlocks), dim3(kMbBlock), 0, st, static_cast<uint4*>(rank_table), vecs,
+                       state, kRankedPayloadBits, static_cast<int64_t*>(nullptr), 0, int64_t{0});
+    APT_LAUNCH_CHECK("mb_begin_kernel");
+  }
+  SampleMark mark{RankTable{static_cast<uint32_t*>(rank_table), rank_table_len, state,
+                            reinterpret_cast<uint8_t*>(static_cast<char*>(workspace) + L.displaced_off)},
+                  slot_states, continued == 0 ? 1 : 0, num_outside_dev};
+  return sample_launch(graph, frontier, num_frontier, num_frontier_dev, fanout, replace, rng_seed, nullptr, hop,
+                       out_neighbors, out_counts, out_total, st, "apt_sample_neighbors_bidding", &mark);
+}
+
 extern "C" int apt_relabel_ranked(const int64_t* seeds, int64_t num_seeds, const int64_t* num_seeds_dev,
                                   const int64_t* neighbors, int64_t num_neighbors, int64_t neighbor_stride,
                                   int continued, void* rank_table, int64_t rank_table_len,
@@ -754,7 +797,25 @@ extern "C" int apt_relabel_ranked(const int64_t* seeds, int64_t num_seeds, const
   hp.mark_seeds = 1;
   hp.prefix_src = nullptr;
   const dim3 mark_grid = grid_for(std::max(num_neighbors, num_seeds), kMbBlock, 1 << 16);
-  if (continued == 0) {
+  const bool marked = (continued & 2) != 0;   // apt_sample_neighbors_bidding has placed this call's bids
+  continued &= 1;
+  if (marked) {
+    APT_REQUIRE(num_neighbors > 0, APT_EINVAL, "apt_relabel_ranked: a call whose bids are placed needs neighbours");
+    const dim3 tiles = grid_for(continued ? num_neighbors : items, kMbTile, int64_t{1} << 30);
+    if (continued != 0) {
+      if (unique != seeds)
+        APT_HIP(hipMemcpyAsync(unique, seeds, sizeof(int64_t) * static_cast<size_t>(num_seeds), hipMemcpyDeviceToDevice, st));
+      hipLaunchKernelGGL(mb_count_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_count_kernel");
+      hipLaunchKernelGGL(mb_place_kernel<false>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_place_kernel");
+    } else {
+      hipLaunchKernelGGL(mb_count_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_count_kernel");
+      hipLaunchKernelGGL(mb_place_kernel<true>, tiles, dim3(kMbBlock), 0, st, hp);
+      APT_LAUNCH_CHECK("mb_place_kernel");
+    }
+  } else if (continued == 0) {
     // a new batch of the table: next epoch (refill when they have run out); *num_unique_dev = num_seeds for now
     const int64_t vecs = static_cast<int64_t>(table_state_offset(rank_table_len) / 16);
     hipLaunchKernelGGL(mb_begin_kernel, dim3(kBeginBlocks), dim3(kMbBlock), 0, st, static_cast<uint4*>(rank_table), vecs,

@@ -27,6 +27,15 @@ struct RankTable {
   uint8_t* displaced;       // per slot of the current hop: set when a smaller bid took the node over
 };
 
+// What the sampling kernel needs to do the rank-table step for every id it has just loaded (the marking fused
+// into sampling).
+struct SampleMark {
+  RankTable table;
+  int64_t* relabeled;          // [rows * fanout]: receives the slot states / ids of rank_table_bid
+  int first_hop;               // the frontier rows bid for their nodes too (with their row index)
+  int64_t* outside = nullptr;  // optional, first hop: counts the frontier ids the table cannot hold
+};
+
 // Smallest entry value of the current batch.
 __device__ __forceinline__ uint32_t table_base(const uint32_t* state) { return state[0] << state[1]; }
 

@@ -27,13 +27,6 @@ namespace apt {
 static thread_local hipEvent_t t_sample_start = nullptr, t_sample_stop = nullptr;
 static thread_local int t_sample_hop = -1;
 
-// Arguments of the fused relabel marking (see SampleParams).
-struct SampleMark {
-  RankTable table;
-  int64_t* relabeled;
-  int first_hop;
-};
-
 struct SampleParams {
   apt_graph g;
   const int64_t* frontier;
@@ -53,6 +46,7 @@ struct SampleParams {
   RankTable table;       // entries == NULL: plain sampling
   int64_t* relabeled;    // [n * fanout]
   int first_hop;
+  int64_t* outside;      // optional, first hop: counts the frontier ids the table cannot hold (>= table.len)
 };
 
 constexpr int kSampleBlock = 512;
@@ -207,8 +201,10 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
           }
           // First hop of the fused driver: the row's seed bids for its node with
           // its own index, like its neighbours below (seeds may repeat).
-          if (p.first_hop != 0 && p.table.entries != nullptr && l == 0 && node >= 0 && node < p.table.len)
-            atomicMin(&p.table.entries[node], ep.base + static_cast<uint32_t>(gis[u]));
+          if (p.first_hop != 0 && p.table.entries != nullptr && l == 0 && node >= 0) {
+            if (node < p.table.len) atomicMin(&p.table.entries[node], ep.base + static_cast<uint32_t>(gis[u]));
+            else if (p.outside != nullptr) atomicAdd(reinterpret_cast<unsigned long long*>(p.outside), 1ull);
+          }
           pos[u] = slot_position<LPS, REPLACE>(l, fanout, deg, node, seed, p.hop);
           if (l == 0) {
             const int64_t cnt = REPLACE ? (deg > 0 ? fanout : 0) : (deg < fanout ? deg : fanout);
@@ -390,6 +386,7 @@ int sample_launch(const apt_graph* graph, const int64_t* frontier, int64_t num_f
     p.table = mark->table;
     p.relabeled = mark->relabeled;
     p.first_hop = mark->first_hop;
+    p.outside = mark->outside;
   }
 
   // Lanes per frontier row: the smallest power of two that holds the fanout

@@ -63,6 +63,15 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
   Tensor ranked_table, ranked_ws, ranked_counts, ranked_last;
   uint32_t ranked_last_version = 0;
   bool ranked_enabled = true;
+  // A sampling operator call that has placed the bids of the relabel_csc call the reference's sampler makes
+  // next (apt_sample_neighbors_bidding): its seeds and sampled ids (kept alive, with their versions) and the slot
+  // states that call will take over.  A relabel_csc with other tensors finds abandoned bids in the table and
+  // starts a fresh batch.
+  struct RankedPending {
+    bool valid = false, continued = false;
+    Tensor seeds, neighbors, states;
+    uint32_t seeds_version = 0, neighbors_version = 0;
+  } ranked_pending;
   // pinned host words that the relabel operators read their counts into (a copy to pageable memory is staged)
   Tensor pinned_counts;
   // fused multi-hop driver: rank table of the registered graph, workspace of the last plan
@@ -163,9 +172,11 @@ void SetMissCheck(std::string mode) {
 
 // relabel_csc goes through the registered graph's rank table where it can (default) or always through the
 // hash table (false).
+static void drop_pending_bids();
 void SetRankedRelabel(bool enabled) {
   S().ranked_enabled = enabled;
   S().ranked_last = Tensor();
+  drop_pending_bids();
 }
 
 // How many registry-owned sets of output buffers sample_blocks hands out in turn.  0 (the default) = fresh
@@ -247,7 +258,9 @@ void MixCacheGraphs(IdType num_cached_nodes, Tensor cached_node_idx, Tensor cach
   s.graph.num_total_nodes = total;
   s.rank_table = Tensor();
   s.ranked_table = Tensor();
+  s.ranked_ws = Tensor();
   s.ranked_last = Tensor();
+  s.ranked_pending = {};
   s.adj_pos_map = Tensor();
   if (num_cached_nodes > 0) {
     auto idx = ids_on_device(cached_node_idx, "cached_node_idx");
@@ -283,7 +296,9 @@ void RegisterGraphPartition(Tensor indptr, Tensor indices, IdType row_begin, IdT
   s.graph.num_total_nodes = num_total_nodes;
   s.rank_table = Tensor();
   s.ranked_table = Tensor();
+  s.ranked_ws = Tensor();
   s.ranked_last = Tensor();
+  s.ranked_pending = {};
   s.has_graph = true;
 }
 
@@ -300,6 +315,79 @@ void RegisterMultiMachinesScheme(Tensor remote_worker_map, Tensor remote_worker_
 }
 
 // ---------------------------------------------------------------- hot path
+static bool same_tensor(const Tensor& kept, uint32_t version, const Tensor& t) {
+  return kept.defined() && kept.data_ptr() == t.data_ptr() && kept.numel() == t.numel() && version == t._version();
+}
+
+// Forgets bids that a sampling call placed for a relabel_csc call that did not come.  Those of a call that
+// continued a batch have also set per-slot flags in the workspace, which only that relabel_csc would have
+// consumed: the workspace is cleared.  (The bids themselves are harmless: the next call on the table starts a new
+// batch.)
+static void drop_pending_bids() {
+  auto& s = S();
+  if (s.ranked_pending.valid && s.ranked_pending.continued && s.ranked_ws.defined())
+    check(apt_minibatch_workspace_init(s.ranked_ws.data_ptr(), static_cast<size_t>(s.ranked_ws.numel()), stream()));
+  s.ranked_pending = {};
+}
+
+// The rank table of the registered graph for relabel_csc (a table of its own) and a workspace for `items` items.
+static bool ranked_resources(int64_t items) {
+  auto& s = S();
+  auto u8 = torch::TensorOptions().dtype(torch::kUInt8).device(device());
+  if (!s.ranked_table.defined()) {
+    const size_t bytes = apt_rank_table_bytes(s.graph.num_total_nodes);
+    if (bytes == 0) return false;
+    s.ranked_table = torch::empty({static_cast<int64_t>(bytes)}, u8);
+    check(apt_rank_table_init(s.ranked_table.data_ptr(), bytes, stream()));
+    s.ranked_counts = torch::zeros({2}, i64_opts());
+    s.ranked_last = Tensor();
+    s.ranked_pending = {};
+  }
+  const size_t need = apt_relabel_ranked_workspace_bytes(items);
+  if (need == 0) return false;
+  if (!s.ranked_ws.defined() || static_cast<size_t>(s.ranked_ws.numel()) < need) {
+    // (a new workspace starts with clean flags; bids placed under the old one are abandoned)
+    s.ranked_ws = torch::empty({static_cast<int64_t>(std::max<size_t>(need, 256) * 2)}, u8);
+    check(apt_minibatch_workspace_init(s.ranked_ws.data_ptr(), static_cast<size_t>(s.ranked_ws.numel()), stream()));
+    s.ranked_last = Tensor();
+    s.ranked_pending = {};
+  }
+  return true;
+}
+
+// One hop of sampling.  Where the relabel_csc call that the reference's sampler makes next
+// (python/npc/sampler.py:187-203) will go through the rank table, its bids are placed here, by the sampling kernel
+// itself, and that call only ranks the owners.
+static void sample_hop(const Tensor& f, IdType fanout, bool replace, uint64_t rng_seed, int hop, Tensor& out,
+                       int64_t* counts) {
+  auto& s = S();
+  const int64_t n = f.numel(), items = n + n * fanout;
+  if (s.ranked_enabled && fanout <= 64 && items > 8192 && items <= apt_relabel_ranked_max_items() &&
+      s.graph.num_total_nodes > 0 && ranked_resources(items)) {
+    // the batch continues if these seeds are the unique list the last relabel_csc returned and nothing has bid since
+    const bool continued = !s.ranked_pending.valid && same_tensor(s.ranked_last, s.ranked_last_version, f);
+    s.ranked_last = Tensor();
+    drop_pending_bids();
+    auto states = torch::empty({n * fanout}, i64_opts());
+    check(apt_sample_neighbors_bidding(&s.graph, i64(f), n, nullptr, static_cast<int>(fanout), replace, rng_seed, hop,
+                                       out.data_ptr<int64_t>(), counts, nullptr, continued ? 1 : 0,
+                                       s.ranked_table.data_ptr(), s.graph.num_total_nodes, states.data_ptr<int64_t>(),
+                                       s.ranked_counts.data_ptr<int64_t>() + 1, s.ranked_ws.data_ptr(),
+                                       static_cast<size_t>(s.ranked_ws.numel()), stream()));
+    auto& p = s.ranked_pending;
+    p.valid = true;
+    p.continued = continued;
+    p.seeds = f;
+    p.neighbors = out;
+    p.states = states;
+    p.seeds_version = f._version();
+    p.neighbors_version = out._version();
+    return;
+  }
+  check(apt_sample_neighbors(&s.graph, i64(f), n, nullptr, static_cast<int>(fanout), replace, rng_seed, hop,
+                             out.data_ptr<int64_t>(), counts, nullptr, stream()));
+}
+
 std::tuple<Tensor, Tensor> SampleNeighbors(Tensor seeds, IdType fanout, bool replace, IdType rng_seed,
                                            IdType hop) {
   auto& s = S();
@@ -308,9 +396,7 @@ std::tuple<Tensor, Tensor> SampleNeighbors(Tensor seeds, IdType fanout, bool rep
   auto f = ids_on_device(seeds, "seeds");
   auto out = torch::empty({f.numel() * fanout}, i64_opts());
   auto cnt = torch::empty({f.numel()}, i64_opts());
-  check(apt_sample_neighbors(&s.graph, i64(f), f.numel(), nullptr, static_cast<int>(fanout), replace,
-                             static_cast<uint64_t>(rng_seed), static_cast<int>(hop),
-                             out.data_ptr<int64_t>(), cnt.data_ptr<int64_t>(), nullptr, stream()));
+  sample_hop(f, fanout, replace, static_cast<uint64_t>(rng_seed), static_cast<int>(hop), out, cnt.data_ptr<int64_t>());
   return {out, cnt};
 }
 
@@ -487,9 +573,7 @@ std::vector<Tensor> LocalSamplingNeibhorsOneLayer(Tensor seeds, IdType fanout) {
   TORCH_CHECK(fanout > 0, "npc: fanout must be > 0");
   auto f = ids_on_device(seeds, "seeds");
   auto out = torch::empty({f.numel() * fanout}, i64_opts());
-  check(apt_sample_neighbors(&s.graph, i64(f), f.numel(), nullptr, static_cast<int>(fanout), 1,
-                             s.rng_seed, static_cast<int>(s.sample_calls), out.data_ptr<int64_t>(),
-                             nullptr, nullptr, stream()));
+  sample_hop(f, fanout, true, s.rng_seed, static_cast<int>(s.sample_calls), out, nullptr);
   s.sample_calls += 1;
   return {f, out};
 }
@@ -502,29 +586,23 @@ static bool RelabelRanked(const Tensor& sd, const Tensor& nb, Tensor& unique, Te
   auto& s = S();
   const int64_t items = sd.numel() + nb.numel();
   const int64_t len = s.graph.num_total_nodes;
-  auto u8 = torch::TensorOptions().dtype(torch::kUInt8).device(device());
-  if (!s.ranked_table.defined()) {
-    const size_t bytes = apt_rank_table_bytes(len);
-    if (bytes == 0) return false;
-    s.ranked_table = torch::empty({static_cast<int64_t>(bytes)}, u8);
-    check(apt_rank_table_init(s.ranked_table.data_ptr(), bytes, stream()));
-    s.ranked_counts = torch::zeros({2}, i64_opts());
-    s.ranked_last = Tensor();
-  }
-  const size_t need = apt_relabel_ranked_workspace_bytes(items);
-  if (!s.ranked_ws.defined() || static_cast<size_t>(s.ranked_ws.numel()) < need) {
-    s.ranked_ws = torch::empty({static_cast<int64_t>(std::max<size_t>(need, 256) * 2)}, u8);
-    check(apt_minibatch_workspace_init(s.ranked_ws.data_ptr(), static_cast<size_t>(s.ranked_ws.numel()), stream()));
-  }
-  const bool continued = s.ranked_last.defined() && s.ranked_last.data_ptr() == sd.data_ptr() &&
-                         s.ranked_last.numel() == sd.numel() && s.ranked_last_version == sd._version();
+  if (!ranked_resources(items)) return false;
+  // bids placed by the sampling call for exactly these tensors?  Bids placed for others are abandoned: the table's
+  // batch cannot be continued then.
+  auto& p = s.ranked_pending;
+  const bool marked = p.valid && nb.numel() > 0 && same_tensor(p.neighbors, p.neighbors_version, nb) &&
+                      same_tensor(p.seeds, p.seeds_version, sd);
+  const bool continued = marked ? p.continued
+                                : !p.valid && same_tensor(s.ranked_last, s.ranked_last_version, sd);
   s.ranked_last = Tensor();
   unique = torch::empty({items}, i64_opts());
-  relabeled = torch::empty({nb.numel()}, i64_opts());
+  relabeled = marked ? p.states : torch::empty({nb.numel()}, i64_opts());
+  if (marked) s.ranked_pending = {};
+  else drop_pending_bids();
   int64_t* host = pinned_counts();
   host[0] = host[1] = -1;
   // ranked_counts[1] counts ids beyond the graph; it is zero unless the previous call found some
-  check(apt_relabel_ranked(i64(sd), sd.numel(), nullptr, i64(nb), nb.numel(), 0, continued ? 1 : 0,
+  check(apt_relabel_ranked(i64(sd), sd.numel(), nullptr, i64(nb), nb.numel(), 0, (continued ? 1 : 0) | (marked ? 2 : 0),
                            s.ranked_table.data_ptr(), len,
                            unique.data_ptr<int64_t>(), nb.numel() ? relabeled.data_ptr<int64_t>() : nullptr,
                            s.ranked_counts.data_ptr<int64_t>(), s.ranked_counts.data_ptr<int64_t>() + 1, host,
@@ -532,6 +610,7 @@ static bool RelabelRanked(const Tensor& sd, const Tensor& nb, Tensor& unique, Te
                            static_cast<size_t>(s.ranked_ws.numel()), stream()));
   if (host[1] != 0) {  // ids beyond the graph: not a valid relabel, and the table's batch is not continued
     s.ranked_counts.zero_();
+    relabeled = Tensor();
     return false;
   }
   unique = unique.narrow(0, 0, host[0]);
@@ -554,6 +633,10 @@ std::vector<Tensor> RelabelCSC(Tensor seeds, Tensor neighbors) {
     if (RelabelRanked(sd, nb, unique, relabeled)) return {unique, relabeled};
   }
   s.ranked_last = Tensor();
+  if (s.ranked_pending.valid) {   // a sampling call has counted ids beyond the graph, or its bids are not used
+    drop_pending_bids();
+    if (s.ranked_counts.defined()) s.ranked_counts.zero_();
+  }
   const size_t need = apt_relabel_workspace_bytes(items);
   TORCH_CHECK(need > 0, "npc: relabel_csc: ", items, " items exceed the supported maximum");
   auto ws = torch::empty({static_cast<int64_t>(need)}, torch::TensorOptions().dtype(torch::kUInt8).device(device()));

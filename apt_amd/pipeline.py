@@ -40,7 +40,9 @@ class MiniBatchPipeline:
         is what follows the sampling (fused driver, features gathered, no requests, no formats).
 
         relabel (per-hop driver, fused=False): "hash" = apt_relabel's hash table per hop; "ranked" =
-        apt_relabel_ranked, the per-hop calls through a node-indexed rank table, later hops continuing the batch.
+        apt_relabel_ranked, the per-hop calls through a node-indexed rank table, later hops continuing the batch;
+        "ranked_bidding" = the same with the table's bids placed by the sampling call of the hop
+        (apt_sample_neighbors_bidding; fanouts up to 64, wider hops fall back to "ranked").
 
         table: the rank table of another pipeline (fused driver) whose batches run on the same stream as this
         one's: batches that follow each other on one stream can share a table (444 MB at 111 M nodes).
@@ -73,9 +75,10 @@ class MiniBatchPipeline:
             self.frontier = [None] + [torch.empty(self.caps[h + 1], **i64) for h in range(H)]
             # sizes[h] = rows of the frontier entering hop h; sizes[H] = input nodes; then edges
             self.sizes = torch.zeros(H + 2, **i64)
-            if relabel not in ("hash", "ranked"):
-                raise ValueError("relabel must be 'hash' or 'ranked'")
-            self.ranked = capi.RankedRelabel(graph.num_total_nodes, dev) if relabel == "ranked" else None
+            if relabel not in ("hash", "ranked", "ranked_bidding"):
+                raise ValueError("relabel must be 'hash', 'ranked' or 'ranked_bidding'")
+            self.ranked = capi.RankedRelabel(graph.num_total_nodes, dev) if relabel != "hash" else None
+            self.bid_in_sampler = relabel == "ranked_bidding"
             self.ranked_outside = torch.zeros(1, **i64)    # ids the rank table cannot hold (stays 0 for a valid graph)
             self.workspace = torch.empty(capi.relabel_workspace_bytes(self.caps[-1]), dtype=torch.uint8,
                                          device=dev)
@@ -128,6 +131,17 @@ class MiniBatchPipeline:
         total = self.sizes[-1:]
         for h, f in enumerate(self.fanouts):
             n_dev = None if h == 0 else self._size(h)
+            if self.ranked is not None and self.bid_in_sampler and f <= 64:
+                # the sampler places the relabel's bids on the way (what the operators do for the reference's
+                # per-hop calls)
+                self.ranked.sample_bidding(self.graph, self.frontier[h], f, self.replace, rng_seed, h, h > 0,
+                                           self.neighbors[h], self.relabeled[h], num_frontier_dev=n_dev,
+                                           out_counts=self.counts[h], out_total=total,
+                                           num_outside_dev=self.ranked_outside)
+                self.ranked.enqueue(self.frontier[h], self.neighbors[h], h > 0, self.frontier[h + 1], self.relabeled[h],
+                                    self._size(h + 1), self.ranked_outside, num_seeds_dev=n_dev, neighbor_stride=f,
+                                    bids_placed=True)
+                continue
             capi.sample_neighbors(self.graph, self.frontier[h], f, self.replace, rng_seed, h,
                                   num_frontier_dev=n_dev, out_neighbors=self.neighbors[h],
                                   out_counts=self.counts[h], out_total=total)

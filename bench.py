@@ -88,11 +88,12 @@ def parse_args():
                     help="seconds of CPU-oracle work for the cpu_baseline leg (0 = skip, also skips its parity check)")
     ap.add_argument("--cpu_threads", type=int, default=None)
     ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused", "unfused_hash"],
+    ap.add_argument("--driver", default="fused", choices=["graph", "fused", "unfused", "unfused_pass", "unfused_hash"],
                     help="graph: fused C driver replayed as a HIP graph; fused: same, launched eagerly; "
                          "unfused: the reference's call pattern, a sampling call and a relabel call per hop, the "
-                         "relabel through the graph's rank table (apt_relabel_ranked); unfused_hash: the same with the "
-                         "hash-table relabel (apt_relabel)")
+                         "relabel through the graph's rank table with its bids placed by the sampling call "
+                         "(apt_sample_neighbors_bidding + apt_relabel_ranked); unfused_pass: the same with the bids "
+                         "as a pass of the relabel call; unfused_hash: with the hash-table relabel (apt_relabel)")
     ap.add_argument("--inflight", type=int, default=4,
                     help="after the timed single-stream region, also run the K batches with N of them in "
                          "flight (N pipelines on N HIP streams) and report it under stages.in_flight; 1 = skip")
@@ -269,7 +270,7 @@ def driver_kw(args):
     """MiniBatchPipeline arguments of --driver."""
     if args.driver in ("fused", "graph"):
         return dict(fused=True)
-    return dict(fused=False, relabel="ranked" if args.driver == "unfused" else "hash")
+    return dict(fused=False, relabel={"unfused": "ranked_bidding", "unfused_pass": "ranked"}.get(args.driver, "hash"))
 
 
 def make_seed_sets(ctx, wl, B, count, seed):

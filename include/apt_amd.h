@@ -186,6 +186,11 @@ int apt_relabel(const int64_t* seeds, int64_t num_seeds,
  *                 (same values, same order, no other call on the table since):
  *                 the table still holds their ids, so only the neighbours are
  *                 looked up or bid for.  The result is what a fresh call gives.
+ *                 Bit 1 (values 2 and 3, for a fresh and a continued call): the
+ *                 neighbours come from apt_sample_neighbors_bidding, which has
+ *                 placed this call's bids already and left the slot states in
+ *                 `relabeled` (in / out then); same table, same workspace, same
+ *                 seeds, no other call on the table in between; num_neighbors > 0.
  *   unique        device int64[num_seeds + num_neighbors] capacity
  *   num_unique_dev   device int64[1], receives the number of unique ids
  *   num_outside_dev  device int64[1], incremented once per id that the table
@@ -209,6 +214,35 @@ int apt_relabel_ranked(const int64_t* seeds, int64_t num_seeds, const int64_t* n
                        int64_t* num_unique_dev, int64_t* num_outside_dev,
                        int64_t* counts_host, void* workspace,
                        size_t workspace_bytes, void* stream);
+
+/* apt_sample_neighbors (src/sampling.cc:13-17) that places the rank-table bids of
+ * the apt_relabel_ranked call that follows on the way (the reference's sampler
+ * calls the two back to back per hop, python/npc/sampler.py:187-203): the
+ * sampling kernel has every id in registers, and a bid placed there overlaps
+ * with its own random reads.  Sampled ids are those of apt_sample_neighbors.
+ *   fanout          at most 64
+ *   continued       0: the frontier starts a batch (its rows bid for their nodes
+ *                   too).  != 0: the frontier is the unique list the previous
+ *                   apt_relabel_ranked on this table wrote, as for that call
+ *   slot_states     device int64[num_frontier * fanout]: pass it as `relabeled`
+ *                   to apt_relabel_ranked with bit 1 of `continued` set
+ *   num_outside_dev optional device int64[1]: incremented per frontier id that
+ *                   the table cannot hold (fresh calls; the caller clears it)
+ *   workspace       the workspace of that apt_relabel_ranked call
+ * A call that is not followed by its apt_relabel_ranked leaves bids of an
+ * abandoned batch in the table: the next call on the table must then be a fresh
+ * one (continued == 0), which ignores them; and, if the abandoned call was a
+ * continued one, flags in the workspace that only its apt_relabel_ranked would
+ * have consumed: the workspace is then cleared again with
+ * apt_minibatch_workspace_init. */
+int apt_sample_neighbors_bidding(const apt_graph* graph, const int64_t* frontier,
+                                 int64_t num_frontier, const int64_t* num_frontier_dev,
+                                 int fanout, int replace, uint64_t rng_seed, int hop,
+                                 int64_t* out_neighbors, int64_t* out_counts,
+                                 int64_t* out_total, int continued, void* rank_table,
+                                 int64_t rank_table_len, int64_t* slot_states,
+                                 int64_t* num_outside_dev, void* workspace,
+                                 size_t workspace_bytes, void* stream);
 
 /* apt_relabel without a workspace argument and without any allocation.
  * No counterpart in the reference.  It is for callers that cannot allocate:

@@ -193,13 +193,15 @@ def test_full_scale_vs_oracle(orc, capi, full):
     try:
         for replace in (False, True):
             pipes = [MiniBatchPipeline(graph, store, 4096, hops, replace=replace),
-                     MiniBatchPipeline(graph, None, 4096, hops, replace=replace, gather=False, fused=False)]
+                     MiniBatchPipeline(graph, None, 4096, hops, replace=replace, gather=False, fused=False),
+                     MiniBatchPipeline(graph, None, 4096, hops, replace=replace, gather=False, fused=False,
+                                       relabel="ranked_bidding")]
             for batch in range(2):
                 seeds = torch.randperm(FULL_N, generator=gen, device=DEV)[:4096].contiguous()
                 key = 31337 + 10 * batch + int(replace)
                 want_in, want_blocks = orc.sample_blocks(og, seeds.cpu().numpy(), hops, replace, key)
                 assert sum(int(b["counts"].sum()) for b in want_blocks) > 500_000
-                for pipe in pipes[:1 if batch else 2]:
+                for pipe in pipes[:1 if batch else 3]:
                     pipe.run(seeds, key)
                     res = pipe.result()
                     assert np.array_equal(res["input_nodes"].cpu().numpy(), want_in)
@@ -303,6 +305,8 @@ def test_fused_and_per_hop_drivers_agree_over_many_batches(capi):
     fused = MiniBatchPipeline(graph, None, 1024, hops, gather=False)
     per_hop = MiniBatchPipeline(graph, None, 1024, hops, gather=False, fused=False)
     ranked = MiniBatchPipeline(graph, None, 1024, hops, gather=False, fused=False, relabel="ranked")
+    # ... and the same with the bids placed by each hop's sampling call (apt_sample_neighbors_bidding)
+    bidding = MiniBatchPipeline(graph, None, 1024, hops, gather=False, fused=False, relabel="ranked_bidding")
     gen = torch.Generator(device=DEV)
     gen.manual_seed(21)
     for batch in range(300):
@@ -310,11 +314,12 @@ def test_fused_and_per_hop_drivers_agree_over_many_batches(capi):
         fused.run(seeds, 9000 + batch)
         per_hop.run(seeds, 9000 + batch)
         ranked.run(seeds, 9000 + batch)
+        bidding.run(seeds, 9000 + batch)
         a = fused.result()
-        for other in (per_hop, ranked):
+        for other in (per_hop, ranked, bidding):
             b = other.result()
             assert a["sizes"] == b["sizes"], batch
             assert torch.equal(a["input_nodes"], b["input_nodes"]), batch
             for x, y in zip(a["blocks"], b["blocks"]):
                 assert torch.equal(x["relabeled"], y["relabeled"]) and torch.equal(x["neighbors"], y["neighbors"]), batch
-        assert int(ranked.ranked_outside) == 0
+        assert int(ranked.ranked_outside) == 0 and int(bidding.ranked_outside) == 0

@@ -19,7 +19,7 @@ def _setup(orc, capi, n=30000, deg=14, dim=100, seed=21):
     return indptr, indices, feats
 
 
-@pytest.mark.parametrize("mode", ["fused", "graph", "unfused"])
+@pytest.mark.parametrize("mode", ["fused", "graph", "unfused", "unfused_ranked", "unfused_ranked_bidding"])
 @pytest.mark.parametrize("replace", [False, True])
 def test_pipeline_matches_oracle_driver(orc, capi, replace, mode):
     from apt_amd.pipeline import MiniBatchPipeline
@@ -28,8 +28,8 @@ def test_pipeline_matches_oracle_driver(orc, capi, replace, mode):
     dg = capi.Graph(dev(indptr), dev(indices))
     fs = capi.FeatStore(dev(feats))
     hops = [5, 10, 15]
-    pipe = MiniBatchPipeline(dg, fs, 512, hops, replace=replace, fused=mode != "unfused",
-                             use_graph=mode == "graph")
+    pipe = MiniBatchPipeline(dg, fs, 512, hops, replace=replace, fused=not mode.startswith("unfused"),
+                             use_graph=mode == "graph", relabel=mode[len("unfused_"):] or "hash")
     rng = np.random.default_rng(0)
     for batch in range(4):                                   # buffers (and the graph) are reused
         seeds = rng.permutation(len(indptr) - 1)[:512]
@@ -155,6 +155,64 @@ def test_operator_relabel_csc_uses_the_rank_table_and_falls_back(orc, capi):
                     u, r = npc.ops.tensor_relabel_csc(frontier, dev(nbrs))
                     assert np.array_equal(u.cpu().numpy(), want_u) and np.array_equal(r.cpu().numpy(), want_r), (ranked, chain, f)
                     frontier = u
+    finally:
+        npc.ops.set_ranked_relabel(True)
+
+
+def test_operator_sampling_places_the_bids_of_the_relabel_that_follows(orc, capi):
+    """The reference's per-hop pattern through the operators (python/npc/sampler.py:187-203): local_sample_one_layer
+    or sample_neighbors, then relabel_csc on the same tensors, the unique list being the next hop's seeds.  The
+    sampling operator places the relabel's bids; everything else a caller may do in between -- relabel other
+    tensors, sample twice, change the sampled ids in place, pass seeds the graph does not have, switch the rank
+    table off -- must give the oracle's answer too."""
+    import apt_amd as npc
+    indptr, indices, feats = _setup(orc, capi, n=60_000, deg=12, dim=8, seed=16)
+    n = len(indptr) - 1
+    og = orc.Graph(indptr, indices)
+    npc.set_topology(0, 1)
+    e = torch.empty(0, dtype=torch.int64)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
+    rng = np.random.default_rng(9)
+
+    def check_relabel(frontier, nbrs, tag):
+        want_u, want_r = orc.relabel(frontier.cpu().numpy(), nbrs.cpu().numpy())
+        u, r = npc.ops.tensor_relabel_csc(frontier, nbrs)
+        assert np.array_equal(u.cpu().numpy(), want_u), tag
+        assert np.array_equal(r.cpu().numpy(), want_r), tag
+        return u
+
+    def check_sample(frontier, f, replace, key, hop, tag):
+        nbrs, cnt = npc.ops.sample_neighbors(frontier, f, replace, key, hop)
+        want_n, want_c = orc.sample_neighbors(og, frontier.cpu().numpy(), f, replace, key, hop)
+        assert np.array_equal(nbrs.cpu().numpy(), want_n) and np.array_equal(cnt.cpu().numpy(), want_c), tag
+        return nbrs
+
+    try:
+        for ranked in (True, False, True):
+            npc.ops.set_ranked_relabel(ranked)
+            for chain, replace in enumerate((False, True, False, False, False, False)):
+                frontier = dev(rng.integers(0, n, 2500))             # repeated seeds happen
+                if chain == 5:
+                    frontier[7] = n + 5                              # a seed the graph does not have
+                for hop, f in enumerate((5, 6, 4)):
+                    tag = (ranked, chain, hop)
+                    nbrs = check_sample(frontier, f, replace, 700 + chain, hop, tag)
+                    if chain == 2 and hop == 1:
+                        nbrs = check_sample(frontier, f, replace, 900, hop, tag)        # sampled twice: the first bids are dropped
+                    if chain == 3 and hop == 1:
+                        other = dev(rng.integers(0, n, 30_000))                         # a relabel of other tensors in between
+                        check_relabel(dev(rng.integers(0, n, 4000)), other, tag)
+                    if chain == 4 and hop == 2:
+                        nbrs[11] = nbrs[12]                                             # changed in place: not what was bid for
+                    frontier = check_relabel(frontier, nbrs, tag)
+        # the reference's own operator: with replacement, keyed by the call counter
+        npc.set_rng_seed(77)
+        frontier = dev(rng.permutation(n)[:3000])
+        for hop, f in enumerate((5, 5)):
+            seeds_out, nbrs = npc.ops.local_sample_one_layer(frontier, f)
+            want_n, _ = orc.sample_neighbors(og, frontier.cpu().numpy(), f, True, 77, hop)
+            assert np.array_equal(nbrs.cpu().numpy(), want_n)
+            frontier = check_relabel(seeds_out, nbrs, ("one_layer", hop))
     finally:
         npc.ops.set_ranked_relabel(True)
 
