@@ -327,6 +327,7 @@ static void drop_pending_bids() {
   auto& s = S();
   if (s.ranked_pending.valid && s.ranked_pending.continued && s.ranked_ws.defined())
     check(apt_minibatch_workspace_init(s.ranked_ws.data_ptr(), static_cast<size_t>(s.ranked_ws.numel()), stream()));
+  if (s.ranked_pending.valid && s.ranked_counts.defined()) s.ranked_counts.zero_();   // seeds it counted as outside
   s.ranked_pending = {};
 }
 
