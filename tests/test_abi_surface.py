@@ -204,3 +204,27 @@ def test_epoch_driver_argument_checks_need_no_gpu():
     assert L.apt_epoch_next(None, None, None, None) != 0 and L.apt_epoch_release(None, None) != 0
     assert L.apt_epoch_begin(None, None, 0, 0, None) != 0 and L.apt_epoch_end(None) != 0
     assert L.apt_epoch_destroy(None) == 0
+
+
+def test_bidding_sampler_argument_checks_need_no_gpu():
+    """apt_sample_neighbors_bidding rejects what it cannot do before it touches the GPU."""
+    from apt_amd import capi
+    L = capi.lib()
+    g = capi.CGraph()
+    table = ctypes.c_void_p(256)                      # never dereferenced by the checks
+    assert L.apt_sample_neighbors_bidding(ctypes.byref(g), None, 10, None, 65, 0, 1, 0, None, None, None, 0, table, 100,
+                                          ctypes.c_void_p(8), None, ctypes.c_void_p(16), 1 << 20, None) != 0
+    assert b"fanout" in L.apt_last_error()
+    assert L.apt_sample_neighbors_bidding(ctypes.byref(g), None, 10, None, 5, 0, 1, 0, None, None, None, 0, table, 100,
+                                          None, None, ctypes.c_void_p(16), 1 << 20, None) != 0
+    assert b"slot_states" in L.apt_last_error()
+    assert L.apt_sample_neighbors_bidding(ctypes.byref(g), None, 10, None, 5, 0, 1, 0, None, None, None, 0, None, 100,
+                                          ctypes.c_void_p(8), None, ctypes.c_void_p(16), 1 << 20, None) != 0
+    assert b"rank table" in L.apt_last_error()
+    assert L.apt_sample_neighbors_bidding(ctypes.byref(g), None, 10, None, 5, 0, 1, 0, None, None, None, 0, table, 100,
+                                          ctypes.c_void_p(8), None, ctypes.c_void_p(16), 8, None) != 0
+    assert b"workspace" in L.apt_last_error()
+    # apt_relabel_ranked: a call that takes placed bids over needs neighbours
+    assert L.apt_relabel_ranked(ctypes.c_void_p(8), 4, None, None, 0, 0, 2, table, 100, ctypes.c_void_p(8), None,
+                                ctypes.c_void_p(8), ctypes.c_void_p(16), None, ctypes.c_void_p(16), 1 << 20, None) != 0
+    assert b"neighbours" in L.apt_last_error()
