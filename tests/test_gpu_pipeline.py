@@ -217,6 +217,56 @@ def test_operator_sampling_places_the_bids_of_the_relabel_that_follows(orc, capi
         npc.ops.set_ranked_relabel(True)
 
 
+def test_operator_sequences_at_random(orc, capi):
+    """Random sequences of the sampling and relabel operators on a registered graph -- chains as the reference's
+    sampler makes them, chains broken off, relabels of unrelated tensors, repeated sampling, ids changed in place,
+    small and large inputs, the rank table switched off and on -- every result against the oracle.  The operators
+    keep state between calls (the rank table's batch, bids placed ahead of relabel_csc); no sequence may show it."""
+    import apt_amd as npc
+    indptr, indices, feats = _setup(orc, capi, n=40_000, deg=10, dim=8, seed=23)
+    n = len(indptr) - 1
+    og = orc.Graph(indptr, indices)
+    npc.set_topology(0, 1)
+    e = torch.empty(0, dtype=torch.int64)
+    npc.mix_cache_graphs(0, e, e, e, torch.from_numpy(indptr), torch.from_numpy(indices))
+    rng = np.random.default_rng(31)
+    frontier = nbrs = None
+    key = 0
+    try:
+        for step in range(260):
+            what = rng.choice(["seeds", "sample", "sample", "relabel", "relabel", "other", "poke", "toggle"],
+                              p=[0.14, 0.2, 0.2, 0.17, 0.17, 0.06, 0.04, 0.02])
+            if what == "seeds" or frontier is None:
+                frontier = dev(rng.integers(0, n, int(rng.choice([300, 1500, 2600, 4000]))))
+                nbrs = None
+            elif what == "sample":
+                f = int(rng.choice([3, 5, 8]))
+                replace = bool(rng.integers(0, 2))
+                key += 1
+                nbrs, cnt = npc.ops.sample_neighbors(frontier, f, replace, key, step % 5)
+                want_n, want_c = orc.sample_neighbors(og, frontier.cpu().numpy(), f, replace, key, step % 5)
+                assert np.array_equal(nbrs.cpu().numpy(), want_n) and np.array_equal(cnt.cpu().numpy(), want_c), step
+            elif what == "relabel" and nbrs is not None:
+                want_u, want_r = orc.relabel(frontier.cpu().numpy(), nbrs.cpu().numpy())
+                u, r = npc.ops.tensor_relabel_csc(frontier, nbrs)
+                assert np.array_equal(u.cpu().numpy(), want_u) and np.array_equal(r.cpu().numpy(), want_r), step
+                if u.numel() < 60_000:                           # the chain goes on from the unique list
+                    frontier, nbrs = u, None
+                else:
+                    frontier = nbrs = None
+            elif what == "other":
+                a, b = dev(rng.integers(0, n, 2000)), dev(rng.integers(-1, n, 15_000))
+                want_u, want_r = orc.relabel(a.cpu().numpy(), b.cpu().numpy())
+                u, r = npc.ops.tensor_relabel_csc(a, b)
+                assert np.array_equal(u.cpu().numpy(), want_u) and np.array_equal(r.cpu().numpy(), want_r), step
+            elif what == "poke" and nbrs is not None:
+                nbrs[int(rng.integers(0, nbrs.numel()))] = int(rng.integers(0, n))
+            elif what == "toggle":
+                npc.ops.set_ranked_relabel(bool(rng.integers(0, 2)))
+    finally:
+        npc.ops.set_ranked_relabel(True)
+
+
 def test_cpu_load_subtensor_rejects_ids_without_a_local_row(orc, capi):
     """Ids are checked on the host before anything is enqueued: a node outside the map, or one
     that has no local row (map entry -1, or a cache-only node), raises IndexError."""
