@@ -39,6 +39,12 @@ class CFeatStore(C.Structure):
 MAX_HOPS, MAX_SLOTS = 8, 16
 
 
+class CBlockBuffers(C.Structure):    # apt_block_buffers
+    _fields_ = [("coo_row", C.c_void_p), ("coo_col", C.c_void_p), ("csc_indptr", C.c_void_p),
+                ("csr_indptr", C.c_void_p), ("csr_indices", C.c_void_p), ("csr_eids", C.c_void_p),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
+
+
 class CBatchSlot(C.Structure):       # apt_batch_slot
     _fields_ = [("stream", C.c_void_p), ("nodes", C.c_void_p),
                 ("neighbors", C.c_void_p * MAX_HOPS), ("relabeled", C.c_void_p * MAX_HOPS),
@@ -46,7 +52,8 @@ class CBatchSlot(C.Structure):       # apt_batch_slot
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("features", C.c_void_p),
                 ("miss_count", C.c_void_p), ("request_sizes", C.c_void_p), ("request_offsets", C.c_void_p),
                 ("request_ids", C.c_void_p), ("request_perm", C.c_void_p), ("request_workspace", C.c_void_p),
-                ("request_workspace_bytes", C.c_size_t)]
+                ("request_workspace_bytes", C.c_size_t), ("blocks", CBlockBuffers * MAX_HOPS),
+                ("block_edges", C.c_void_p)]
 
 
 class CEpochDesc(C.Structure):       # apt_epoch_desc
@@ -54,7 +61,8 @@ class CEpochDesc(C.Structure):       # apt_epoch_desc
                 ("hop_fanouts", C.c_int * MAX_HOPS), ("replace", C.c_int), ("rank_table_len", C.c_int64),
                 ("has_requests", C.c_int), ("request_pos_map", C.c_void_p), ("request_num_total_nodes", C.c_int64),
                 ("remote_worker_map", C.c_void_p), ("min_vids", C.c_void_p), ("world_size", C.c_int),
-                ("num_remote_workers", C.c_int), ("num_slots", C.c_int), ("slots", CBatchSlot * MAX_SLOTS)]
+                ("num_remote_workers", C.c_int), ("formats", C.c_int), ("num_slots", C.c_int),
+                ("slots", CBatchSlot * MAX_SLOTS)]
 
 
 class CEpochCost(C.Structure):       # apt_epoch_cost
@@ -623,8 +631,8 @@ class MinibatchPlan:
 
 
 class EpochDriver:
-    """apt_epoch over the buffers of a list of MiniBatchPipeline objects (one slot each, fused driver, no
-    formats) and their streams.  The pipelines keep owning the buffers; this object must not outlive them."""
+    """apt_epoch over the buffers of a list of MiniBatchPipeline objects (one slot each, fused driver) and
+    their streams.  The pipelines keep owning the buffers; this object must not outlive them."""
 
     def __init__(self, pipes, streams):
         p0 = pipes[0]
@@ -646,6 +654,7 @@ class EpochDriver:
             d.request_num_total_nodes = rq["feat_pos_map"].numel()
             d.remote_worker_map, d.min_vids = rq["remote_worker_map"].data_ptr(), rq["min_vids"].data_ptr()
             d.world_size, d.num_remote_workers = int(rq["world_size"]), int(rq["num_remote_workers"])
+        d.formats = 1 if p0.formats is not None else 0
         d.num_slots = len(pipes)
         for k, (p, st) in enumerate(zip(pipes, streams)):
             s = d.slots[k]
@@ -662,13 +671,23 @@ class EpochDriver:
                 s.request_sizes, s.request_offsets = p.request_sizes.data_ptr(), p.request_offsets.data_ptr()
                 s.request_ids, s.request_perm = p.request_ids.data_ptr(), p.request_perm.data_ptr()
                 s.request_workspace, s.request_workspace_bytes = p.request_ws.data_ptr(), p.request_ws.numel()
+            if p.formats is not None:
+                s.block_edges = p.format_edges.data_ptr()
+                for h, f in enumerate(p.formats):
+                    b = s.blocks[h]
+                    b.coo_row, b.coo_col, b.csc_indptr = f.coo_row.data_ptr(), f.coo_col.data_ptr(), f.csc_indptr.data_ptr()
+                    if f.want_csr:
+                        b.csr_indptr, b.csr_indices = f.csr_indptr.data_ptr(), f.csr_indices.data_ptr()
+                        b.csr_eids = f.csr_eids.data_ptr()
+                    b.workspace, b.workspace_bytes = f.workspace.data_ptr(), f.workspace.numel()
         self._desc, self._keep = d, (pipes, streams)
         self.num_hops = H
+        self.formats = bool(d.formats)
         self.num_requests = d.num_remote_workers if rq is not None else 0
         self.handle = C.c_void_p()
         check(lib().apt_epoch_create(C.byref(d), C.byref(self.handle)))
         self._slot = C.c_int()
-        self._sizes = (C.c_int64 * (H + 2))()
+        self._sizes = (C.c_int64 * (2 * H + 2))()
         self._req = (C.c_int64 * max(self.num_requests, 1))()
 
     def begin(self, seeds, num_batches, rng_seed0, ready_event=None):
@@ -681,10 +700,14 @@ class EpochDriver:
                                     C.c_void_p(ready_event.cuda_event) if ready_event is not None else None))
 
     def next(self):
-        """Blocks until the next batch is complete -> (slot, sizes list, request sizes list or None)."""
+        """Blocks until the next batch is complete -> (slot, sizes list, request sizes list or None, edge counts of
+        the blocks' formats or None)."""
         check(lib().apt_epoch_next(self.handle, C.byref(self._slot), self._sizes,
                                    self._req if self.num_requests else None))
-        return self._slot.value, list(self._sizes), (list(self._req)[:self.num_requests] if self.num_requests else None)
+        H = self.num_hops
+        sizes = list(self._sizes)
+        return (self._slot.value, sizes[:H + 2], (list(self._req)[:self.num_requests] if self.num_requests else None),
+                sizes[H + 2:] if self.formats else None)
 
     def release(self):
         check(lib().apt_epoch_release(self.handle, _stream()))

@@ -7,7 +7,7 @@
 // third for the features.  Here a batch is enqueued by a worker thread of this
 // library -- fused sampling + relabel, the gather (or, for a partitioned feature
 // store, the bucketing of the requests and the gather of the rows present here),
-// the copy of the batch's sizes to pinned host memory and the event that marks
+// the blocks' COO / CSC / CSR where asked for, the copy of the batch's sizes to pinned host memory and the event that marks
 // it complete -- on one of a few "slots" (a set of device buffers and a HIP
 // stream each), so that several batches are in flight and the consumer's thread
 // does nothing per batch but wait for the next one and say when it is done with
@@ -37,16 +37,21 @@ constexpr int kCoResidentStreams = 4;
 constexpr int kCoResidentSampleBlocks = 512;
 constexpr int kCoResidentGatherBlocks = 1024;
 
-constexpr int kPinnedPerSlot = APT_MAX_HOPS + 2 + APT_MAX_BUCKETS;  // int64 words of pinned memory per slot
+// int64 words of pinned memory per slot: the sizes, the request bucket sizes, the blocks' edge counts
+constexpr int kPinnedReq = APT_MAX_HOPS + 2;
+constexpr int kPinnedEdges = kPinnedReq + APT_MAX_BUCKETS;
+constexpr int kPinnedPerSlot = kPinnedEdges + APT_MAX_HOPS;
 
 // The batch's sizes (and request bucket sizes) go to pinned host memory by a one-wavefront kernel rather than a
 // hipMemcpyAsync of 40 bytes: the stores stay on the stream's compute queue, with no hand-over to a copy engine
 // and back between a batch and the next one on the stream.
 __global__ void publish_sizes_kernel(const int64_t* __restrict__ sizes, int n, const int64_t* __restrict__ req,
-                                     int r, int64_t* __restrict__ host_words) {
+                                     int r, const int64_t* __restrict__ edges, int e,
+                                     int64_t* __restrict__ host_words) {
   const int t = threadIdx.x;
   if (t < n) host_words[t] = sizes[t];
-  if (t < r) host_words[APT_MAX_HOPS + 2 + t] = req[t];
+  if (t < r) host_words[kPinnedReq + t] = req[t];
+  if (t < e) host_words[kPinnedEdges + t] = edges[t];
 }
 
 struct EpochWork {
@@ -129,9 +134,21 @@ static int enqueue_batch(apt_epoch* ep, const EpochWork& w) {
       }
     }
   }
+  if (d.formats != 0) {
+    // the blocks in the formats a layer consumes, after the relabel's last pass (which may have ridden in the gather)
+    for (int h = 0; h < H; ++h) {
+      const apt_block_buffers& b = s.blocks[h];
+      rc = apt_block_formats(s.relabeled[h], apt_minibatch_capacity(d.batch, d.hop_fanouts, H, h), s.sizes + h,
+                             d.hop_fanouts[h], apt_minibatch_capacity(d.batch, d.hop_fanouts, H, h + 1), b.coo_row,
+                             b.coo_col, b.csc_indptr, s.block_edges + h, b.csr_indptr, b.csr_indices, b.csr_eids,
+                             b.workspace, b.workspace_bytes, st);
+      if (rc != APT_OK) return rc;
+    }
+  }
   static_assert(APT_MAX_HOPS + 2 <= 64 && APT_MAX_BUCKETS <= 64, "publish_sizes_kernel runs one wavefront");
   hipLaunchKernelGGL(publish_sizes_kernel, dim3(1), dim3(64), 0, st, s.sizes, H + 2,
                      d.has_requests != 0 ? s.request_sizes : nullptr, d.has_requests != 0 ? d.num_remote_workers : 0,
+                     d.formats != 0 ? s.block_edges : nullptr, d.formats != 0 ? H : 0,
                      ep->pinned_dev + static_cast<size_t>(w.slot) * kPinnedPerSlot);
   APT_LAUNCH_CHECK("publish_sizes_kernel");
   APT_HIP(hipEventRecord(ep->done[w.slot], st));
@@ -203,6 +220,23 @@ static int check_desc(const apt_epoch_desc* d) {
       APT_REQUIRE(s.request_sizes != nullptr && s.request_ids != nullptr && s.request_perm != nullptr &&
                       s.request_workspace != nullptr,
                   APT_EINVAL, "apt_epoch_create: slot %d: request buffers missing", k);
+    if (d->formats != 0) {
+      APT_REQUIRE(s.block_edges != nullptr, APT_EINVAL, "apt_epoch_create: slot %d: block_edges is NULL", k);
+      for (int h = 0; h < d->num_hops; ++h) {
+        const apt_block_buffers& b = s.blocks[h];
+        APT_REQUIRE(b.coo_row != nullptr && b.coo_col != nullptr && b.csc_indptr != nullptr && b.workspace != nullptr,
+                    APT_EINVAL, "apt_epoch_create: slot %d: block buffers of hop %d missing", k, h);
+        APT_REQUIRE((b.csr_indptr == nullptr) == (b.csr_indices == nullptr) && (b.csr_indptr == nullptr) == (b.csr_eids == nullptr),
+                    APT_EINVAL, "apt_epoch_create: slot %d: hop %d: all three CSR buffers or none", k, h);
+        const size_t want = apt_block_workspace_bytes(apt_minibatch_capacity(d->batch, d->hop_fanouts, d->num_hops, h),
+                                                      d->hop_fanouts[h],
+                                                      apt_minibatch_capacity(d->batch, d->hop_fanouts, d->num_hops, h + 1),
+                                                      b.csr_indptr != nullptr);
+        APT_REQUIRE(b.workspace_bytes >= want, APT_EWORKSPACE,
+                    "apt_epoch_create: slot %d: hop %d: block workspace of %zu bytes, %zu needed", k, h, b.workspace_bytes,
+                    want);
+      }
+    }
   }
   return APT_OK;
 }
@@ -326,8 +360,10 @@ extern "C" int apt_epoch_next(apt_epoch* ep, int* slot, int64_t* sizes_host, int
   const double gpu_wait = std::chrono::duration<double>(std::chrono::steady_clock::now() - t1).count();
   const int64_t* pin = ep->pinned + static_cast<size_t>(k) * kPinnedPerSlot;
   for (int j = 0; j < ep->d.num_hops + 2; ++j) sizes_host[j] = pin[j];
+  if (ep->d.formats != 0)
+    for (int j = 0; j < ep->d.num_hops; ++j) sizes_host[ep->d.num_hops + 2 + j] = pin[kPinnedEdges + j];
   if (request_sizes_host != nullptr && ep->d.has_requests != 0)
-    for (int j = 0; j < ep->d.num_remote_workers; ++j) request_sizes_host[j] = pin[APT_MAX_HOPS + 2 + j];
+    for (int j = 0; j < ep->d.num_remote_workers; ++j) request_sizes_host[j] = pin[kPinnedReq + j];
   {
     std::lock_guard<std::mutex> lk(ep->mu);
     ep->handed_out = i + 1;

@@ -10,9 +10,9 @@ receives batch i while batches i+1 .. i+in_flight-1 are being built.
 
 The per-batch host work (a dozen kernel launches, the copy of the sizes, the
 events) is done by a thread of the C library (apt_epoch_*, capi.EpochDriver):
-the Python thread only waits for the next batch and narrows its buffers.  With
-block formats or graph replay requested the batches are enqueued from Python
-instead (driver="python" forces that path).
+the Python thread only waits for the next batch and narrows its buffers, block
+formats (COO / CSC / CSR) included.  With graph replay requested the batches are
+enqueued from Python instead (driver="python" forces that path).
 """
 import torch
 
@@ -32,7 +32,7 @@ class MiniBatchLoader:
         replays a captured HIP graph, which costs the host less per batch (worth it
         for small batches, where the host's launch calls are the limit).  as_blocks:
         batch["blocks"] are sampler.Block objects, ready for apt_amd.layers.
-        driver: "c" = batches are enqueued by the C library's epoch thread (not with formats or use_graph),
+        driver: "c" = batches are enqueued by the C library's epoch thread (not with use_graph),
         "python" = from this thread, "auto" = "c" where it applies.
         streams: the torch.cuda.Stream objects to build batches on, one per batch in flight (default: new ones;
         never the consumer's stream).  A process has few hardware queues (HIP's GPU_MAX_HW_QUEUES, 4 by default) and
@@ -67,9 +67,9 @@ class MiniBatchLoader:
         self.epoch = 0
         if driver not in ("auto", "c", "python"):
             raise ValueError("driver must be 'auto', 'c' or 'python'")
-        c_ok = not formats and not use_graph
+        c_ok = not use_graph
         if driver == "c" and not c_ok:
-            raise ValueError("the C epoch driver does not emit block formats or replay graphs: use driver='python'")
+            raise ValueError("the C epoch driver does not replay graphs: use driver='python'")
         from . import capi
         if len(self.pipes) > capi.MAX_SLOTS:
             if driver == "c":
@@ -155,10 +155,10 @@ class MiniBatchLoader:
             drv.begin(full.reshape(-1), self.num_full, rng0, ready)
             try:
                 for i in range(self.num_full):
-                    k, sizes, rs = drv.next()
+                    k, sizes, rs, fe = drv.next()
                     pipe = slots[k]
                     pipe.seeds = batches[i]
-                    out = pipe.result(as_blocks=self.as_blocks, sizes=sizes, request_sizes=rs)
+                    out = pipe.result(as_blocks=self.as_blocks, sizes=sizes, request_sizes=rs, format_edges=fe)
                     out["output_nodes"] = batches[i]
                     yield out
                     drv.release()

@@ -259,12 +259,12 @@ class MiniBatchPipeline:
                 self.format_edges_host = torch.empty(len(self.fanouts), dtype=torch.int64, pin_memory=True)
             self.format_edges_host.copy_(self.format_edges, non_blocking=True)
 
-    def result(self, staged=False, as_blocks=False, sizes=None, request_sizes=None):
+    def result(self, staged=False, as_blocks=False, sizes=None, request_sizes=None, format_edges=None):
         """Waits for the batch and narrows the buffers to their real sizes ->
         dict(input_nodes, blocks (outermost first), features, num_edges).
         staged: the sizes were copied by stage_sizes() and that copy has finished.
-        sizes (and request_sizes): the batch's sizes as host lists, when the caller already has them (the
-        epoch driver reads them from pinned memory); nothing is waited for then.
+        sizes (and request_sizes, format_edges): the batch's sizes as host lists, when the caller already has them
+        (the epoch driver reads them from pinned memory); nothing is waited for then.
         as_blocks: the blocks come as sampler.Block objects (what the layers of
         apt_amd.layers take) instead of dicts; they live in this pipeline's buffers
         like everything else, so a training step must finish with them before the
@@ -275,7 +275,8 @@ class MiniBatchPipeline:
             sizes = self.sizes_host.tolist() if staged else self.sizes.cpu().tolist()
         fmt_edges = None
         if self.formats is not None:
-            fmt_edges = self.format_edges_host.tolist() if staged else self.format_edges.cpu().tolist()
+            fmt_edges = (format_edges if format_edges is not None else
+                         self.format_edges_host.tolist() if staged else self.format_edges.cpu().tolist())
         H = len(self.fanouts)
         blocks = []
         for h, f in enumerate(self.fanouts):

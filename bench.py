@@ -940,7 +940,8 @@ def main():
     fmt = None
     if args.formats:
         fmt = extra.stage_formats(args=args, B=B, graph=wl.graph, hops=hops, K=K, MiniBatchPipeline=MiniBatchPipeline,
-                                  requests=wl.requests, seed_sets=seed_sets, store=wl.store, torch=torch, W=W)
+                                  requests=wl.requests, seed_sets=seed_sets, store=wl.store, torch=torch, W=W,
+                                  time_loader=time_loader)
     shuffle = None
     if args.shuffle:
         shuffle = extra.stage_shuffle(args=args, capi=capi, dev=dev, hops=hops, N=wl.N, seed_sets=seed_sets,

@@ -134,7 +134,7 @@ def stage_aggregation(capi, dev, synth, torch, pipe, seeds, rng_seed, data_seed=
     return agg
 
 
-def stage_formats(args, B, graph, hops, K, MiniBatchPipeline, requests, seed_sets, store, torch, W):
+def stage_formats(args, B, graph, hops, K, MiniBatchPipeline, requests, seed_sets, store, torch, W, time_loader=None):
     """Every hop's block as COO + CSC (+ CSR), device-side sizes, after sampling."""
     ev = lambda: torch.cuda.Event(enable_timing=True)
     fmt = {}
@@ -158,6 +158,16 @@ def stage_formats(args, B, graph, hops, K, MiniBatchPipeline, requests, seed_set
         torch.cuda.synchronize()
         fmt[name + "_whole_batch_ms"] = (time.perf_counter() - t0) / K * 1e3   # sampling + formats beside the gather
         del fp
+        if time_loader is not None and args.inflight > 1:
+            # what a trainer receives: the epoch loader with the formats in every batch, through the library's
+            # epoch thread and through the Python driver
+            from apt_amd.loader import MiniBatchLoader
+            for drv in ("c", "python"):
+                ld = MiniBatchLoader(graph, store, torch.cat(seed_sets), B, hops, in_flight=args.inflight, shuffle=False,
+                                     replace=args.replace, seed=args.seed, requests=requests, formats=what, driver=drv)
+                t_ld, _, _ = time_loader(torch, ld, W)
+                fmt[f"{name}_loader_{drv}_ms"] = t_ld / K * 1e3
+                del ld
     return fmt
 
 

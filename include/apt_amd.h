@@ -485,6 +485,19 @@ int apt_gather_rows_with_lookup(const apt_feat_store* store, const int64_t* inde
  * Nothing here allocates device memory; pinned host memory for the sizes, the
  * events and the thread belong to the handle. */
 #define APT_MAX_SLOTS 16
+/* One hop's block in the formats a GNN layer consumes (apt_block_formats), buffers
+ * sized for the hop's upper bounds; csr_* NULL: COO + CSC only. */
+typedef struct apt_block_buffers {
+  int64_t* coo_row;
+  int64_t* coo_col;
+  int64_t* csc_indptr;
+  int64_t* csr_indptr;
+  int64_t* csr_indices;
+  int64_t* csr_eids;
+  void* workspace;                    /* apt_block_workspace_bytes(capacity(h), fanout, capacity(h + 1), csr) */
+  size_t workspace_bytes;
+} apt_block_buffers;
+
 typedef struct apt_batch_slot {
   void* stream;                       /* hipStream_t of this slot (not the default stream) */
   int64_t* nodes;                     /* as in apt_minibatch_sample, sized by apt_minibatch_capacity */
@@ -504,6 +517,9 @@ typedef struct apt_batch_slot {
   int64_t* request_perm;              /* device int64[capacity(num_hops)] */
   void* request_workspace;            /* apt_bucket_workspace_bytes(capacity(num_hops), num_remote_workers) */
   size_t request_workspace_bytes;
+  /* block formats only (apt_epoch_desc.formats): */
+  apt_block_buffers blocks[APT_MAX_HOPS];
+  int64_t* block_edges;               /* device int64[num_hops]: receives every hop's edge count */
 } apt_batch_slot;
 
 typedef struct apt_epoch_desc {
@@ -521,6 +537,8 @@ typedef struct apt_epoch_desc {
   const int64_t* min_vids;
   int world_size;
   int num_remote_workers;
+  int formats;                        /* != 0: every hop's block is also emitted as COO + CSC (+ CSR where the
+                                         slot's csr_* buffers are not NULL), python/npc/sampler.py:44-69,76-91 */
   int num_slots;
   apt_batch_slot slots[APT_MAX_SLOTS];
 } apt_epoch_desc;
@@ -538,8 +556,10 @@ typedef struct apt_epoch apt_epoch;   /* opaque */
  * apt_epoch_next     blocks until the next batch (they come in order) is
  *                    complete on the GPU; *slot = the slot that holds it,
  *                    sizes_host[num_hops + 2] = its sizes as apt_minibatch_sample
- *                    defines them, request_sizes_host[num_remote_workers]
- *                    (optional) the request buckets.  The slot's buffers are
+ *                    defines them, followed, with formats, by num_hops more
+ *                    entries, the blocks' edge counts (sizes_host then has
+ *                    2 * num_hops + 2 entries); request_sizes_host
+ *                    [num_remote_workers] (optional) the request buckets.  The slot's buffers are
  *                    the caller's to read until apt_epoch_release.
  * apt_epoch_release  the caller is done with the batch apt_epoch_next returned
  *                    last: work it has enqueued on consumer_stream so far is

@@ -77,8 +77,9 @@ def test_loader_c_and_python_drivers_agree(capi):
     a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", **kw)
     b = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="python", **kw)
     assert a._use_c and not b._use_c and MiniBatchLoader(g, store, ids, 200, [4], **kw)._use_c
+    assert MiniBatchLoader(g, store, ids, 200, [4], formats=True, **kw)._use_c
     with pytest.raises(ValueError):
-        MiniBatchLoader(g, store, ids, 200, [4], driver="c", formats=True)
+        MiniBatchLoader(g, store, ids, 200, [4], driver="c", use_graph=True)
     # the caller's own streams (one per batch in flight, never the default stream)
     mine = [torch.cuda.Stream() for _ in range(3)]
     a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", streams=mine, **kw)
@@ -96,6 +97,23 @@ def test_loader_c_and_python_drivers_agree(capi):
             for p, q in zip(x["blocks"], y["blocks"]):
                 for k in ("seeds", "neighbors", "relabeled", "counts", "unique"):
                     assert torch.equal(p[k], q[k]), k
+            n += 1
+        assert n == 11
+    # block formats through either driver: COO + CSC + CSR, and COO + CSC only
+    for formats in (True, "csc"):
+        a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", formats=formats, **kw)
+        b = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="python", formats=formats, **kw)
+        n = 0
+        for x, y in zip(a, b):
+            assert torch.equal(x["input_nodes"], y["input_nodes"]) and torch.equal(x["features"], y["features"])
+            for p, q in zip(x["blocks"], y["blocks"]):
+                assert torch.equal(p["relabeled"], q["relabeled"])
+                fp, fq = p["formats"], q["formats"]
+                assert fp["num_edges"] == fq["num_edges"] == int((p["relabeled"] >= 0).sum())
+                assert sorted(fp) == sorted(fq) and ("csr_indptr" in fp) == (formats is True)
+                for k in fp:
+                    if k != "num_edges":
+                        assert torch.equal(fp[k], fq[k]), (formats, k)
             n += 1
         assert n == 11
 
