@@ -140,13 +140,18 @@ def test_loader_with_partitioned_store(capi):
     rq = dict(feat_pos_map=pos, remote_worker_map=torch.tensor([1, 0, 2, 3], device="cuda"),
               min_vids=torch.tensor([0, 10000, 20000, 25000, 30000], device="cuda"), world_size=P, num_remote_workers=P)
     ids = torch.arange(lo, lo + 1280).cuda()
-    lone = MiniBatchPipeline(g, store, 128, [4, 4], requests=rq)
-    for driver in ("c", "python"):
+    for driver, formats in (("c", False), ("python", False), ("c", True)):
+        lone = MiniBatchPipeline(g, store, 128, [4, 4], requests=rq, formats=formats)
         loader = MiniBatchLoader(g, store, ids, 128, [4, 4], in_flight=3, shuffle=False, seed=2, requests=rq,
-                                 driver=driver)
+                                 driver=driver, formats=formats)
         for i, batch in enumerate(loader):
             lone.run(ids[i * 128:(i + 1) * 128], 2 * 7919 * 10 + i)
             want = lone.result()
+            if formats:
+                for p, q in zip(batch["blocks"], want["blocks"]):
+                    assert sorted(p["formats"]) == sorted(q["formats"]) and "csr_eids" in p["formats"]
+                    for k, v in p["formats"].items():
+                        assert v == q["formats"][k] if k == "num_edges" else torch.equal(v, q["formats"][k]), k
             assert batch["request_sizes"] == want["request_sizes"] and sum(batch["request_sizes"]) == want["sizes"][-1]
             assert batch["request_sizes"][0] > 0 and sum(batch["request_sizes"][1:]) > 0
             assert torch.equal(batch["request_ids"], want["request_ids"])
