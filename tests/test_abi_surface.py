@@ -201,6 +201,27 @@ def test_epoch_driver_argument_checks_need_no_gpu():
     d.num_slots = 17
     assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"num_slots" in L.apt_last_error()
     assert not h.value
+    # a slot whose sampling buffers are there (never dereferenced by the checks) but whose block buffers are not
+    d.num_slots, d.formats = 1, 1
+    fan = (ctypes.c_int * 2)(5, 5)
+    s = d.slots[0]
+    fake = 4096
+    p64 = lambda: fake
+    s.nodes, s.sizes, s.rank_table, s.workspace = fake, fake, fake, fake
+    s.workspace_bytes = L.apt_minibatch_workspace_bytes(64, fan, 2)
+    for k in range(2):
+        s.neighbors[k], s.relabeled[k] = p64(), p64()
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"block_edges" in L.apt_last_error()
+    s.block_edges = p64()
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"block buffers of hop 0" in L.apt_last_error()
+    for k in range(2):
+        b = s.blocks[k]
+        b.coo_row, b.coo_col, b.csc_indptr, b.workspace, b.workspace_bytes = p64(), p64(), p64(), fake, 1 << 30
+    s.blocks[1].csr_indptr = p64()
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"all three CSR" in L.apt_last_error()
+    s.blocks[1].csr_indices, s.blocks[1].csr_eids, s.blocks[1].workspace_bytes = p64(), p64(), 8
+    assert L.apt_epoch_create(ctypes.byref(d), ctypes.byref(h)) != 0 and b"hop 1: block workspace" in L.apt_last_error()
+    assert not h.value
     assert L.apt_epoch_next(None, None, None, None) != 0 and L.apt_epoch_release(None, None) != 0
     assert L.apt_epoch_begin(None, None, 0, 0, None) != 0 and L.apt_epoch_end(None) != 0
     assert L.apt_epoch_destroy(None) == 0
