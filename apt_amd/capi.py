@@ -39,6 +39,9 @@ class CFeatStore(C.Structure):
 MAX_HOPS, MAX_SLOTS = 8, 16
 
 
+ABI_VERSION = 2          # APT_ABI_VERSION of include/apt_amd.h
+
+
 class CBlockBuffers(C.Structure):    # apt_block_buffers
     _fields_ = [("coo_row", C.c_void_p), ("coo_col", C.c_void_p), ("csc_indptr", C.c_void_p),
                 ("csr_indptr", C.c_void_p), ("csr_indices", C.c_void_p), ("csr_eids", C.c_void_p),
@@ -157,6 +160,9 @@ def lib():
             fn = getattr(L, name)
             fn.restype = res
             fn.argtypes = args
+        if L.apt_abi_version() != ABI_VERSION:
+            raise ImportError(f"{LIB_PATH} has ABI version {L.apt_abi_version()}, these bindings are written against "
+                              f"{ABI_VERSION}: rebuild it with `python apt_amd/build.py`")
         _lib = L
     return _lib
 

@@ -50,7 +50,7 @@ int tuning_block_fused_scan() { return g_block_fused_scan; }
 
 extern "C" const char* apt_last_error(void) { return apt::last_error_buf(); }
 
-extern "C" int apt_abi_version(void) { return 1; }
+extern "C" int apt_abi_version(void) { return APT_ABI_VERSION; }
 
 extern "C" int apt_set_tuning(const char* key, int value) {
   if (key == nullptr) return apt::fail(APT_EINVAL, "apt_set_tuning: key is NULL");

@@ -91,6 +91,13 @@ struct State {  // counterpart of NPCState, reference src/state.h:32-63
 };
 
 State& S() {
+  // the C library found at run time must be the one this file's header describes
+  static const bool abi_ok = [] {
+    TORCH_CHECK(apt_abi_version() == APT_ABI_VERSION, "npc: libapt_hip.so has ABI version ", apt_abi_version(),
+                ", libnpc.so was built against ", APT_ABI_VERSION);
+    return true;
+  }();
+  (void)abi_ok;
   static State s;
   return s;
 }

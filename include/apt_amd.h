@@ -55,6 +55,10 @@ typedef struct apt_pending_lookup {
 #define APT_MAX_BUCKETS 64 /* reference: MAX_NUM_DEVICES 33 (src/cuda/npc_kernel.h:13) */
 
 const char* apt_last_error(void);
+/* Raised whenever a struct of this header or a signature changes; a binding
+ * compares apt_abi_version() of the library it loaded with the header it was
+ * written against. */
+#define APT_ABI_VERSION 2
 int apt_abi_version(void);
 
 /* Kernel-variant knobs for measurement (process-wide, not thread-safe, no

@@ -27,7 +27,8 @@ def test_header_symbols_are_exported_and_bound():
             assert hasattr(lib, name), f"{name} declared in include/{hdr} but not exported by {path}"
             assert name in table, f"{name} has no ctypes prototype in capi"
         assert sorted(table) == declared, f"capi binds symbols that include/{hdr} does not declare"
-    assert capi.lib().apt_abi_version() == 1
+    version = int(re.search(r"#define APT_ABI_VERSION (\d+)", open(os.path.join(ROOT, "include", "apt_amd.h")).read()).group(1))
+    assert capi.lib().apt_abi_version() == version == capi.ABI_VERSION
     capi.bench_lib()
 
 
