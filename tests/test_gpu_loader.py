@@ -160,6 +160,55 @@ def test_loader_with_partitioned_store(capi):
         assert i == 9
 
 
+@pytest.mark.parametrize("layout", [[0], [0, 0, 0, 0, 0], [0, 1, 0], [0, 1, 2, 3, 0, 1, 2]])
+def test_epoch_driver_slot_layouts_and_restart(capi, layout):
+    """The library's epoch driver on its own: slots spread unevenly over streams (every slot with a table of its own),
+    a consumer that keeps every batch busy on its stream before releasing it, an epoch begun while the one before
+    is half consumed, and one ended early; every batch equals a lone pipeline's for the same seeds and key."""
+    import torch
+
+    from apt_amd.pipeline import MiniBatchPipeline
+    g, store, table = _setup(capi)
+    B, hops = 96, [4, 3]
+    streams = [torch.cuda.Stream() for _ in range(max(layout) + 1)]
+    pipes = [MiniBatchPipeline(g, store, B, hops) for _ in layout]
+    lone = MiniBatchPipeline(g, store, B, hops)
+    drv = capi.EpochDriver(pipes, [streams[k] for k in layout])
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    sink = torch.zeros(1 << 20, device="cuda")
+
+    def epoch(num, key0, consume):
+        seeds = torch.randint(0, 30000, (num * B,), generator=gen, device="cuda")
+        ready = torch.cuda.Event()
+        ready.record()
+        drv.begin(seeds, num, key0, ready)
+        for i in range(consume):
+            k, sizes, rs, fe = drv.next()
+            assert k == i % len(layout) and rs is None and fe is None
+            pipe = pipes[k]
+            pipe.seeds = seeds[i * B:(i + 1) * B]
+            got = pipe.result(sizes=sizes)
+            for _ in range(3):                           # work on the consumer's stream that reads the slot's buffers
+                sink[:got["features"].numel()] += got["features"].reshape(-1)
+            kept = (got["input_nodes"].clone(), got["features"].clone(), [b["relabeled"].clone() for b in got["blocks"]])
+            drv.release()
+            lone.run(seeds[i * B:(i + 1) * B], key0 + i)
+            want = lone.result()
+            assert sizes[:len(hops) + 1] == want["sizes"] and torch.equal(kept[0], want["input_nodes"])
+            assert torch.equal(kept[1], want["features"]) and torch.equal(kept[1], table[kept[0]])
+            for a, b in zip(kept[2], want["blocks"]):
+                assert torch.equal(a, b["relabeled"])
+
+    epoch(9, 1000, 9)
+    epoch(7, 2000, 3)          # left half consumed: the next begin ends it
+    epoch(2 * len(layout) + 1, 3000, 2 * len(layout) + 1)
+    drv.end()
+    drv.end()                  # ending twice is harmless
+    epoch(1, 4000, 1)
+    drv.close()
+
+
 def test_loader_without_shuffle_and_early_exit(capi):
     import torch
 
