@@ -166,6 +166,7 @@ static void worker_main(apt_epoch* ep) {
   if (streams >= kCoResidentStreams) set_thread_launch_caps(kCoResidentSampleBlocks, kCoResidentGatherBlocks);
   for (;;) {
     EpochWork w;
+    bool failed;  // an earlier batch (or a release) has failed: nothing more is enqueued
     {
       std::unique_lock<std::mutex> lk(ep->mu);
       ep->cv_work.wait(lk, [ep] { return ep->stop || !ep->queue.empty(); });
@@ -173,9 +174,10 @@ static void worker_main(apt_epoch* ep) {
       w = ep->queue.front();
       ep->queue.pop_front();
       ep->busy = true;
+      failed = ep->error != 0;
     }
     const auto t0 = std::chrono::steady_clock::now();
-    const int rc = ep->error == 0 ? enqueue_batch(ep, w) : APT_OK;
+    const int rc = failed ? APT_OK : enqueue_batch(ep, w);
     const double dt = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     {
       std::lock_guard<std::mutex> lk(ep->mu);
