@@ -421,22 +421,42 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(SortParams p)
 }
 
 // csr_indptr[s] = first position of a key >= s in the sorted keys, s in [0, num_src].
+// Position e starts a run of its key k when the key before it, kp, is smaller: then e is the answer for every
+// s in (kp, k].  One lane per position writes those entries itself when they are few (in a sampled block nearly
+// every source has an edge, so the run before a key is one or two entries long); a longer stretch is filled by the
+// whole wavefront.  Sources above the largest key get the edge total.  No searching: every offset is written
+// once, from a coalesced read of the keys.
+constexpr int kIndptrShortGap = 4;
+
 __global__ __launch_bounds__(kFmtBlock) void csr_indptr_kernel(const uint32_t* __restrict__ keys,
                                                                const int64_t* num_edges_dev, int64_t max_edges,
                                                                int64_t num_src, int64_t* __restrict__ csr_indptr) {
   const int64_t n = actual_count(max_edges, num_edges_dev);
   const int64_t last = n > 0 ? static_cast<int64_t>(keys[n - 1]) : -1;
-  for (int64_t s = static_cast<int64_t>(blockIdx.x) * kFmtBlock + threadIdx.x; s <= num_src;
-       s += static_cast<int64_t>(gridDim.x) * kFmtBlock) {
-    int64_t lo = 0, hi = n;
-    if (s > last) lo = n;
-    while (lo < hi) {
-      const int64_t mid = lo + (hi - lo) / 2;
-      if (static_cast<int64_t>(keys[mid]) < s) lo = mid + 1;
-      else hi = mid;
+  const int lane = lane_id();
+  const int64_t tid = static_cast<int64_t>(blockIdx.x) * kFmtBlock + threadIdx.x;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kFmtBlock;
+  for (int64_t e0 = tid - lane; e0 < n; e0 += stride) {   // e0: the wavefront's first position (wave-uniform)
+    const int64_t e = e0 + lane;
+    int64_t k = -1, kp = -1;
+    if (e < n) {
+      k = static_cast<int64_t>(keys[e]);
+      if (e > 0) kp = static_cast<int64_t>(keys[e - 1]);
+      if (k > num_src) k = num_src;    // keys beyond the bound have no offset of their own
+      if (kp > num_src) kp = num_src;
     }
-    csr_indptr[s] = lo;
+    const int64_t gap = k - kp;        // entries (kp, k] hold e
+    if (gap > 0 && gap <= kIndptrShortGap)
+      for (int64_t t = kp + 1; t <= k; ++t) csr_indptr[t] = e;
+    uint64_t wide = ballot(gap > kIndptrShortGap);
+    while (wide != 0) {
+      const int src = __ffsll(static_cast<long long>(wide)) - 1;
+      wide &= wide - 1;
+      const int64_t a = __shfl(kp, src, kWave) + 1, b = __shfl(k, src, kWave);
+      for (int64_t t = a + lane; t <= b; t += kWave) csr_indptr[t] = e0 + src;
+    }
   }
+  for (int64_t t = last + 1 + tid; t <= num_src; t += stride) csr_indptr[t] = n;
 }
 
 // An empty block: offsets all zero.
@@ -583,7 +603,8 @@ extern "C" int apt_block_formats(const int64_t* relabeled, int64_t num_dst, cons
     APT_LAUNCH_CHECK("radix_scatter_kernel");
   }
   const uint32_t* sorted = reinterpret_cast<uint32_t*>(ws + L.key_off[(passes - 1) & 1]);
-  const unsigned iblocks = static_cast<unsigned>(std::min<int64_t>(ceil_div(num_src + 1, kFmtBlock), 16384));
+  const unsigned iblocks =
+      static_cast<unsigned>(std::min<int64_t>(ceil_div(std::max<int64_t>(num_src + 1, L.slots), kFmtBlock), 4096));
   hipLaunchKernelGGL(csr_indptr_kernel, dim3(iblocks), dim3(kFmtBlock), 0, st, sorted, num_edges_dev, L.slots,
                      num_src, csr_indptr);
   APT_LAUNCH_CHECK("csr_indptr_kernel");
