@@ -58,7 +58,8 @@ def test_gpu_block_formats(orc, capi):
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
     host = lambda d: {k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in d.items()}
     rng = np.random.default_rng(1)
-    big = [(70000, 15, 300000), (5000, 64, 2 ** 24 + 5), (300000, 5, 17)]      # 3 / 4 / 1 digit passes
+    big = [(70000, 15, 300000), (5000, 64, 2 ** 24 + 5), (300000, 5, 17),      # 3 / 4 / 1 digit passes
+           (10, 2, 3_000_000), (1, 1, 70_000)]                                # a few edges, sources far apart
     for num_dst, fanout, num_src in CASES + big:
         for hole in (0.0, 0.3, 1.0):
             r = _random_block(rng, num_dst, fanout, num_src, hole)
