@@ -281,10 +281,16 @@ __global__ __launch_bounds__(kSortBlock) void radix_hist_kernel(SortParams p) {
   __syncthreads();
   const int64_t n = actual_count(p.max_edges, p.num_edges_dev);
   const int64_t base = static_cast<int64_t>(blockIdx.x) * kSortTile;
+  // all of a thread's keys are requested before the first is counted
+  uint32_t key[kSortTile / kSortBlock];
+#pragma unroll
   for (int k = 0; k < kSortTile / kSortBlock; ++k) {
     const int64_t i = base + k * kSortBlock + tid;
-    if (i < n) atomicAdd(&s_hist[(sort_key<FIRST>(p, i) >> p.shift) & (kRadix - 1)], 1u);
+    key[k] = i < n ? sort_key<FIRST>(p, i) : 0u;
   }
+#pragma unroll
+  for (int k = 0; k < kSortTile / kSortBlock; ++k)
+    if (base + k * kSortBlock + tid < n) atomicAdd(&s_hist[(key[k] >> p.shift) & (kRadix - 1)], 1u);
   __syncthreads();
   const int64_t at = p.fused ? static_cast<int64_t>(blockIdx.x) * kRadix + tid
                              : static_cast<int64_t>(tid) * p.tiles + blockIdx.x;
@@ -333,14 +339,14 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(SortParams p)
   const int64_t wave_base = tile_base + static_cast<int64_t>(wave) * kSortWaveItems;
   uint32_t key[kSortRounds], pay[kSortRounds];
 #pragma unroll
-  for (int r = 0; r < kSortRounds; ++r) {
+  for (int r = 0; r < kSortRounds; ++r) {   // every load of the lane is requested before the first is used
     const int64_t i = wave_base + r * kWave + lane;
-    if (i < n) {
-      key[r] = sort_key<FIRST>(p, i);
-      pay[r] = FIRST ? static_cast<uint32_t>(i) : p.pay_in[i];
-      atomicAdd(&s_pos[wave][(key[r] >> p.shift) & (kRadix - 1)], 1u);
-    }
+    key[r] = i < n ? sort_key<FIRST>(p, i) : 0u;
+    pay[r] = FIRST ? static_cast<uint32_t>(i) : (i < n ? p.pay_in[i] : 0u);
   }
+#pragma unroll
+  for (int r = 0; r < kSortRounds; ++r)
+    if (wave_base + r * kWave + lane < n) atomicAdd(&s_pos[wave][(key[r] >> p.shift) & (kRadix - 1)], 1u);
   // First output position of this tile's items of digit `tid`: items with a
   // smaller digit anywhere, plus items with the same digit in earlier tiles.
   uint32_t first;
@@ -406,13 +412,25 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(SortParams p)
   }
   __syncthreads();
   const int count = static_cast<int>(min(static_cast<int64_t>(kSortTile), n - tile_base));
-  for (int j = tid; j < count; j += kSortBlock) {
+  // (in the last pass an item's destination is a dependent read: all of a thread's are requested before any store)
+  int64_t col[LAST ? kSortRounds : 1];
+  if (LAST) {
+#pragma unroll
+    for (int q = 0; q < kSortRounds; ++q) {
+      const int j = q * kSortBlock + tid;
+      col[q] = j < count ? p.coo_col[s_pay[j]] : 0;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < kSortRounds; ++q) {
+    const int j = q * kSortBlock + tid;
+    if (j >= count) break;
     const uint32_t k = s_key[j];
     const uint32_t v = s_pay[j];
     const uint32_t pos = s_delta[(k >> p.shift) & (kRadix - 1)] + j;
     if (LAST) {
       p.csr_eids[pos] = v;
-      p.csr_indices[pos] = p.coo_col[v];
+      p.csr_indices[pos] = col[q];
     } else {
       p.pay_out[pos] = v;
     }
