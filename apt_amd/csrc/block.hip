@@ -193,9 +193,12 @@ __global__ __launch_bounds__(kFmtBlock) void fmt_place_kernel(CompactParams p) {
   int64_t v[kCompactIters];
   uint32_t below[kCompactIters];
 #pragma unroll
-  for (int it = 0; it < kCompactIters; ++it) {
+  for (int it = 0; it < kCompactIters; ++it) {   // the tile's slots are all requested before the first is looked at
     const int64_t s = base + it * kFmtBlock + threadIdx.x;
     v[it] = s < slots ? p.relabeled[s] : -1;
+  }
+#pragma unroll
+  for (int it = 0; it < kCompactIters; ++it) {
     const uint64_t m = ballot(v[it] >= 0);
     below[it] = rank_below(m);
     if (lane == 0) s_cnt[it * kFmtWaves + wave] = __popcll(m);
@@ -223,13 +226,16 @@ __global__ __launch_bounds__(kFmtBlock) void fmt_place_kernel(CompactParams p) {
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    uint32_t acc = first;
-    for (int k = 0; k < kCompactIters * kFmtWaves; ++k) {
-      const uint32_t c = s_cnt[k];
-      s_cnt[k] = acc;
-      acc += c;
+  static_assert(kCompactIters * kFmtWaves <= kWave, "one wavefront scans the tile's per-wave counts");
+  if (wave == 0) {   // exclusive prefix of the (iteration, wave) counts, in the order the edges are numbered
+    const uint32_t c = lane < kCompactIters * kFmtWaves ? s_cnt[lane] : 0u;
+    uint32_t incl = c;
+#pragma unroll
+    for (int off = 1; off < kCompactIters * kFmtWaves; off <<= 1) {
+      const uint32_t y = __shfl_up(incl, off, kWave);
+      if (lane >= off) incl += y;
     }
+    if (lane < kCompactIters * kFmtWaves) s_cnt[lane] = first + incl - c;
   }
   __syncthreads();
 #pragma unroll
@@ -237,10 +243,12 @@ __global__ __launch_bounds__(kFmtBlock) void fmt_place_kernel(CompactParams p) {
     const int64_t s = base + it * kFmtBlock + threadIdx.x;
     if (s >= upper) continue;
     const int64_t e = static_cast<int64_t>(s_cnt[it * kFmtWaves + wave]) + below[it];
-    const int64_t d = s / p.fanout;
+    // (slot numbers fit 32 bits, fmt_sizes_ok: a 32-bit division, a fraction of the cost of a 64-bit one)
+    const uint32_t fan = static_cast<uint32_t>(p.fanout);
+    const uint32_t d = static_cast<uint32_t>(s) / fan;
     // Valid slots before the first slot of a destination = its CSC offset;
     // destinations past the device-side count get the edge total (empty rows).
-    if (s - d * p.fanout == 0) p.csc_indptr[d] = e;
+    if (static_cast<uint32_t>(s) - d * fan == 0) p.csc_indptr[d] = e;
     if (v[it] >= 0) {
       p.coo_row[e] = v[it];
       p.coo_col[e] = d;
