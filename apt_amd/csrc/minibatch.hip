@@ -212,12 +212,26 @@ __global__ __launch_bounds__(kMbBlock) void mb_count_kernel(HopParams p) {
   const int wave = threadIdx.x / kWave;
   uint32_t c = 0;
   if (FIRST) {
+    // First hop: an item (seed or neighbour, its index is its bid) owns its node iff the table still holds its
+    // bid.  The tile's ids, then its table entries, are requested together: two round trips for the tile, not
+    // two per iteration.
     const HopSizes s = hop_sizes(p);
     const int64_t items = s.ns + s.nn;
     if (base >= items) return;
+    const uint32_t tb = table_base(p.state);
+    int64_t v[kMbIters];
+    uint32_t held[kMbIters];
 #pragma unroll
     for (int it = 0; it < kMbIters; ++it) {
-      const uint64_t m = ballot(mb_is_owner<FIRST>(p, s, base + it * kMbBlock + threadIdx.x, items));
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      v[it] = i < items ? (i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns]) : -1;
+    }
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it) held[it] = in_table(p, v[it]) ? p.table[v[it]] : 0u;
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it) {
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      const uint64_t m = ballot(in_table(p, v[it]) && held[it] == tb + static_cast<uint32_t>(i));
       if (lane_id() == 0) p.flags[(static_cast<int64_t>(blockIdx.x) * kMbIters + it) * kMbWaves + wave] = m;
       c += __popcll(m);
     }
@@ -298,6 +312,13 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
   if (ahead_ok) load_tile(slot_capacity(p));
   const HopSizes s = hop_sizes(p);
   const int64_t items = FIRST ? s.ns + s.nn : s.nn;
+  if (FIRST) {   // the first hop's items: seeds, then neighbours (the row count is the host's, nothing to wait for)
+#pragma unroll
+    for (int it = 0; it < kMbIters; ++it) {
+      const int64_t i = base + it * kMbBlock + threadIdx.x;
+      ahead[it] = i < items ? (i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns]) : -1;
+    }
+  }
   const int64_t first_id = FIRST ? 0 : s.ns;
   if (items == 0) {
     if (blockIdx.x == 0 && threadIdx.x == 0) *p.n_next = first_id;
@@ -329,12 +350,10 @@ __global__ __launch_bounds__(kMbBlock) void mb_place_kernel(HopParams p) {
     if ((mine >> lane) & 1) {
       const int64_t i = base + it * kMbBlock + threadIdx.x;
       const int64_t id = before + rank_below(mine);
-      int64_t v;
+      const int64_t v = ahead[it];
       if (FIRST) {
-        v = i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns];
         if (i >= s.ns) p.relabeled[i - s.ns] = id;
       } else {
-        v = ahead[it];
         p.relabeled[i] = id;
       }
       if (id < p.nodes_cap) {
