@@ -172,29 +172,6 @@ __global__ __launch_bounds__(kMbBlock) void mb_mark_neighbors_kernel(HopParams p
   }
 }
 
-// Item i of a hop: FIRST -> seeds followed by neighbours (index = bid);
-// later hops -> neighbours only (bid = ns + index).
-template <bool FIRST>
-__device__ __forceinline__ bool mb_is_owner(const HopParams& p, const HopSizes& s, int64_t i,
-                                            int64_t items) {
-  if (i >= items) return false;
-  int64_t v;
-  uint32_t bid;
-  if (FIRST) {
-    v = i < s.ns ? p.seeds[i] : p.neighbors[i - s.ns];
-    bid = static_cast<uint32_t>(i);
-    if (!in_table(p, v)) return false;
-  } else {
-    // Later hops: the bidding itself settled ownership (rank_table.hpp); the
-    // flag is consumed so that the buffer is clean for the next hop.
-    if (p.relabeled[i] != kSlotOwner) return false;
-    if (p.displaced[i] == 0) return true;
-    p.displaced[i] = 0;
-    return false;
-  }
-  return p.table[v] == table_base(p.state) + bid;
-}
-
 // Upper bound of a hop's neighbour slots as the host knows it: what the buffers hold whatever the device-side
 // row count says.  Loads of per-slot arrays below this bound are safe before that count has arrived, which
 // takes a memory round trip or two out of the start of the small kernels of a batch (they are chains of three
