@@ -36,17 +36,17 @@ MEASURED_GATHER_TRAFFIC_PER_ROW = {
     ("target", "symmetric", "bf16", 128, 1024): (519.5, "profiles/gather_kernel_target_bf16_pmc.txt"),
     ("target", "symmetric", "fp32", 128, 1024): (1030.7, "profiles/gather_kernel_target_fp32_pmc.txt"),
     ("medium", "symmetric", "fp32", 100, 1024): (916.6, "profiles/gather_kernel_medium_pmc.txt"),
-    ("partition", "symmetric", "fp32", 128, 1024): (1197.6, "profiles/gather_kernel_partition_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (1197.7, "profiles/gather_kernel_partition_pmc.txt"),
     ("small", "directed", "fp32", 128, 1024): (1054.7, "profiles/gather_kernel_small_pmc.txt"),
 }
 # The same for the last hop's sampling kernel (rank-table bids included): HBM bytes per sampled edge.
 MEASURED_SAMPLE_TRAFFIC_PER_EDGE = {
     ("full", "symmetric", "bf16", 128, 4096): (257.7, "profiles/gather_kernel_full_pmc.txt"),
-    ("target", "symmetric", "bf16", 128, 1024): (259.9, "profiles/gather_kernel_target_bf16_pmc.txt"),
-    ("target", "symmetric", "fp32", 128, 1024): (259.6, "profiles/gather_kernel_target_fp32_pmc.txt"),
-    ("medium", "symmetric", "fp32", 100, 1024): (219.4, "profiles/gather_kernel_medium_pmc.txt"),
-    ("partition", "symmetric", "fp32", 128, 1024): (417.0, "profiles/gather_kernel_partition_pmc.txt"),
-    ("small", "directed", "fp32", 128, 1024): (204.1, "profiles/gather_kernel_small_pmc.txt"),
+    ("target", "symmetric", "bf16", 128, 1024): (259.8, "profiles/gather_kernel_target_bf16_pmc.txt"),
+    ("target", "symmetric", "fp32", 128, 1024): (259.7, "profiles/gather_kernel_target_fp32_pmc.txt"),
+    ("medium", "symmetric", "fp32", 100, 1024): (220.1, "profiles/gather_kernel_medium_pmc.txt"),
+    ("partition", "symmetric", "fp32", 128, 1024): (417.5, "profiles/gather_kernel_partition_pmc.txt"),
+    ("small", "directed", "fp32", 128, 1024): (201.9, "profiles/gather_kernel_small_pmc.txt"),
 }
 
 WORKLOADS = {
