@@ -64,7 +64,27 @@ def build(force=True, verbose=False):
     for lib, parts in ((LIB, objs), (BENCH_LIB, bench_objs)):
         subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", lib, *parts])
     build_torch_binding(verbose=verbose)
+    build_c_consumer(verbose=verbose)
     return LIB
+
+
+C_CONSUMER_SRC = os.path.join(HERE, "..", "tests", "c_abi", "epoch_consumer.c")
+C_CONSUMER = os.path.join(HERE, "..", "tests", "c_abi", "epoch_consumer")
+
+
+def build_c_consumer(verbose=False):
+    """Compile the plain-C program that drives the library through include/apt_amd.h alone (gcc, C11; the GPU
+    tests run it).  Skipped when the source is not there (an installed copy of the package without the tests)."""
+    if not os.path.exists(C_CONSUMER_SRC):
+        return None
+    cmd = [os.environ.get("CC", "gcc"), "-std=c11", "-O1", "-Wall", "-Wextra", "-Werror",
+           f"-I{os.path.join(HERE, '..', 'include')}", "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__",
+           C_CONSUMER_SRC, f"-L{HERE}", "-lapt_hip", "-L/opt/rocm/lib", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../apt_amd", "-Wl,-rpath,/opt/rocm/lib", "-o", C_CONSUMER]
+    if verbose:
+        print(" ".join(cmd), file=sys.stderr)
+    subprocess.check_call(cmd)
+    return C_CONSUMER
 
 
 def build_torch_binding(verbose=False):
