@@ -7,7 +7,8 @@
  * apt_epoch_create, takes the batches of two epochs in order and checks each one
  * on the host (seeds first among the input nodes, every relabeled entry names the
  * sampled neighbour, every feature row is the row of its node, edge count = the
- * valid slots).  It prints one line a test can compare with what the Python
+ * valid slots, and the last hop's block in COO, CSC and CSR says the same as its
+ * fixed-stride form).  It prints one line a test can compare with what the Python
  * pipeline gets for the same seeds and keys:
  *     ok batches=<n> edges=<sampled edges> nodes=<input nodes> checksum=<sum of all input node ids>
  *
@@ -138,7 +139,23 @@ int main(void) {
     s->features = dev_alloc(sizeof(float) * cap[HOPS] * DIM);
     s->miss_count = dev_alloc(sizeof(int64_t));
     HIP(hipMemset(s->miss_count, 0, sizeof(int64_t)));
+    /* every hop's block also in COO + CSC + CSR */
+    s->block_edges = dev_alloc(sizeof(int64_t) * HOPS);
+    for (int h = 0; h < HOPS; ++h) {
+      apt_block_buffers* b = &s->blocks[h];
+      const int64_t slots = cap[h] * fanouts[h];
+      b->coo_row = dev_alloc(sizeof(int64_t) * slots);
+      b->coo_col = dev_alloc(sizeof(int64_t) * slots);
+      b->csc_indptr = dev_alloc(sizeof(int64_t) * (cap[h] + 1));
+      b->csr_indptr = dev_alloc(sizeof(int64_t) * (cap[h + 1] + 1));
+      b->csr_indices = dev_alloc(sizeof(int64_t) * slots);
+      b->csr_eids = dev_alloc(sizeof(int64_t) * slots);
+      b->workspace_bytes = apt_block_workspace_bytes(cap[h], fanouts[h], cap[h + 1], 1);
+      REQUIRE(b->workspace_bytes > 0, "block sizes out of range");
+      b->workspace = dev_alloc(b->workspace_bytes);
+    }
   }
+  d.formats = 1;
   HIP(hipDeviceSynchronize());
 
   apt_epoch* ep = NULL;
@@ -150,6 +167,13 @@ int main(void) {
   int64_t* h_nbr = malloc(sizeof(int64_t) * cap[HOPS - 1] * fanouts[HOPS - 1]);
   int64_t* h_rel = malloc(sizeof(int64_t) * cap[HOPS - 1] * fanouts[HOPS - 1]);
   float* h_feat = malloc(sizeof(float) * cap[HOPS] * DIM);
+  const int64_t last_slots = cap[HOPS - 1] * fanouts[HOPS - 1];
+  int64_t* h_row = malloc(sizeof(int64_t) * last_slots);
+  int64_t* h_col = malloc(sizeof(int64_t) * last_slots);
+  int64_t* h_csc = malloc(sizeof(int64_t) * (cap[HOPS - 1] + 1));
+  int64_t* h_csr = malloc(sizeof(int64_t) * (cap[HOPS] + 1));
+  int64_t* h_csr_idx = malloc(sizeof(int64_t) * last_slots);
+  int64_t* h_csr_eid = malloc(sizeof(int64_t) * last_slots);
   long long total_edges = 0, total_nodes = 0, checksum = 0;
   int batches_seen = 0;
   for (int epoch = 0; epoch < 2; ++epoch) {
@@ -170,6 +194,15 @@ int main(void) {
       HIP(hipMemcpyAsync(h_feat, s->features, sizeof(float) * n_in * DIM, hipMemcpyDeviceToHost, consumer));
       HIP(hipMemcpyAsync(h_nbr, s->neighbors[HOPS - 1], sizeof(int64_t) * n_mid * fanouts[HOPS - 1], hipMemcpyDeviceToHost, consumer));
       HIP(hipMemcpyAsync(h_rel, s->relabeled[HOPS - 1], sizeof(int64_t) * n_mid * fanouts[HOPS - 1], hipMemcpyDeviceToHost, consumer));
+      const apt_block_buffers* b = &s->blocks[HOPS - 1];
+      const int64_t block_edges = sizes[HOPS + 2 + HOPS - 1];   /* the blocks' edge counts follow the sizes */
+      REQUIRE(block_edges >= 0 && block_edges <= n_mid * fanouts[HOPS - 1], "edge count %lld", (long long)block_edges);
+      HIP(hipMemcpyAsync(h_row, b->coo_row, sizeof(int64_t) * block_edges, hipMemcpyDeviceToHost, consumer));
+      HIP(hipMemcpyAsync(h_col, b->coo_col, sizeof(int64_t) * block_edges, hipMemcpyDeviceToHost, consumer));
+      HIP(hipMemcpyAsync(h_csc, b->csc_indptr, sizeof(int64_t) * (n_mid + 1), hipMemcpyDeviceToHost, consumer));
+      HIP(hipMemcpyAsync(h_csr, b->csr_indptr, sizeof(int64_t) * (n_in + 1), hipMemcpyDeviceToHost, consumer));
+      HIP(hipMemcpyAsync(h_csr_idx, b->csr_indices, sizeof(int64_t) * block_edges, hipMemcpyDeviceToHost, consumer));
+      HIP(hipMemcpyAsync(h_csr_eid, b->csr_eids, sizeof(int64_t) * block_edges, hipMemcpyDeviceToHost, consumer));
       APT(apt_epoch_release(ep, consumer));
       HIP(hipStreamSynchronize(consumer));
       for (int64_t k = 0; k < BATCH; ++k)
@@ -190,6 +223,26 @@ int main(void) {
         REQUIRE(found, "node %lld has no neighbour %lld", (long long)v, (long long)h_nbr[j]);
       }
       REQUIRE(valid <= sizes[HOPS + 1], "edge total %lld below the last hop's %lld", (long long)sizes[HOPS + 1], valid);
+      /* COO = the valid slots in order; CSC offsets count them per destination */
+      REQUIRE(valid == block_edges, "the block has %lld edges, its COO %lld", valid, (long long)block_edges);
+      int64_t e = 0;
+      for (int64_t j = 0; j < n_mid * fanouts[HOPS - 1]; ++j) {
+        if (j % fanouts[HOPS - 1] == 0) REQUIRE(h_csc[j / fanouts[HOPS - 1]] == e, "csc_indptr[%lld]", (long long)(j / fanouts[HOPS - 1]));
+        if (h_nbr[j] < 0) continue;
+        REQUIRE(h_row[e] == h_rel[j] && h_col[e] == j / fanouts[HOPS - 1], "COO edge %lld", (long long)e);
+        ++e;
+      }
+      REQUIRE(h_csc[n_mid] == block_edges, "csc_indptr ends at %lld", (long long)h_csc[n_mid]);
+      /* CSR: the same edges grouped by source, a source's edges by increasing edge id */
+      REQUIRE(h_csr[0] == 0 && h_csr[n_in] == block_edges, "csr_indptr spans %lld..%lld", (long long)h_csr[0], (long long)h_csr[n_in]);
+      for (int64_t src = 0; src < n_in; ++src) {
+        REQUIRE(h_csr[src] <= h_csr[src + 1], "csr_indptr decreases at %lld", (long long)src);
+        for (int64_t q = h_csr[src]; q < h_csr[src + 1]; ++q) {
+          const int64_t id = h_csr_eid[q];
+          REQUIRE(id >= 0 && id < block_edges && h_row[id] == src && h_col[id] == h_csr_idx[q], "CSR entry %lld", (long long)q);
+          REQUIRE(q == h_csr[src] || h_csr_eid[q - 1] < id, "CSR entry %lld out of order", (long long)q);
+        }
+      }
       for (int64_t k = 0; k < n_in; ++k) {
         checksum += h_nodes[k];
         for (int c = 0; c < DIM; ++c)
