@@ -32,6 +32,8 @@ class MiniBatchLoader:
         replays a captured HIP graph, which costs the host less per batch (worth it
         for small batches, where the host's launch calls are the limit).  as_blocks:
         batch["blocks"] are sampler.Block objects, ready for apt_amd.layers.
+        formats: as MiniBatchPipeline's (True / "inner" / "csc": the blocks also in COO + CSC, with CSR for all /
+        all but the outermost / none).
         driver: "c" = batches are enqueued by the C library's epoch thread (not with use_graph),
         "python" = from this thread, "auto" = "c" where it applies.
         streams: the torch.cuda.Stream objects to build batches on, one per batch in flight (default: new ones;

@@ -47,9 +47,11 @@ class MiniBatchPipeline:
         table: the rank table of another pipeline (fused driver) whose batches run on the same stream as this
         one's: batches that follow each other on one stream can share a table (444 MB at 111 M nodes).
 
-        formats: True or "csc" also emits every hop's block as COO + CSC (+ CSR
-        with True), what DGL derives from (row, col) in the reference
-        (python/npc/sampler.py:59-69); result() then carries them per block."""
+        formats: True, "inner" or "csc" also emits every hop's block as COO + CSC, what DGL derives from
+        (row, col) in the reference (python/npc/sampler.py:59-69); result() then carries them per block.
+        True adds CSR for every block, "inner" for all but the outermost one (the largest; its CSR serves the
+        gradient with respect to the layer's input, which a first layer that aggregates the raw features never
+        asks for), "csc" for none."""
         self.graph, self.feat = graph, feat
         self.fanouts = [int(f) for f in hop_fanouts]
         self.replace = bool(replace)
@@ -97,8 +99,11 @@ class MiniBatchPipeline:
             self.request_ws = torch.empty(need, dtype=torch.uint8, device=dev)
         self.formats = None
         if formats:
+            if formats is not True and formats not in ("csc", "inner"):
+                raise ValueError("formats must be False, True, 'inner' or 'csc'")
             self.format_edges = torch.zeros(H, **i64)             # edge count of every hop's block, read in one go
-            self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=formats != "csc", device=dev,
+            with_csr = lambda h: formats is True or (formats == "inner" and h < H - 1)   # hop H - 1 = the outermost block
+            self.formats = [capi.BlockFormats(self.caps[h], f, self.caps[h + 1], want_csr=with_csr(h), device=dev,
                                               num_edges=self.format_edges[h:h + 1])
                             for h, f in enumerate(self.fanouts)]
             # with CSR a hop's formats are a string of ~10 small dependent launches: the hops then run beside

@@ -135,10 +135,11 @@ def stage_aggregation(capi, dev, synth, torch, pipe, seeds, rng_seed, data_seed=
 
 
 def stage_formats(args, B, graph, hops, K, MiniBatchPipeline, requests, seed_sets, store, torch, W, time_loader=None):
-    """Every hop's block as COO + CSC (+ CSR), device-side sizes, after sampling."""
+    """Every hop's block as COO + CSC (+ CSR of all blocks, or of all but the outermost), device-side sizes, after
+    sampling."""
     ev = lambda: torch.cuda.Event(enable_timing=True)
     fmt = {}
-    for name, what in (("coo_csc", "csc"), ("coo_csc_csr", True)):
+    for name, what in (("coo_csc", "csc"), ("coo_csc_csr_inner", "inner"), ("coo_csc_csr", True)):
         fp = MiniBatchPipeline(graph, store, B, hops, replace=args.replace, formats=what, requests=requests)
         t = 0.0
         for i in range(W + K):

@@ -100,7 +100,7 @@ def test_loader_c_and_python_drivers_agree(capi):
             n += 1
         assert n == 11
     # block formats through either driver: COO + CSC + CSR, and COO + CSC only
-    for formats in (True, "csc"):
+    for formats in (True, "csc", "inner"):
         a = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="c", formats=formats, **kw)
         b = MiniBatchLoader(g, store, ids, 200, [4, 3, 2], driver="python", formats=formats, **kw)
         n = 0
@@ -110,7 +110,9 @@ def test_loader_c_and_python_drivers_agree(capi):
                 assert torch.equal(p["relabeled"], q["relabeled"])
                 fp, fq = p["formats"], q["formats"]
                 assert fp["num_edges"] == fq["num_edges"] == int((p["relabeled"] >= 0).sum())
-                assert sorted(fp) == sorted(fq) and ("csr_indptr" in fp) == (formats is True)
+                outermost = p is x["blocks"][0]
+                assert sorted(fp) == sorted(fq)
+                assert ("csr_indptr" in fp) == (formats is True or (formats == "inner" and not outermost))
                 for k in fp:
                     if k != "num_edges":
                         assert torch.equal(fp[k], fq[k]), (formats, k)
@@ -227,7 +229,7 @@ def test_loader_without_shuffle_and_early_exit(capi):
         MiniBatchLoader(g, store, ids[:10], 128, [5])
 
 
-@pytest.mark.parametrize("formats", [False, True])
+@pytest.mark.parametrize("formats", [False, True, "inner"])
 def test_training_loop_on_the_loader(capi, formats):
     """The loader's batches as Block objects feed apt_amd.layers directly: two SAGE
     layers trained on them learn a label that needs the neighbourhood; with formats=True
@@ -258,7 +260,10 @@ def test_training_loop_on_the_loader(capi, formats):
             blocks = batch["blocks"]
             assert all(isinstance(b, Block) for b in blocks) and blocks[-1].num_dst == 256
             if formats:
-                assert blocks[0].formats is not None and "csr_indptr" in blocks[0].formats
+                # "inner": CSR for every block but the outermost, whose backward pass (towards the raw features)
+                # nobody asks for
+                assert blocks[0].formats is not None and ("csr_indptr" in blocks[0].formats) == (formats is True)
+                assert "csr_indptr" in blocks[1].formats
             h = l2(blocks[1], l1(blocks[0], batch["features"]))
             loss = torch.nn.functional.cross_entropy(h, labels[batch["output_nodes"]])
             opt.zero_grad()
