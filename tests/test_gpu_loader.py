@@ -211,6 +211,36 @@ def test_epoch_driver_slot_layouts_and_restart(capi, layout):
     drv.close()
 
 
+def test_loader_with_frequent_table_refills(capi):
+    """The rank table runs out of epochs every other batch (or every batch) when its id field is made as wide as it
+    gets: the epoch driver's batches, two buffer sets sharing a stream's table, stay what a lone pipeline with the
+    default width builds."""
+    import torch
+
+    from apt_amd.loader import MiniBatchLoader
+    from apt_amd.pipeline import MiniBatchPipeline
+    g, store, table = _setup(capi)
+    ids = torch.arange(0, 200 * 24).cuda() % 30000
+    lone = MiniBatchPipeline(g, store, 200, [4, 3])
+    want = []
+    for i in range(24):
+        lone.run(ids[i * 200:(i + 1) * 200], 5 * 7919 * 24 + i)          # the loader's key for seed 5, first epoch
+        r = lone.result()
+        want.append((r["input_nodes"].clone(), r["features"].clone(), [b["relabeled"].clone() for b in r["blocks"]]))
+    try:
+        for bits in (30, 31):
+            capi.check(capi.lib().apt_set_tuning(b"minibatch_payload_bits", bits))
+            for in_flight in (1, 4):
+                loader = MiniBatchLoader(g, store, ids, 200, [4, 3], in_flight=in_flight, shuffle=False, seed=5, driver="c")
+                for i, b in enumerate(loader):
+                    assert torch.equal(b["input_nodes"], want[i][0]) and torch.equal(b["features"], want[i][1]), (bits, i)
+                    for x, y in zip(b["blocks"], want[i][2]):
+                        assert torch.equal(x["relabeled"], y), (bits, in_flight, i)
+                assert i == 23
+    finally:
+        capi.check(capi.lib().apt_set_tuning(b"minibatch_payload_bits", 0))
+
+
 def test_loader_without_shuffle_and_early_exit(capi):
     import torch
 
