@@ -64,8 +64,11 @@ __device__ __forceinline__ RankEpoch rank_epoch(const uint32_t* state) {
 //   never flagged.)
 // first_hop: the table holds seed indices, not ids, so hits cannot be resolved
 // yet and ownership is decided by re-reading the table; no flags are kept.
+// probe: read the entry before bidding (a plain read is cheaper than an atomic, and a third of a large hop's
+// slots need no atomic after it).  A launch too small to be bound by the number of its atomics skips the read:
+// there it is one more dependent round trip in a chain of them, and the returning atomic tells the same.
 __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const RankEpoch& ep, bool first_hop,
-                                                  int64_t v, int64_t ns, int64_t j) {
+                                                  int64_t v, int64_t ns, int64_t j, bool probe = true) {
   const uint32_t tb = ep.base;
   if (v < 0) return v < kSlotStatesEnd ? -1 : v;  // padding; never one of the states above
   if (v >= t.len) return -1;  // an id the table cannot hold: treated as padding
@@ -73,7 +76,7 @@ __device__ __forceinline__ int64_t rank_table_bid(const RankTable& t, const Rank
   const uint32_t bid = first_bid + static_cast<uint32_t>(j);
   // A stale read can only show a larger value than the table holds now, which
   // at worst causes a redundant atomic.
-  const uint32_t cur = t.entries[v];
+  const uint32_t cur = probe ? t.entries[v] : 0xFFFFFFFFu;
   if (first_hop) {
     if (cur > bid) atomicMin(&t.entries[v], bid);
     return kSlotOwner;

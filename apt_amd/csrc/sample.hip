@@ -147,6 +147,7 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
   if (static_cast<int64_t>(blockIdx.x) * tile >= n) return;  // block-uniform
 
   const int fanout = p.fanout;
+  const bool probe = gridDim.x > 512;   // small launches bid without reading the entry first (rank_table_bid)
   int64_t my_total = 0;
   if (tid == 0) s_total = 0;
   // Stage 1 of a tile puts its rows into LDS, one lane per row, so the dependent
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(kSampleBlock) void sample_kernel(SampleParams p) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
           rel[u] = (gis[u] < n && l < fanout)
-                       ? rank_table_bid(p.table, ep, p.first_hop != 0, val[u], n, gis[u] * fanout + l)
+                       ? rank_table_bid(p.table, ep, p.first_hop != 0, val[u], n, gis[u] * fanout + l, probe)
                        : -1;
 #pragma unroll
         for (int u = 0; u < U; ++u)
